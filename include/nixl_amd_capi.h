@@ -1,0 +1,193 @@
+/*
+ * C ABI over the agent (libnixl_amd_agent.so), for callers that cannot include C++:
+ * ctypes tests, benchmarks, other-language bindings.  Function names, argument order and
+ * status values are those of the reference's C wrapper for its Rust bindings
+ * (src/bindings/rust/wrapper.h:28-47,90-116,119-128,178-180,187-197,204-207,221-251,
+ * 266-269,279-291,294-326), restricted to the single-agent transfer path.  Functions
+ * marked "extension" have no counterpart there.
+ */
+#ifndef NIXL_AMD_CAPI_H
+#define NIXL_AMD_CAPI_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    NIXL_CAPI_SUCCESS = 0,
+    NIXL_CAPI_ERROR_INVALID_PARAM = -1,
+    NIXL_CAPI_ERROR_BACKEND = -2,
+    NIXL_CAPI_ERROR_INVALID_STATE = -3,
+    NIXL_CAPI_ERROR_EXCEPTION = -4,
+    NIXL_CAPI_IN_PROG = 1,
+    NIXL_CAPI_ERROR_NO_TELEMETRY = -5,
+    NIXL_CAPI_ERROR_NOT_FOUND = -6,
+} nixl_capi_status_t;
+
+typedef enum {
+    NIXL_CAPI_MEM_DRAM = 0,
+    NIXL_CAPI_MEM_VRAM = 1,
+    NIXL_CAPI_MEM_BLOCK = 2,
+    NIXL_CAPI_MEM_OBJECT = 3,
+    NIXL_CAPI_MEM_FILE = 4,
+    NIXL_CAPI_MEM_UNKNOWN = 5
+} nixl_capi_mem_type_t;
+
+typedef enum {
+    NIXL_CAPI_XFER_OP_READ = 0,
+    NIXL_CAPI_XFER_OP_WRITE = 1,
+} nixl_capi_xfer_op_t;
+
+typedef enum {
+    NIXL_CAPI_THREAD_SYNC_NONE = 0,
+    NIXL_CAPI_THREAD_SYNC_STRICT = 1,
+    NIXL_CAPI_THREAD_SYNC_RW = 2,
+    NIXL_CAPI_THREAD_SYNC_DEFAULT = NIXL_CAPI_THREAD_SYNC_NONE,
+} nixl_capi_thread_sync_t;
+
+typedef struct nixl_capi_agent_config_s {
+    bool enable_prog_thread;
+    bool enable_listen_thread;
+    int listen_port;
+    nixl_capi_thread_sync_t thread_sync;
+    unsigned int num_workers;
+    uint64_t pthr_delay_us;
+    uint64_t lthr_delay_us;
+    bool capture_telemetry;
+} nixl_capi_agent_config_t;
+
+struct nixl_capi_xfer_telemetry_s {
+    uint64_t start_time_us;
+    uint64_t post_duration_us;
+    uint64_t xfer_duration_us;
+    uint64_t total_bytes;
+    uint64_t desc_count;
+};
+
+typedef struct nixl_capi_agent_s *nixl_capi_agent_t;
+typedef struct nixl_capi_params_s *nixl_capi_params_t;
+typedef struct nixl_capi_backend_s *nixl_capi_backend_t;
+typedef struct nixl_capi_opt_args_s *nixl_capi_opt_args_t;
+typedef struct nixl_capi_xfer_dlist_s *nixl_capi_xfer_dlist_t;
+typedef struct nixl_capi_xfer_dlist_handle_s *nixl_capi_xfer_dlist_handle_t;
+typedef struct nixl_capi_reg_dlist_s *nixl_capi_reg_dlist_t;
+typedef struct nixl_capi_xfer_req_s *nixl_capi_xfer_req_t;
+typedef struct nixl_capi_xfer_telemetry_s *nixl_capi_xfer_telemetry_t;
+
+/* agent */
+nixl_capi_status_t nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent);
+nixl_capi_status_t nixl_capi_create_configured_agent(const char *name,
+                                                     const nixl_capi_agent_config_t *cfg,
+                                                     nixl_capi_agent_t *agent);
+nixl_capi_status_t nixl_capi_destroy_agent(nixl_capi_agent_t agent);
+
+/* backend parameters and creation */
+nixl_capi_status_t nixl_capi_create_params(nixl_capi_params_t *params);
+nixl_capi_status_t nixl_capi_params_add(nixl_capi_params_t params, const char *key, const char *value);
+nixl_capi_status_t nixl_capi_destroy_params(nixl_capi_params_t params);
+nixl_capi_status_t nixl_capi_create_backend(nixl_capi_agent_t agent,
+                                            const char *plugin_name,
+                                            nixl_capi_params_t params,
+                                            nixl_capi_backend_t *backend);
+nixl_capi_status_t nixl_capi_destroy_backend(nixl_capi_backend_t backend);
+
+/* optional arguments */
+nixl_capi_status_t nixl_capi_create_opt_args(nixl_capi_opt_args_t *args);
+nixl_capi_status_t nixl_capi_destroy_opt_args(nixl_capi_opt_args_t args);
+nixl_capi_status_t nixl_capi_opt_args_add_backend(nixl_capi_opt_args_t args, nixl_capi_backend_t backend);
+nixl_capi_status_t nixl_capi_opt_args_set_notif_msg(nixl_capi_opt_args_t args, const void *data, size_t len);
+nixl_capi_status_t nixl_capi_opt_args_set_has_notif(nixl_capi_opt_args_t args, bool has_notif);
+nixl_capi_status_t nixl_capi_opt_args_set_skip_desc_merge(nixl_capi_opt_args_t args, bool skip_merge);
+
+/* descriptor lists */
+nixl_capi_status_t nixl_capi_create_xfer_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_xfer_dlist_t *dlist);
+nixl_capi_status_t nixl_capi_destroy_xfer_dlist(nixl_capi_xfer_dlist_t dlist);
+nixl_capi_status_t nixl_capi_xfer_dlist_add_desc(nixl_capi_xfer_dlist_t dlist, uintptr_t addr, size_t len, uint64_t dev_id);
+nixl_capi_status_t nixl_capi_xfer_dlist_desc_count(nixl_capi_xfer_dlist_t dlist, size_t *count);
+nixl_capi_status_t nixl_capi_xfer_dlist_clear(nixl_capi_xfer_dlist_t dlist);
+nixl_capi_status_t nixl_capi_create_reg_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_reg_dlist_t *dlist);
+nixl_capi_status_t nixl_capi_destroy_reg_dlist(nixl_capi_reg_dlist_t dlist);
+nixl_capi_status_t nixl_capi_reg_dlist_add_desc(nixl_capi_reg_dlist_t dlist,
+                                                uintptr_t addr,
+                                                size_t len,
+                                                uint64_t dev_id,
+                                                const void *metadata,
+                                                size_t metadata_len);
+nixl_capi_status_t nixl_capi_reg_dlist_desc_count(nixl_capi_reg_dlist_t dlist, size_t *count);
+
+/* registration */
+nixl_capi_status_t nixl_capi_register_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t dlist, nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_deregister_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t dlist, nixl_capi_opt_args_t opt_args);
+
+/* transfers */
+nixl_capi_status_t nixl_capi_prep_xfer_dlist(nixl_capi_agent_t agent,
+                                             const char *agent_name,
+                                             nixl_capi_xfer_dlist_t descs,
+                                             nixl_capi_xfer_dlist_handle_t *dlist_hndl,
+                                             nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_release_xfer_dlist_handle(nixl_capi_agent_t agent, nixl_capi_xfer_dlist_handle_t dlist_handle);
+nixl_capi_status_t nixl_capi_make_xfer_req(nixl_capi_agent_t agent,
+                                           nixl_capi_xfer_op_t operation,
+                                           nixl_capi_xfer_dlist_handle_t local_descs,
+                                           const int *local_indices,
+                                           size_t local_indices_count,
+                                           nixl_capi_xfer_dlist_handle_t remote_descs,
+                                           const int *remote_indices,
+                                           size_t remote_indices_count,
+                                           nixl_capi_xfer_req_t *req_hndl,
+                                           nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_create_xfer_req(nixl_capi_agent_t agent,
+                                             nixl_capi_xfer_op_t operation,
+                                             nixl_capi_xfer_dlist_t local_descs,
+                                             nixl_capi_xfer_dlist_t remote_descs,
+                                             const char *remote_agent,
+                                             nixl_capi_xfer_req_t *req_hndl,
+                                             nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_post_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_get_xfer_status(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl);
+nixl_capi_status_t nixl_capi_get_xfer_telemetry(nixl_capi_agent_t agent,
+                                                nixl_capi_xfer_req_t req_hndl,
+                                                nixl_capi_xfer_telemetry_t telemetry);
+nixl_capi_status_t nixl_capi_release_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req);
+nixl_capi_status_t nixl_capi_destroy_xfer_req(nixl_capi_xfer_req_t req);
+
+/* ---- extensions ---- */
+
+/* Raw nixl_status_t (src/api/cpp/nixl_types.h:53-68) of the last agent call made through
+ * this API on the calling thread; the coarse nixl_capi_status_t above loses detail. */
+int nixl_capi_last_nixl_status(void);
+
+/* Append n descriptors at once (parallel arrays); dev_ids may be NULL for all-zero. */
+nixl_capi_status_t nixl_capi_xfer_dlist_add_descs(nixl_capi_xfer_dlist_t dlist,
+                                                  const uint64_t *addrs,
+                                                  const uint64_t *lens,
+                                                  const uint64_t *dev_ids,
+                                                  size_t n);
+
+/* Number of descriptors the backend received after index expansion and merging
+ * (nixlXferTelemetry::descCount, src/api/cpp/nixl_types.h:283-287); no telemetry needed. */
+nixl_capi_status_t nixl_capi_xfer_req_desc_count(nixl_capi_xfer_req_t req, size_t *count, size_t *bytes);
+
+/* Copy out descriptor i of the request as resolved for the backend: local (addr, len)
+ * and remote addr. */
+nixl_capi_status_t nixl_capi_xfer_req_get_desc(nixl_capi_xfer_req_t req,
+                                               size_t i,
+                                               uint64_t *local_addr,
+                                               uint64_t *remote_addr,
+                                               uint64_t *len);
+
+/* Number of stride runs a prepared list holds for its first backend. */
+nixl_capi_status_t nixl_capi_xfer_dlist_handle_run_count(nixl_capi_xfer_dlist_handle_t h, size_t *runs);
+
+/* Post, then poll until the request leaves NIXL_IN_PROG; returns the final status.
+ * Saves one foreign-function round trip per poll in timing loops. */
+nixl_capi_status_t nixl_capi_post_and_wait(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NIXL_AMD_CAPI_H */

@@ -1,0 +1,114 @@
+/*
+ * C ABI of the descriptor-copy kernel layer (libnixl_amd_kernels.so).
+ *
+ * This is the lowest drop-in level of the HIP backend: a NIXL transfer request, once the
+ * agent has resolved it to two equally long lists of (address, length) spans, becomes ONE
+ * device-resident copy plan and ONE kernel launch per post.  The reference has no such
+ * layer: its VRAM->VRAM path issues one UCX put/get per descriptor from a host loop
+ * (src/plugins/ucx/ucx_backend.cpp:1216-1244 -> ucp_put_nbx / ucp_get_nbx,
+ * src/plugins/ucx/ucx_utils.cpp:288,313) and then flushes the endpoint (:1246-1262).  The
+ * result that must match is that loop's: for every descriptor i, in list order,
+ * memcpy(dst_i, src_i, len_i).
+ *
+ * All handles are plain pointers; `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Every function returns 0 on success or a negative nixl_amd_status
+ * value; nixl_amd_last_error() gives the text of the last failure on the calling thread.
+ * No function falls back to a host copy: without a usable HIP device they fail.
+ */
+#ifndef NIXL_AMD_HIP_H
+#define NIXL_AMD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum nixl_amd_status {
+    NIXL_AMD_OK = 0,
+    NIXL_AMD_ERR_INVALID = -1, /* bad argument (null pointer, zero count, bad variant) */
+    NIXL_AMD_ERR_HIP = -2, /* a HIP runtime call failed; see nixl_amd_last_error() */
+    NIXL_AMD_ERR_NO_DEVICE = -3, /* no gfx950-class device visible */
+    NIXL_AMD_ERR_BUSY = -4, /* plan destroyed or relaunched while still running */
+    NIXL_AMD_ERR_TOO_LARGE = -5 /* request exceeds a documented fixed limit */
+};
+
+/* One span to copy: `len` bytes from device address `src` to device address `dst`.
+ * This is one (local, remote) pair of nixlMetaDesc entries
+ * (src/api/cpp/backend/backend_aux.h:92-105) with the direction already applied:
+ * NIXL_WRITE copies local->remote, NIXL_READ remote->local
+ * (src/plugins/ucx/ucx_backend.cpp:1227-1229). */
+typedef struct nixl_amd_copy_desc {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t len;
+} nixl_amd_copy_desc_t;
+
+/* Launch-shape knobs.  Zero in any field selects the built-in default. */
+typedef struct nixl_amd_copy_tuning {
+    int units_per_lane; /* 16-byte units one lane moves per chunk: 4, 8 or 16 */
+    int nontemporal; /* 1 = non-temporal loads/stores, 2 = plain; 0 = default */
+    int max_workgroups; /* grid cap; waves loop over chunks beyond it */
+} nixl_amd_copy_tuning_t;
+
+typedef struct nixl_amd_copy_plan nixl_amd_copy_plan_t;
+
+/* Text of the most recent error on this thread ("" if none). */
+const char *
+nixl_amd_last_error(void);
+
+/* Number of HIP devices, or a negative status. */
+int
+nixl_amd_device_count(void);
+
+/* Lower `n` host-side descriptors into a device-resident plan on `device`.
+ * Replaces the per-request set-up of nixlUcxEngine::prepXfer
+ * (src/plugins/ucx/ucx_backend.cpp:1061-1084), which defers all work to post time.
+ * Zero-length descriptors are dropped.  Descriptors whose src, dst and len are all
+ * multiples of 16 take the 128-bit streaming path; all others take a byte-exact path.
+ * The descriptor array may be freed as soon as this returns. */
+int
+nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
+                          size_t n,
+                          int device,
+                          const nixl_amd_copy_tuning_t *tuning,
+                          nixl_amd_copy_plan_t **out);
+
+/* Enqueue the whole plan on `stream`: the per-post work of
+ * nixlUcxEngine::postXfer -> sendXferRange (src/plugins/ucx/ucx_backend.cpp:1183-1310).
+ * Re-launching re-reads the current source bytes; nothing is cached at plan creation
+ * (repost semantics of test/unit/plugins/posix/nixl_posix_test.cpp:714-770). */
+int
+nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream);
+
+/* Free the plan's device arrays.  The caller must have synchronised with every launch. */
+int
+nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan);
+
+/* Plan facts: total payload bytes, descriptors on the 128-bit path, descriptors on the
+ * byte path, device bytes held by the plan's own arrays, workgroups per launch. */
+typedef struct nixl_amd_copy_plan_info {
+    uint64_t payload_bytes;
+    uint64_t vec_descs;
+    uint64_t generic_descs;
+    uint64_t plan_device_bytes;
+    uint32_t vec_chunks;
+    uint32_t vec_workgroups;
+    uint32_t generic_items;
+    uint32_t units_per_lane;
+} nixl_amd_copy_plan_info_t;
+
+int
+nixl_amd_copy_plan_query(const nixl_amd_copy_plan_t *plan, nixl_amd_copy_plan_info_t *info);
+
+/* Convenience: launch the plan `iters` times back to back on `stream`, bracketed by HIP
+ * events recorded on that same stream, wait, and return the mean milliseconds per launch.
+ * Used by benchmarks to time the kernel itself. */
+int
+nixl_amd_copy_plan_time(nixl_amd_copy_plan_t *plan, void *stream, int iters, float *ms_per_launch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NIXL_AMD_HIP_H */

@@ -1,0 +1,159 @@
+"""ctypes loaders for the in-tree native libraries.
+
+The libraries are built by ``__graft_entry__.build()`` (``make -C nixl_amd/csrc``) into
+``nixl_amd/lib``.  Nothing here builds, and nothing falls back to Python or to a CPU
+implementation: a missing library raises ``NativeLibraryMissing``.
+"""
+import ctypes
+import os
+from ctypes import (POINTER, Structure, c_bool, c_char_p, c_float, c_int, c_int64, c_size_t,
+                    c_uint, c_uint32, c_uint64, c_void_p)
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+PLUGIN_DIR = os.path.join(LIB_DIR, "plugins")
+
+
+class NativeLibraryMissing(RuntimeError):
+    pass
+
+
+def _load(name):
+    path = os.path.join(LIB_DIR, name)
+    if not os.path.exists(path):
+        raise NativeLibraryMissing(
+            f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or `make -C nixl_amd/csrc`) first")
+    return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+# ---------------------------------------------------------------------------------------
+# Kernel layer (include/nixl_amd_hip.h, include/nixl_amd_ep.h)
+# ---------------------------------------------------------------------------------------
+
+class CopyDesc(Structure):
+    _fields_ = [("src", c_uint64), ("dst", c_uint64), ("len", c_uint64)]
+
+
+class CopyTuning(Structure):
+    _fields_ = [("units_per_lane", c_int), ("nontemporal", c_int), ("max_workgroups", c_int)]
+
+
+class CopyPlanInfo(Structure):
+    _fields_ = [("payload_bytes", c_uint64), ("vec_descs", c_uint64), ("generic_descs", c_uint64),
+                ("plan_device_bytes", c_uint64), ("vec_chunks", c_uint32),
+                ("vec_workgroups", c_uint32), ("generic_items", c_uint32),
+                ("units_per_lane", c_uint32)]
+
+
+_kernels = None
+
+
+def kernels():
+    """libnixl_amd_kernels.so with argument types declared."""
+    global _kernels
+    if _kernels is not None:
+        return _kernels
+    lib = _load("libnixl_amd_kernels.so")
+    lib.nixl_amd_last_error.restype = c_char_p
+    lib.nixl_amd_device_count.restype = c_int
+    lib.nixl_amd_copy_plan_create.argtypes = [POINTER(CopyDesc), c_size_t, c_int,
+                                              POINTER(CopyTuning), POINTER(c_void_p)]
+    lib.nixl_amd_copy_plan_launch.argtypes = [c_void_p, c_void_p]
+    lib.nixl_amd_copy_plan_destroy.argtypes = [c_void_p]
+    lib.nixl_amd_copy_plan_query.argtypes = [c_void_p, POINTER(CopyPlanInfo)]
+    lib.nixl_amd_copy_plan_time.argtypes = [c_void_p, c_void_p, c_int, POINTER(c_float)]
+    for fn in ("nixl_amd_copy_plan_create", "nixl_amd_copy_plan_launch",
+               "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
+               "nixl_amd_copy_plan_time"):
+        getattr(lib, fn).restype = c_int
+    _kernels = lib
+    return lib
+
+
+def kernels_error():
+    return kernels().nixl_amd_last_error().decode()
+
+
+# ---------------------------------------------------------------------------------------
+# Agent C API (include/nixl_amd_capi.h)
+# ---------------------------------------------------------------------------------------
+
+class AgentConfig(Structure):
+    _fields_ = [("enable_prog_thread", c_bool), ("enable_listen_thread", c_bool),
+                ("listen_port", c_int), ("thread_sync", c_int), ("num_workers", c_uint),
+                ("pthr_delay_us", c_uint64), ("lthr_delay_us", c_uint64),
+                ("capture_telemetry", c_bool)]
+
+
+class XferTelemetry(Structure):
+    _fields_ = [("start_time_us", c_uint64), ("post_duration_us", c_uint64),
+                ("xfer_duration_us", c_uint64), ("total_bytes", c_uint64),
+                ("desc_count", c_uint64)]
+
+
+_agent = None
+
+_CAPI_SIGS = {
+    "nixl_capi_create_agent": [c_char_p, POINTER(c_void_p)],
+    "nixl_capi_create_configured_agent": [c_char_p, POINTER(AgentConfig), POINTER(c_void_p)],
+    "nixl_capi_destroy_agent": [c_void_p],
+    "nixl_capi_create_params": [POINTER(c_void_p)],
+    "nixl_capi_params_add": [c_void_p, c_char_p, c_char_p],
+    "nixl_capi_destroy_params": [c_void_p],
+    "nixl_capi_create_backend": [c_void_p, c_char_p, c_void_p, POINTER(c_void_p)],
+    "nixl_capi_destroy_backend": [c_void_p],
+    "nixl_capi_create_opt_args": [POINTER(c_void_p)],
+    "nixl_capi_destroy_opt_args": [c_void_p],
+    "nixl_capi_opt_args_add_backend": [c_void_p, c_void_p],
+    "nixl_capi_opt_args_set_notif_msg": [c_void_p, c_char_p, c_size_t],
+    "nixl_capi_opt_args_set_has_notif": [c_void_p, c_bool],
+    "nixl_capi_opt_args_set_skip_desc_merge": [c_void_p, c_bool],
+    "nixl_capi_create_xfer_dlist": [c_int, POINTER(c_void_p)],
+    "nixl_capi_destroy_xfer_dlist": [c_void_p],
+    "nixl_capi_xfer_dlist_add_desc": [c_void_p, c_uint64, c_size_t, c_uint64],
+    "nixl_capi_xfer_dlist_add_descs": [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t],
+    "nixl_capi_xfer_dlist_desc_count": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_xfer_dlist_clear": [c_void_p],
+    "nixl_capi_create_reg_dlist": [c_int, POINTER(c_void_p)],
+    "nixl_capi_destroy_reg_dlist": [c_void_p],
+    "nixl_capi_reg_dlist_add_desc": [c_void_p, c_uint64, c_size_t, c_uint64, c_char_p, c_size_t],
+    "nixl_capi_reg_dlist_desc_count": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_register_mem": [c_void_p, c_void_p, c_void_p],
+    "nixl_capi_deregister_mem": [c_void_p, c_void_p, c_void_p],
+    "nixl_capi_prep_xfer_dlist": [c_void_p, c_char_p, c_void_p, POINTER(c_void_p), c_void_p],
+    "nixl_capi_release_xfer_dlist_handle": [c_void_p, c_void_p],
+    "nixl_capi_xfer_dlist_handle_run_count": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_make_xfer_req": [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
+                                c_size_t, POINTER(c_void_p), c_void_p],
+    "nixl_capi_create_xfer_req": [c_void_p, c_int, c_void_p, c_void_p, c_char_p,
+                                  POINTER(c_void_p), c_void_p],
+    "nixl_capi_post_xfer_req": [c_void_p, c_void_p, c_void_p],
+    "nixl_capi_get_xfer_status": [c_void_p, c_void_p],
+    "nixl_capi_post_and_wait": [c_void_p, c_void_p],
+    "nixl_capi_get_xfer_telemetry": [c_void_p, c_void_p, POINTER(XferTelemetry)],
+    "nixl_capi_xfer_req_desc_count": [c_void_p, POINTER(c_size_t), POINTER(c_size_t)],
+    "nixl_capi_xfer_req_get_desc": [c_void_p, c_size_t, POINTER(c_uint64), POINTER(c_uint64),
+                                    POINTER(c_uint64)],
+    "nixl_capi_release_xfer_req": [c_void_p, c_void_p],
+    "nixl_capi_destroy_xfer_req": [c_void_p],
+}
+
+
+def agent_lib():
+    """libnixl_amd_agent.so with argument types declared."""
+    global _agent
+    if _agent is not None:
+        return _agent
+    lib = _load("libnixl_amd_agent.so")
+    for name, args in _CAPI_SIGS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    lib.nixl_capi_last_nixl_status.restype = c_int
+    _agent = lib
+    return lib
+
+
+def capi_symbols():
+    return sorted(list(_CAPI_SIGS) + ["nixl_capi_last_nixl_status"])

@@ -1,0 +1,349 @@
+"""Python view of the agent, shaped after the reference's ``nixl_agent``
+(src/api/python/_api.py:189-1221): same method names, argument meaning and "DONE" /
+"PROC" / "ERR" transfer states, over the C ABI in include/nixl_amd_capi.h.
+
+Descriptor lists are numpy ``uint64`` arrays of shape (N, 3) holding (addr, len, devId),
+lists of such triples, or lists of torch tensors (reference: get_xfer_descs,
+_api.py:999-1092).  Only the single-agent loopback subset exists; there is no metadata
+exchange or notification path.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import _lib
+
+NIXL_INIT_AGENT = ""
+
+# nixl_status_t, src/api/cpp/nixl_types.h:53-68
+NIXL_IN_PROG = 1
+NIXL_SUCCESS = 0
+NIXL_ERR_NOT_POSTED = -1
+NIXL_ERR_INVALID_PARAM = -2
+NIXL_ERR_BACKEND = -3
+NIXL_ERR_NOT_FOUND = -4
+NIXL_ERR_MISMATCH = -5
+NIXL_ERR_NOT_ALLOWED = -6
+NIXL_ERR_REPOST_ACTIVE = -7
+NIXL_ERR_UNKNOWN = -8
+NIXL_ERR_NOT_SUPPORTED = -9
+NIXL_ERR_REMOTE_DISCONNECT = -10
+NIXL_ERR_CANCELED = -11
+NIXL_ERR_NO_TELEMETRY = -12
+
+_STATUS_NAMES = {v: k for k, v in list(globals().items()) if k.startswith("NIXL_") and isinstance(v, int)}
+
+_MEM = {"DRAM": 0, "VRAM": 1, "BLOCK": 2, "BLK": 2, "OBJ": 3, "FILE": 4,
+        "cpu": 0, "cuda": 1}
+
+
+class NixlError(RuntimeError):
+    """A nixl_status_t error (reference bindings raise one exception class per code)."""
+
+    def __init__(self, where, capi_status, nixl_status):
+        self.capi_status = capi_status
+        self.status = nixl_status
+        super().__init__(f"{where}: {_STATUS_NAMES.get(nixl_status, nixl_status)} (capi {capi_status})")
+
+
+def _check(where, rc, ok=(0,)):
+    if rc not in ok:
+        st = _lib.agent_lib().nixl_capi_last_nixl_status() if rc not in (-1, -3, -4) else NIXL_ERR_INVALID_PARAM
+        raise NixlError(where, rc, st)
+    return rc
+
+
+def _as_triples(descs):
+    """Normalise a descriptor list to a C-contiguous (N, 3) uint64 array."""
+    if isinstance(descs, np.ndarray):
+        arr = descs
+    else:
+        rows = []
+        for d in descs:
+            if hasattr(d, "data_ptr"):
+                dev = d.device.index if d.device.type == "cuda" and d.device.index is not None else 0
+                rows.append((d.data_ptr(), d.numel() * d.element_size(), dev))
+            else:
+                rows.append(tuple(d)[:3])
+        arr = np.array(rows, dtype=np.uint64).reshape(-1, 3)
+    if arr.ndim != 2 or arr.shape[1] != 3:
+        raise ValueError("descriptor array must have shape (N, 3): addr, len, devId")
+    return np.ascontiguousarray(arr, dtype=np.uint64)
+
+
+def _guess_mem(descs, mem_type):
+    if mem_type is not None:
+        return _MEM[mem_type]
+    if not isinstance(descs, np.ndarray) and len(descs) and hasattr(descs[0], "data_ptr"):
+        return _MEM[descs[0].device.type]
+    raise ValueError("mem_type is required for raw address lists")
+
+
+class nixl_agent_config:
+    """Reference: nixl_agent_config, src/api/python/_api.py:148-186."""
+
+    def __init__(self, enable_prog_thread=True, enable_listen_thread=False, listen_port=0,
+                 capture_telemetry=False, num_threads=0, backends=("HIP",)):
+        self.enable_pthread = enable_prog_thread
+        self.enable_listen = enable_listen_thread
+        self.port = listen_port
+        self.capture_telemetry = capture_telemetry
+        self.num_threads = num_threads
+        self.backends = list(backends)
+
+
+class nixl_xfer_dlist:
+    """Owned nixl_xfer_dlist_t (what get_xfer_descs returns in the reference)."""
+
+    def __init__(self, triples, mem):
+        self._lib = _lib.agent_lib()
+        self.mem = mem
+        self.triples = triples
+        h = ctypes.c_void_p()
+        _check("create_xfer_dlist", self._lib.nixl_capi_create_xfer_dlist(mem, ctypes.byref(h)))
+        self._h = h
+        n = triples.shape[0]
+        if n:
+            addrs = np.ascontiguousarray(triples[:, 0])
+            lens = np.ascontiguousarray(triples[:, 1])
+            devs = np.ascontiguousarray(triples[:, 2])
+            _check("xfer_dlist_add_descs",
+                   self._lib.nixl_capi_xfer_dlist_add_descs(h, addrs.ctypes.data, lens.ctypes.data,
+                                                            devs.ctypes.data, n))
+
+    def descCount(self):
+        return int(self.triples.shape[0])
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.nixl_capi_destroy_xfer_dlist(self._h)
+            self._h = None
+
+
+class nixl_reg_dlist:
+    def __init__(self, triples, mem):
+        self._lib = _lib.agent_lib()
+        self.mem = mem
+        self.triples = triples
+        h = ctypes.c_void_p()
+        _check("create_reg_dlist", self._lib.nixl_capi_create_reg_dlist(mem, ctypes.byref(h)))
+        self._h = h
+        for a, l, d in triples:
+            _check("reg_dlist_add_desc", self._lib.nixl_capi_reg_dlist_add_desc(h, int(a), int(l), int(d), None, 0))
+
+    def descCount(self):
+        return int(self.triples.shape[0])
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.nixl_capi_destroy_reg_dlist(self._h)
+            self._h = None
+
+
+class nixl_prepped_dlist_handle:
+    """Reference: _api.py:49-86."""
+
+    def __init__(self, agent, value):
+        self._agent = agent
+        self._handle = value
+
+    def release(self):
+        if self._handle:
+            self._agent.release_dlist_handle(self)
+
+    def run_count(self):
+        n = ctypes.c_size_t()
+        _check("run_count", _lib.agent_lib().nixl_capi_xfer_dlist_handle_run_count(self._handle, ctypes.byref(n)))
+        return n.value
+
+
+class nixl_xfer_handle:
+    """Reference: _api.py:89-127."""
+
+    def __init__(self, agent, value):
+        self._agent = agent
+        self._handle = value
+
+    def release(self):
+        if self._handle:
+            self._agent.release_xfer_handle(self)
+
+    def desc_count(self):
+        n, b = ctypes.c_size_t(), ctypes.c_size_t()
+        _check("desc_count", _lib.agent_lib().nixl_capi_xfer_req_desc_count(self._handle, ctypes.byref(n), ctypes.byref(b)))
+        return n.value, b.value
+
+    def get_desc(self, i):
+        la, ra, ln = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
+        _check("get_desc", _lib.agent_lib().nixl_capi_xfer_req_get_desc(self._handle, i, ctypes.byref(la), ctypes.byref(ra), ctypes.byref(ln)))
+        return la.value, ra.value, ln.value
+
+
+class nixl_agent:
+    """Reference: nixl_agent, src/api/python/_api.py:189-296."""
+
+    def __init__(self, agent_name, nixl_conf=None, plugin_dirs=()):
+        self._lib = _lib.agent_lib()
+        self.name = agent_name
+        conf = nixl_conf or nixl_agent_config(backends=())
+        dirs = [_lib.PLUGIN_DIR] + list(plugin_dirs)
+        prev = os.environ.get("NIXL_PLUGIN_DIR")
+        if prev:
+            dirs.append(prev)
+        os.environ["NIXL_PLUGIN_DIR"] = ":".join(dict.fromkeys(dirs))
+        cfg = _lib.AgentConfig(conf.enable_pthread, conf.enable_listen, conf.port, 0, 1, 0, 100000,
+                               conf.capture_telemetry)
+        h = ctypes.c_void_p()
+        _check("create_agent", self._lib.nixl_capi_create_configured_agent(agent_name.encode(), ctypes.byref(cfg), ctypes.byref(h)))
+        self._h = h
+        self.backends = {}
+        self.nixl_ops = {"WRITE": 1, "READ": 0}
+        for b in conf.backends:
+            self.create_backend(b)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            for b in self.backends.values():
+                self._lib.nixl_capi_destroy_backend(b)
+            self.backends = {}
+            self._lib.nixl_capi_destroy_agent(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    # -- backends ---------------------------------------------------------------------
+    def create_backend(self, backend, initParams=None):
+        params = ctypes.c_void_p()
+        _check("create_params", self._lib.nixl_capi_create_params(ctypes.byref(params)))
+        try:
+            for k, v in (initParams or {}).items():
+                _check("params_add", self._lib.nixl_capi_params_add(params, str(k).encode(), str(v).encode()))
+            h = ctypes.c_void_p()
+            _check(f"create_backend({backend})",
+                   self._lib.nixl_capi_create_backend(self._h, backend.encode(), params, ctypes.byref(h)))
+            self.backends[backend] = h
+        finally:
+            self._lib.nixl_capi_destroy_params(params)
+
+    def _opt_args(self, backends=(), skip_desc_merge=False, notif_msg=b""):
+        if not backends and not skip_desc_merge and not notif_msg:
+            return None
+        o = ctypes.c_void_p()
+        _check("create_opt_args", self._lib.nixl_capi_create_opt_args(ctypes.byref(o)))
+        for b in backends:
+            self._lib.nixl_capi_opt_args_add_backend(o, self.backends[b])
+        if skip_desc_merge:
+            self._lib.nixl_capi_opt_args_set_skip_desc_merge(o, True)
+        if notif_msg:
+            self._lib.nixl_capi_opt_args_set_notif_msg(o, notif_msg, len(notif_msg))
+            self._lib.nixl_capi_opt_args_set_has_notif(o, True)
+        return o
+
+    def _free_opt(self, o):
+        if o:
+            self._lib.nixl_capi_destroy_opt_args(o)
+
+    # -- descriptors ------------------------------------------------------------------
+    def get_xfer_descs(self, descs, mem_type=None):
+        if isinstance(descs, nixl_xfer_dlist):
+            return descs
+        return nixl_xfer_dlist(_as_triples(descs), _guess_mem(descs, mem_type))
+
+    def get_reg_descs(self, descs, mem_type=None):
+        if isinstance(descs, nixl_reg_dlist):
+            return descs
+        return nixl_reg_dlist(_as_triples(descs), _guess_mem(descs, mem_type))
+
+    # -- registration -----------------------------------------------------------------
+    def register_memory(self, reg_list, mem_type=None, backends=()):
+        reg = self.get_reg_descs(reg_list, mem_type)
+        o = self._opt_args(backends)
+        try:
+            _check("register_memory", self._lib.nixl_capi_register_mem(self._h, reg._h, o))
+        finally:
+            self._free_opt(o)
+        return reg
+
+    def deregister_memory(self, dereg_list, backends=()):
+        o = self._opt_args(backends)
+        try:
+            _check("deregister_memory", self._lib.nixl_capi_deregister_mem(self._h, dereg_list._h, o))
+        finally:
+            self._free_opt(o)
+
+    # -- transfers --------------------------------------------------------------------
+    def prep_xfer_dlist(self, agent_name, xfer_list, mem_type=None, backends=()):
+        descs = self.get_xfer_descs(xfer_list, mem_type)
+        if agent_name == "NIXL_INIT_AGENT":
+            agent_name = NIXL_INIT_AGENT
+        o = self._opt_args(backends)
+        h = ctypes.c_void_p()
+        try:
+            _check("prep_xfer_dlist",
+                   self._lib.nixl_capi_prep_xfer_dlist(self._h, agent_name.encode(), descs._h, ctypes.byref(h), o))
+        finally:
+            self._free_opt(o)
+        return nixl_prepped_dlist_handle(self, h)
+
+    def make_prepped_xfer(self, operation, local_xfer_side, local_indices, remote_xfer_side,
+                          remote_indices, notif_msg=b"", backends=(), skip_desc_merge=False):
+        li = np.ascontiguousarray(local_indices, dtype=np.int32)
+        ri = np.ascontiguousarray(remote_indices, dtype=np.int32)
+        o = self._opt_args(backends, skip_desc_merge, notif_msg)
+        h = ctypes.c_void_p()
+        try:
+            _check("make_prepped_xfer",
+                   self._lib.nixl_capi_make_xfer_req(self._h, self.nixl_ops[operation], local_xfer_side._handle,
+                                                     li.ctypes.data, li.size, remote_xfer_side._handle,
+                                                     ri.ctypes.data, ri.size, ctypes.byref(h), o))
+        finally:
+            self._free_opt(o)
+        return nixl_xfer_handle(self, h)
+
+    def initialize_xfer(self, operation, local_descs, remote_descs, remote_agent, notif_msg=b"", backends=()):
+        o = self._opt_args(backends, False, notif_msg)
+        h = ctypes.c_void_p()
+        try:
+            _check("initialize_xfer",
+                   self._lib.nixl_capi_create_xfer_req(self._h, self.nixl_ops[operation], local_descs._h,
+                                                       remote_descs._h, remote_agent.encode(), ctypes.byref(h), o))
+        finally:
+            self._free_opt(o)
+        return nixl_xfer_handle(self, h)
+
+    @staticmethod
+    def _state(rc):
+        return "DONE" if rc == 0 else ("PROC" if rc == 1 else "ERR")
+
+    def transfer(self, handle, notif_msg=b""):
+        o = self._opt_args((), False, notif_msg)
+        try:
+            return self._state(self._lib.nixl_capi_post_xfer_req(self._h, handle._handle, o))
+        finally:
+            self._free_opt(o)
+
+    def check_xfer_state(self, handle):
+        return self._state(self._lib.nixl_capi_get_xfer_status(self._h, handle._handle))
+
+    def transfer_and_wait(self, handle):
+        """Post and poll to completion inside native code (no reference counterpart)."""
+        return self._state(self._lib.nixl_capi_post_and_wait(self._h, handle._handle))
+
+    def last_status(self):
+        return self._lib.nixl_capi_last_nixl_status()
+
+    def get_xfer_telemetry(self, handle):
+        t = _lib.XferTelemetry()
+        _check("get_xfer_telemetry", self._lib.nixl_capi_get_xfer_telemetry(self._h, handle._handle, ctypes.byref(t)))
+        return t
+
+    def release_xfer_handle(self, handle):
+        _check("release_xfer_handle", self._lib.nixl_capi_release_xfer_req(self._h, handle._handle))
+        self._lib.nixl_capi_destroy_xfer_req(handle._handle)
+        handle._handle = None
+
+    def release_dlist_handle(self, handle):
+        _check("release_dlist_handle", self._lib.nixl_capi_release_xfer_dlist_handle(self._h, handle._handle))
+        handle._handle = None

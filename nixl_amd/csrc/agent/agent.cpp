@@ -1,0 +1,965 @@
+// Single-process nixlAgent for the descriptor-transfer path.  Each public member follows
+// the observable behaviour (argument checks, status codes, the sequence of south-bound
+// calls a backend sees) of the reference member cited above it.
+#include <dlfcn.h>
+
+#include <algorithm>
+#include <cstdlib>
+#include <filesystem>
+#include <mutex>
+
+#include "agent_impl.h"
+#include "common/nixl_log.h"
+
+namespace fs = std::filesystem;
+
+// =====================================================================================
+// Plugin cache (reference: src/core/nixl_plugin_manager.cpp:94-122,334-359,385-399,463-529)
+// =====================================================================================
+
+nixlPluginCache &
+nixlPluginCache::instance() {
+    static nixlPluginCache cache;
+    return cache;
+}
+
+std::vector<std::string>
+nixlPluginCache::searchDirs() const {
+    std::vector<std::string> dirs;
+    if (const char *env = std::getenv("NIXL_PLUGIN_DIR")) {
+        std::string s(env);
+        size_t pos = 0;
+        while (pos <= s.size()) {
+            const size_t colon = s.find(':', pos);
+            const std::string part = s.substr(pos, colon == std::string::npos ? std::string::npos : colon - pos);
+            if (!part.empty()) dirs.push_back(part);
+            if (colon == std::string::npos) break;
+            pos = colon + 1;
+        }
+    }
+    Dl_info info;
+    if (dladdr(reinterpret_cast<void *>(&nixlPluginCache::instance), &info) && info.dli_fname)
+        dirs.push_back((fs::path(info.dli_fname).parent_path() / "plugins").string());
+    return dirs;
+}
+
+const nixlLoadedPlugin *
+nixlPluginCache::load(const std::string &type) {
+    std::lock_guard<std::mutex> guard(mutex_);
+    const auto hit = loaded_.find(type);
+    if (hit != loaded_.end()) return &hit->second;
+
+    for (const std::string &dir : searchDirs()) {
+        const fs::path path = fs::path(dir) / ("libplugin_" + type + ".so");
+        std::error_code ec;
+        if (!fs::exists(path, ec)) continue;
+        // NODELETE: a plugin's static tables must outlive every engine it created.
+        void *dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL | RTLD_NODELETE);
+        if (!dl) {
+            NIXL_WARN << "cannot load " << path.string() << ": " << dlerror();
+            continue;
+        }
+        using init_fn = nixlBackendPlugin *(*)();
+        auto init = reinterpret_cast<init_fn>(dlsym(dl, "nixl_plugin_init"));
+        nixlBackendPlugin *table = init ? init() : nullptr;
+        if (!table || table->api_version != NIXL_PLUGIN_API_VERSION) {
+            NIXL_ERROR << path.string() << ": missing nixl_plugin_init, null table or API version mismatch";
+            dlclose(dl);
+            continue;
+        }
+        nixlLoadedPlugin &slot = loaded_[type];
+        slot.dl = dl;
+        slot.table = table;
+        slot.path = path.string();
+        return &slot;
+    }
+    return nullptr;
+}
+
+std::vector<std::string>
+nixlPluginCache::discover() const {
+    std::set<std::string> names;
+    for (const std::string &dir : searchDirs()) {
+        std::error_code ec;
+        for (fs::directory_iterator it(dir, ec), end; !ec && it != end; it.increment(ec)) {
+            const std::string f = it->path().filename().string();
+            if (f.size() > 13 && f.rfind("libplugin_", 0) == 0 && f.substr(f.size() - 3) == ".so")
+                names.insert(f.substr(10, f.size() - 13));
+        }
+    }
+    return {names.begin(), names.end()};
+}
+
+// =====================================================================================
+// Registered-memory sections
+// =====================================================================================
+
+void
+nixlSecDescList::add(std::vector<nixlSectionDesc> batch) {
+    if (batch.empty()) return;
+    std::sort(batch.begin(), batch.end());
+    std::vector<nixlSectionDesc> merged;
+    merged.reserve(descs_.size() + batch.size());
+    // Stable merge: existing entries stay ahead of equal new ones, duplicates are kept.
+    std::merge(descs_.begin(), descs_.end(), batch.begin(), batch.end(), std::back_inserter(merged));
+    descs_ = std::move(merged);
+}
+
+int
+nixlSecDescList::indexOf(const nixlBasicDesc &query) const {
+    const auto it = std::lower_bound(descs_.begin(), descs_.end(), query);
+    if (it == descs_.end() || static_cast<const nixlBasicDesc &>(*it) != query) return -1;
+    return static_cast<int>(it - descs_.begin());
+}
+
+int
+nixlSecDescList::coveringIndex(const nixlBasicDesc &query) const {
+    // First region not ordered before the query: a hit only if it starts exactly at the
+    // query's address.  Otherwise the only candidate is the region just before it.
+    const auto it = std::lower_bound(descs_.begin(), descs_.end(), query);
+    if (it != descs_.end() && it->covers(query)) return static_cast<int>(it - descs_.begin());
+    if (it != descs_.begin() && std::prev(it)->covers(query)) return static_cast<int>(it - descs_.begin()) - 1;
+    return -1;
+}
+
+void
+nixlSecDescList::removeAt(std::vector<size_t> indices) {
+    std::sort(indices.begin(), indices.end());
+    indices.erase(std::unique(indices.begin(), indices.end()), indices.end());
+    size_t out = 0, next = 0;
+    for (size_t i = 0; i < descs_.size(); ++i) {
+        if (next < indices.size() && indices[next] == i) {
+            ++next;
+            continue;
+        }
+        if (out != i) descs_[out] = std::move(descs_[i]);
+        ++out;
+    }
+    descs_.resize(out);
+}
+
+const std::set<nixlBackendEngine *> *
+nixlMemSection::backendsFor(nixl_mem_t mem) const {
+    if (mem < DRAM_SEG || mem > FILE_SEG) return nullptr;
+    return &memToBackend[mem];
+}
+
+// reference: src/infra/nixl_memory_section.cpp:56-104
+nixl_status_t
+nixlMemSection::populate(const nixl_xfer_dlist_t &query, nixlBackendEngine *backend, nixl_meta_dlist_t &resp) const {
+    if (query.getType() != resp.getType() || query.isEmpty()) return NIXL_ERR_INVALID_PARAM;
+    const auto sec = sections.find({query.getType(), backend});
+    if (sec == sections.end()) return NIXL_ERR_NOT_FOUND;
+    const nixlSecDescList &base = sec->second;
+    const int n_base = static_cast<int>(base.size());
+    const int n = query.descCount();
+
+    resp.clear();
+    resp.reserve(n);
+    int at = -1;
+    for (int i = 0; i < n; ++i) {
+        const nixlBasicDesc &q = query[i];
+        if (i == 0 || q < query[i - 1]) {
+            at = base.coveringIndex(q);
+        } else {
+            while (at < n_base && !base[at].covers(q))
+                ++at;
+            if (at == n_base) at = -1;
+        }
+        if (at < 0) {
+            resp.clear();
+            return NIXL_ERR_UNKNOWN;
+        }
+        resp.emplace(q.addr, q.len, q.devId, base[at].metadataP);
+    }
+    return NIXL_SUCCESS;
+}
+
+// reference: src/infra/nixl_memory_section.cpp:106-184
+nixl_status_t
+nixlMemSection::populate(const nixl_xfer_dlist_t &query,
+                         nixlBackendEngine *backend,
+                         nixl_stride_dlist_t &resp) const {
+    if (query.getType() != resp.getType() || query.isEmpty()) return NIXL_ERR_INVALID_PARAM;
+    const auto sec = sections.find({query.getType(), backend});
+    if (sec == sections.end()) return NIXL_ERR_NOT_FOUND;
+    const nixlSecDescList &base = sec->second;
+    const int n_base = static_cast<int>(base.size());
+    const int n = query.descCount();
+
+    resp.clear();
+    int at = base.coveringIndex(query[0]);
+    if (at < 0) return NIXL_ERR_UNKNOWN;
+
+    nixlStrideDesc run(query[0].addr, query[0].len, query[0].devId, base[at].metadataP, query[0].len, 1);
+    uintptr_t prev = query[0].addr;
+    for (int i = 1; i < n; ++i) {
+        const nixlBasicDesc &q = query[i];
+        if (!base[at].covers(q)) {
+            if (q < query[i - 1]) {
+                at = base.coveringIndex(q);
+            } else {
+                while (at < n_base && !base[at].covers(q))
+                    ++at;
+                if (at == n_base) at = -1;
+            }
+            if (at < 0) {
+                resp.clear();
+                return NIXL_ERR_UNKNOWN;
+            }
+        }
+        nixlBackendMD *const md = base[at].metadataP;
+
+        // A run continues while length, device and covering registration stay the same
+        // and the address keeps advancing by the run's stride; the second element of a
+        // run fixes that stride and must lie at a strictly higher address.
+        bool extends = (q.len == run.len && q.devId == run.devId && md == run.metadataP);
+        if (extends) {
+            if (run.count == 1) {
+                extends = q.addr > prev;
+                if (extends) run.stride = q.addr - prev;
+            } else {
+                extends = (q.addr - prev) == run.stride;
+            }
+        }
+        if (extends) {
+            ++run.count;
+        } else {
+            resp.addDesc(run);
+            run = nixlStrideDesc(q.addr, q.len, q.devId, md, q.len, 1);
+            run.start_idx = static_cast<size_t>(i);
+        }
+        prev = q.addr;
+    }
+    resp.addDesc(run);
+    return NIXL_SUCCESS;
+}
+
+// =====================================================================================
+// Agent
+// =====================================================================================
+
+nixlAgentData::~nixlAgentData() {
+    // Deregister whatever the application left registered, then destroy engines through
+    // the plugin that made them (reference: src/infra/nixl_memory_section.cpp:416-423).
+    for (auto &[key, list] : localSection_.sections)
+        for (size_t i = 0; i < list.size(); ++i)
+            key.second->deregisterMem(list[i].metadataP);
+    for (auto it = engines_.rbegin(); it != engines_.rend(); ++it)
+        if ((*it)->engine) (*it)->plugin->table->destroy_engine((*it)->engine);
+}
+
+nixlAgentData::engineSlot *
+nixlAgentData::slotOf(const nixl_backend_t &type) const {
+    for (const auto &s : engines_)
+        if (s->engine->getType() == type) return s.get();
+    return nullptr;
+}
+
+nixlAgent::nixlAgent(const std::string &name, const nixlAgentConfig &cfg)
+    : data(std::make_unique<nixlAgentData>(name, cfg)) {
+    if (name.empty()) throw std::invalid_argument("Agent needs a name");
+}
+
+nixlAgent::~nixlAgent() = default;
+
+// reference: src/core/nixl_agent.cpp:254-263
+nixl_status_t
+nixlAgent::getAvailPlugins(std::vector<nixl_backend_t> &plugins) {
+    plugins = nixlPluginCache::instance().discover();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:265-290
+nixl_status_t
+nixlAgent::getPluginParams(const nixl_backend_t &type, nixl_mem_list_t &mems, nixl_b_params_t &params) const {
+    const nixlLoadedPlugin *p = nixlPluginCache::instance().load(type);
+    if (!p) {
+        NIXL_ERROR_FUNC << "plugin '" << type << "' could not be loaded";
+        return NIXL_ERR_NOT_FOUND;
+    }
+    params = p->table->get_backend_options();
+    mems = p->table->get_backend_mems();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:292-315
+nixl_status_t
+nixlAgent::getBackendParams(const nixlBackendH *backend, nixl_mem_list_t &mems, nixl_b_params_t &params) const {
+    if (!backend) return NIXL_ERR_INVALID_PARAM;
+    std::shared_lock guard(data->lock);
+    mems = backend->engine->getSupportedMems();
+    params = backend->engine->getCustomParams();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:317-426
+nixl_status_t
+nixlAgent::createBackend(const nixl_backend_t &type, const nixl_b_params_t &params, nixlBackendH *&backend) {
+    backend = nullptr;
+    std::unique_lock guard(data->lock);
+    if (data->slotOf(type)) {
+        NIXL_ERROR_FUNC << "backend already created for type '" << type << "'";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    const nixlLoadedPlugin *plugin = nixlPluginCache::instance().load(type);
+    if (!plugin) {
+        NIXL_ERROR_FUNC << "unsupported backend '" << type << "'";
+        return NIXL_ERR_NOT_FOUND;
+    }
+
+    auto slot = std::make_unique<nixlAgentData::engineSlot>();
+    slot->params = params;
+    slot->plugin = plugin;
+
+    nixlBackendInitParams init;
+    init.localAgent = data->name_;
+    init.type = type;
+    init.customParams = &slot->params;
+    init.enableProgTh = data->config_.useProgThread;
+    init.pthrDelay = data->config_.pthrDelay;
+    init.syncMode = data->config_.syncMode;
+    init.enableTelemetry_ = data->config_.captureTelemetry;
+
+    nixlBackendEngine *engine = plugin->table->create_engine(&init);
+    if (!engine) {
+        NIXL_ERROR_FUNC << "backend creation failed for '" << type << "'";
+        return NIXL_ERR_BACKEND;
+    }
+    auto drop = [&](nixl_status_t st) {
+        plugin->table->destroy_engine(engine);
+        return st;
+    };
+    if (engine->getInitErr()) {
+        NIXL_ERROR_FUNC << "backend initialization error for '" << type << "'";
+        return drop(NIXL_ERR_BACKEND);
+    }
+    if (engine->supportsRemote()) {
+        // A remote-capable backend must also carry notifications and connection info.
+        std::string conn;
+        if (!engine->supportsNotif()) return drop(NIXL_ERR_BACKEND);
+        const nixl_status_t st = engine->getConnInfo(conn);
+        if (st != NIXL_SUCCESS) return drop(st);
+    }
+    if (engine->supportsLocal()) {
+        const nixl_status_t st = engine->connect(data->name_);
+        if (st != NIXL_SUCCESS) {
+            NIXL_ERROR_FUNC << "backend '" << type << "' failed intra-agent set-up with status " << st;
+            return drop(st);
+        }
+    }
+    for (nixl_mem_t m : engine->getSupportedMems())
+        data->memToBackend[m].push_back(engine);
+
+    slot->engine = engine;
+    slot->handle = std::make_unique<nixlBackendH>(engine);
+    backend = slot->handle.get();
+    data->engines_.push_back(std::move(slot));
+    return NIXL_SUCCESS;
+}
+
+namespace {
+
+// Registers every region with one backend; all-or-nothing
+// (reference: nixlLocalSection::addDescList, src/infra/nixl_memory_section.cpp:210-286).
+nixl_status_t
+registerWithBackend(nixlAgentData &d, const nixl_reg_dlist_t &descs, nixlBackendEngine *backend) {
+    const nixl_mem_t mem = descs.getType();
+    const bool local = backend->supportsLocal();
+    std::vector<nixlSectionDesc> mine, self;
+    nixl_status_t st = NIXL_SUCCESS;
+
+    for (const nixlBlobDesc &region : descs) {
+        nixlSectionDesc entry(region.addr, region.len, region.devId, nullptr);
+        st = backend->registerMem(region, mem, entry.metadataP);
+        if (st != NIXL_SUCCESS) break;
+        nixlSectionDesc mirror = entry;
+        if (local) {
+            st = backend->loadLocalMD(entry.metadataP, mirror.metadataP);
+            if (st != NIXL_SUCCESS) {
+                backend->deregisterMem(entry.metadataP);
+                break;
+            }
+        }
+        mine.push_back(entry);
+        if (local) self.push_back(mirror);
+    }
+    if (st != NIXL_SUCCESS) {
+        for (size_t i = 0; i < mine.size(); ++i) {
+            if (local && self[i].metadataP != mine[i].metadataP) backend->unloadMD(self[i].metadataP);
+            backend->deregisterMem(mine[i].metadataP);
+        }
+        return st;
+    }
+    d.localSection_.sections[{mem, backend}].add(std::move(mine));
+    d.localSection_.memToBackend[mem].insert(backend);
+    if (local) {
+        nixlMemSection &loop = d.remoteSections_[d.name_];
+        loop.sections[{mem, backend}].add(std::move(self));
+        loop.memToBackend[mem].insert(backend);
+    }
+    return NIXL_SUCCESS;
+}
+
+// reference: nixlLocalSection::remDescList, src/infra/nixl_memory_section.cpp:288-330
+nixl_status_t
+deregisterFromBackend(nixlAgentData &d, const nixl_reg_dlist_t &descs, nixlBackendEngine *backend) {
+    const nixl_mem_t mem = descs.getType();
+    const auto sec = d.localSection_.sections.find({mem, backend});
+    if (sec == d.localSection_.sections.end()) return NIXL_ERR_NOT_FOUND;
+    nixlSecDescList &mine = sec->second;
+
+    // Nothing is deregistered unless every region is found.
+    std::vector<size_t> idx;
+    for (const nixlBlobDesc &region : descs) {
+        const int i = mine.indexOf(region);
+        if (i < 0) return NIXL_ERR_NOT_FOUND;
+        idx.push_back(static_cast<size_t>(i));
+    }
+
+    if (backend->supportsLocal()) {
+        const auto loop = d.remoteSections_.find(d.name_);
+        if (loop != d.remoteSections_.end()) {
+            const auto lsec = loop->second.sections.find({mem, backend});
+            if (lsec != loop->second.sections.end()) {
+                std::vector<size_t> lidx;
+                for (const nixlBlobDesc &region : descs) {
+                    const int i = lsec->second.indexOf(region);
+                    if (i < 0) continue;
+                    const int own = mine.indexOf(region);
+                    if (own >= 0 && lsec->second[i].metadataP != mine[own].metadataP)
+                        backend->unloadMD(lsec->second[i].metadataP);
+                    lidx.push_back(static_cast<size_t>(i));
+                }
+                lsec->second.removeAt(std::move(lidx));
+                if (lsec->second.empty()) {
+                    loop->second.sections.erase(lsec);
+                    loop->second.memToBackend[mem].erase(backend);
+                }
+            }
+        }
+    }
+    for (size_t i : idx)
+        backend->deregisterMem(mine[i].metadataP);
+    mine.removeAt(std::move(idx));
+    if (mine.empty()) {
+        d.localSection_.sections.erase(sec);
+        d.localSection_.memToBackend[mem].erase(backend);
+    }
+    return NIXL_SUCCESS;
+}
+
+void
+carryNotif(const nixl_opt_args_t *extra, nixl_opt_b_args_t &opt) {
+    if (!extra) return;
+    if (extra->notif) {
+        opt.notifMsg = *extra->notif;
+        opt.hasNotif = true;
+    } else if (extra->hasNotif) {
+        opt.notifMsg = extra->notifMsg;
+        opt.hasNotif = true;
+    }
+}
+
+} // namespace
+
+// reference: src/core/nixl_agent.cpp:441-506
+nixl_status_t
+nixlAgent::registerMem(const nixl_reg_dlist_t &descs, const nixl_opt_args_t *extra_params) {
+    std::unique_lock guard(data->lock);
+    std::vector<nixlBackendEngine *> targets;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            targets.push_back(h->engine);
+    } else {
+        if (descs.getType() < DRAM_SEG || descs.getType() > FILE_SEG) return NIXL_ERR_INVALID_PARAM;
+        targets = data->memToBackend[descs.getType()];
+        if (targets.empty()) {
+            NIXL_ERROR_FUNC << "no available backends for mem type '" << descs.getType() << "'";
+            return NIXL_ERR_NOT_FOUND;
+        }
+    }
+    // Best effort over the candidate backends: one success is enough.
+    unsigned ok = 0;
+    for (nixlBackendEngine *b : targets)
+        if (registerWithBackend(*data, descs, b) == NIXL_SUCCESS) ++ok;
+    if (ok) return NIXL_SUCCESS;
+    NIXL_ERROR_FUNC << "registration failed for the specified or all potential backends";
+    return NIXL_ERR_BACKEND;
+}
+
+// reference: src/core/nixl_agent.cpp:508-561
+nixl_status_t
+nixlAgent::deregisterMem(const nixl_reg_dlist_t &descs, const nixl_opt_args_t *extra_params) {
+    std::unique_lock guard(data->lock);
+    std::set<nixlBackendEngine *> targets;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            targets.insert(h->engine);
+    } else {
+        const auto *avail = data->localSection_.backendsFor(descs.getType());
+        if (!avail || avail->empty()) {
+            NIXL_ERROR_FUNC << "no available backends for mem type '" << descs.getType() << "'";
+            return NIXL_ERR_NOT_FOUND;
+        }
+        targets = *avail;
+    }
+    nixl_status_t bad = NIXL_SUCCESS;
+    for (nixlBackendEngine *b : targets) {
+        const nixl_status_t st = deregisterFromBackend(*data, descs, b);
+        if (st != NIXL_SUCCESS) bad = st;
+    }
+    return bad;
+}
+
+// reference: src/core/nixl_agent.cpp:428-439
+nixl_status_t
+nixlAgent::queryMem(const nixl_reg_dlist_t &descs,
+                    std::vector<nixl_query_resp_t> &resp,
+                    const nixl_opt_args_t *extra_params) const {
+    if (!extra_params || extra_params->backends.size() != 1) return NIXL_ERR_INVALID_PARAM;
+    return extra_params->backends[0]->engine->queryMem(descs, resp);
+}
+
+// reference: src/core/nixl_agent.cpp:563-618 (only the agent itself is a known peer here)
+nixl_status_t
+nixlAgent::makeConnection(const std::string &remote_agent, const nixl_opt_args_t *) {
+    std::unique_lock guard(data->lock);
+    if (remote_agent != data->name_) return NIXL_ERR_NOT_FOUND;
+    nixl_status_t st = NIXL_ERR_BACKEND;
+    for (const auto &s : data->engines_) {
+        if (!s->engine->supportsLocal()) continue;
+        st = s->engine->connect(remote_agent);
+        if (st != NIXL_SUCCESS) return st;
+    }
+    return st;
+}
+
+// reference: src/core/nixl_agent.cpp:620-687
+nixl_status_t
+nixlAgent::prepXferDlist(const std::string &agent_name,
+                         const nixl_xfer_dlist_t &descs,
+                         nixlDlistH *&dlist_hndl,
+                         const nixl_opt_args_t *extra_params) const {
+    dlist_hndl = nullptr;
+    const bool init_side = (agent_name == NIXL_INIT_AGENT);
+    std::shared_lock guard(data->lock);
+
+    const nixlMemSection *section = &data->localSection_;
+    if (!init_side) {
+        const auto it = data->remoteSections_.find(agent_name);
+        if (it == data->remoteSections_.end()) {
+            NIXL_ERROR_FUNC << "metadata for remote agent '" << agent_name << "' not found";
+            return NIXL_ERR_NOT_FOUND;
+        }
+        section = &it->second;
+    }
+
+    std::set<nixlBackendEngine *> candidates;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            candidates.insert(h->engine);
+    } else {
+        const auto *avail = section->backendsFor(descs.getType());
+        if (!avail || avail->empty()) {
+            NIXL_ERROR_FUNC << "no available backends for mem type '" << descs.getType() << "'";
+            return NIXL_ERR_NOT_FOUND;
+        }
+        candidates = *avail;
+    }
+
+    nixlDlistH::descs_t prepared;
+    for (nixlBackendEngine *b : candidates) {
+        nixl_stride_dlist_t runs(descs.getType());
+        if (section->populate(descs, b, runs) == NIXL_SUCCESS) {
+            NIXL_DEBUG << "backend " << b->getType() << ": prepared " << descs.descCount()
+                       << " descriptors into " << runs.descCount() << " strides";
+            prepared.try_emplace(b, std::make_unique<nixl_stride_dlist_t>(std::move(runs)));
+        }
+    }
+    if (prepared.empty()) {
+        NIXL_ERROR_FUNC << "failed to prepare the descriptors for any backend for agent '" << agent_name << "'";
+        return NIXL_ERR_NOT_FOUND;
+    }
+    dlist_hndl = new nixlDlistH(agent_name, std::move(prepared));
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlAgent::prepXferDlist(const nixl_xfer_dlist_t &descs,
+                         nixlDlistH *&dlist_hndl,
+                         const nixl_opt_args_t *extra_params) const {
+    return prepXferDlist(NIXL_INIT_AGENT, descs, dlist_hndl, extra_params);
+}
+
+// reference: src/core/nixl_agent.cpp:696-887
+nixl_status_t
+nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
+                       const nixlDlistH *local_side,
+                       const std::vector<int> &local_indices,
+                       const nixlDlistH *remote_side,
+                       const std::vector<int> &remote_indices,
+                       nixlXferReqH *&req_hndl,
+                       const nixl_opt_args_t *extra_params) const {
+    req_hndl = nullptr;
+    if (!local_side || !remote_side) {
+        NIXL_ERROR_FUNC << "local or remote side handle is null";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    if (!local_side->remoteAgent.empty() || remote_side->remoteAgent.empty()) {
+        NIXL_ERROR_FUNC << "invalid sides (local must be local, remote must be remote)";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    const size_t count = local_indices.size();
+    if (count == 0 || count != remote_indices.size()) {
+        NIXL_ERROR_FUNC << "different number of indices for local (" << count << "), remote ("
+                        << remote_indices.size() << ")";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    // First backend that prepared both sides, in the caller's order if one was given.
+    nixlBackendEngine *backend = nullptr;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            if (local_side->descs.count(h->engine) && remote_side->descs.count(h->engine)) {
+                backend = h->engine;
+                break;
+            }
+    } else {
+        for (const auto &kv : local_side->descs)
+            if (remote_side->descs.count(kv.first)) {
+                backend = kv.first;
+                break;
+            }
+    }
+    if (!backend) {
+        NIXL_ERROR_FUNC << "could not find a common backend for the prepped Dlists";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    nixl_opt_b_args_t opt;
+    carryNotif(extra_params, opt);
+    if (opt.hasNotif && !backend->supportsNotif()) {
+        NIXL_ERROR_FUNC << "the selected backend '" << backend->getType() << "' does not support notifications";
+        return NIXL_ERR_BACKEND;
+    }
+
+    std::shared_lock guard(data->lock);
+    if (!data->remoteSections_.count(remote_side->remoteAgent)) return NIXL_ERR_NOT_FOUND;
+
+    const nixl_stride_dlist_t &lruns = *local_side->descs.at(backend);
+    const nixl_stride_dlist_t &rruns = *remote_side->descs.at(backend);
+    auto req = std::make_unique<nixlXferReqH>(remote_side->remoteAgent, operation, lruns.getType(), rruns.getType());
+    req->initiatorDescs.reserve(count);
+    req->targetDescs.reserve(count);
+
+    const bool no_merge = extra_params && extra_params->skipDescMerge;
+    const size_t lflat = lruns.flatSize(), rflat = rruns.flatSize();
+    // Ceiling division keeps find()'s first probe inside the run array.
+    const size_t lguess = (lflat + lruns.descCount() - 1) / lruns.descCount();
+    const size_t rguess = (rflat + rruns.descCount() - 1) / rruns.descCount();
+
+    size_t total = 0;
+    for (size_t i = 0, step = 1; i < count; i += step) {
+        if (local_indices[i] < 0 || static_cast<size_t>(local_indices[i]) >= lflat) {
+            NIXL_ERROR_FUNC << "local index out of range at index " << i << " with value " << local_indices[i];
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        if (remote_indices[i] < 0 || static_cast<size_t>(remote_indices[i]) >= rflat) {
+            NIXL_ERROR_FUNC << "remote index out of range at index " << i << " with value " << remote_indices[i];
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        const size_t li = static_cast<size_t>(local_indices[i]);
+        const size_t ri = static_cast<size_t>(remote_indices[i]);
+        const nixlStrideDesc lrun = lruns.find(li, lguess);
+        const nixlStrideDesc rrun = rruns.find(ri, rguess);
+        if (lrun.len != rrun.len) {
+            NIXL_ERROR_FUNC << "length mismatch at index " << i << " with local index " << li
+                            << " and remote index " << ri;
+            return NIXL_ERR_INVALID_PARAM;
+        }
+
+        // Consecutive indices collapse into one descriptor only when the local run is
+        // dense (stride == len), the remote run has the same stride, both index
+        // sequences advance by one, and neither run ends.
+        step = 1;
+        if (!no_merge && lrun.stride == lrun.len && lrun.stride == rrun.stride) {
+            const size_t room = std::min({lrun.start_idx + lrun.count - li, rrun.start_idx + rrun.count - ri, count - i});
+            while (step < room && static_cast<size_t>(local_indices[i + step]) == li + step &&
+                   static_cast<size_t>(remote_indices[i + step]) == ri + step)
+                ++step;
+        }
+        const nixlMetaDesc &ld = req->initiatorDescs.emplace(lrun.getMetaDesc(li, step));
+        req->targetDescs.emplace(rrun.getMetaDesc(ri, step));
+        total += ld.len;
+    }
+    NIXL_DEBUG << "merged " << count << " indices into " << req->initiatorDescs.descCount() << " descriptors";
+
+    req->engine = backend;
+    req->notifMsg = opt.notifMsg;
+    req->hasNotif = opt.hasNotif;
+    req->telemetry.totalBytes = total;
+    req->telemetry.descCount = static_cast<size_t>(req->initiatorDescs.descCount());
+
+    const nixl_status_t st = backend->prepXfer(req->backendOp, req->initiatorDescs, req->targetDescs,
+                                               req->remoteAgent, req->backendHandle, &opt);
+    if (st != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "backend '" << backend->getType() << "' failed to prepare the transfer request with status " << st;
+        return st;
+    }
+    req_hndl = req.release();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:889-1032 (one descriptor per list entry, no merging)
+nixl_status_t
+nixlAgent::createXferReq(const nixl_xfer_op_t &operation,
+                         const nixl_xfer_dlist_t &local_descs,
+                         const nixl_xfer_dlist_t &remote_descs,
+                         const std::string &remote_agent,
+                         nixlXferReqH *&req_hndl,
+                         const nixl_opt_args_t *extra_params) const {
+    req_hndl = nullptr;
+    if (local_descs.descCount() != remote_descs.descCount()) {
+        NIXL_ERROR_FUNC << "different descriptor list sizes (local=" << local_descs.descCount()
+                        << ", remote=" << remote_descs.descCount() << ")";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    size_t total = 0;
+    for (int i = 0; i < local_descs.descCount(); ++i) {
+        if (local_descs[i].len != remote_descs[i].len) {
+            NIXL_ERROR_FUNC << "length mismatch at index " << i;
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        total += local_descs[i].len;
+    }
+
+    std::shared_lock guard(data->lock);
+    const auto rem = data->remoteSections_.find(remote_agent);
+    if (rem == data->remoteSections_.end()) {
+        NIXL_ERROR_FUNC << "metadata for remote agent '" << remote_agent << "' not found";
+        return NIXL_ERR_NOT_FOUND;
+    }
+
+    std::vector<nixlBackendEngine *> candidates;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            candidates.push_back(h->engine);
+    } else {
+        const auto *lset = data->localSection_.backendsFor(local_descs.getType());
+        const auto *rset = rem->second.backendsFor(remote_descs.getType());
+        if (!lset || !rset) return NIXL_ERR_NOT_FOUND;
+        for (nixlBackendEngine *b : *lset)
+            if (rset->count(b)) candidates.push_back(b);
+        if (candidates.empty()) {
+            NIXL_ERROR_FUNC << "no potential backend found to be able to do the transfer";
+            return NIXL_ERR_NOT_FOUND;
+        }
+    }
+
+    auto req = std::make_unique<nixlXferReqH>(remote_agent, operation, local_descs.getType(), remote_descs.getType());
+    for (nixlBackendEngine *b : candidates) {
+        const nixl_status_t s1 = data->localSection_.populate(local_descs, b, req->initiatorDescs);
+        const nixl_status_t s2 = rem->second.populate(remote_descs, b, req->targetDescs);
+        if (s1 == NIXL_SUCCESS && s2 == NIXL_SUCCESS) {
+            req->engine = b;
+            break;
+        }
+    }
+    if (!req->engine) {
+        NIXL_ERROR_FUNC << "no specified or potential backend had the required registrations";
+        return NIXL_ERR_NOT_FOUND;
+    }
+
+    nixl_opt_b_args_t opt;
+    carryNotif(extra_params, opt);
+    if (extra_params && !extra_params->customParam.empty()) opt.customParam = extra_params->customParam;
+    if (opt.hasNotif && !req->engine->supportsNotif()) {
+        NIXL_ERROR_FUNC << "the selected backend '" << req->engine->getType() << "' does not support notifications";
+        return NIXL_ERR_BACKEND;
+    }
+    req->notifMsg = opt.notifMsg;
+    req->hasNotif = opt.hasNotif;
+    req->telemetry.totalBytes = total;
+    req->telemetry.descCount = static_cast<size_t>(req->initiatorDescs.descCount());
+
+    const nixl_status_t st = req->engine->prepXfer(req->backendOp, req->initiatorDescs, req->targetDescs,
+                                                   req->remoteAgent, req->backendHandle, &opt);
+    if (st != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "backend '" << req->engine->getType() << "' failed to prepare the transfer request with status " << st;
+        return st;
+    }
+    req_hndl = req.release();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:1034-1077
+nixl_status_t
+nixlAgent::estimateXferCost(const nixlXferReqH *req_hndl,
+                            std::chrono::microseconds &duration,
+                            std::chrono::microseconds &err_margin,
+                            nixl_cost_t &method,
+                            const nixl_opt_args_t *extra_params) const {
+    if (!req_hndl || !req_hndl->engine) return NIXL_ERR_UNKNOWN;
+    std::shared_lock guard(data->lock);
+    return req_hndl->engine->estimateXferCost(req_hndl->backendOp, req_hndl->initiatorDescs, req_hndl->targetDescs,
+                                              req_hndl->remoteAgent, req_hndl->backendHandle, duration, err_margin,
+                                              method, extra_params);
+}
+
+// reference: src/core/nixl_agent.cpp:1079-1214
+nixl_status_t
+nixlAgent::postXferReq(nixlXferReqH *req_hndl, const nixl_opt_args_t *extra_params) const {
+    if (!req_hndl) {
+        NIXL_ERROR_FUNC << "transfer request handle is null";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    req_hndl->telemetry.startTime = std::chrono::steady_clock::now();
+
+    std::shared_lock guard(data->lock);
+    if (!data->remoteSections_.count(req_hndl->remoteAgent)) return NIXL_ERR_NOT_FOUND;
+
+    // A request that is still running cannot be posted again.
+    if (req_hndl->status == NIXL_IN_PROG) {
+        req_hndl->status = req_hndl->engine->checkXfer(req_hndl->backendHandle);
+        if (req_hndl->status == NIXL_IN_PROG) {
+            NIXL_ERROR_FUNC << "transfer request is still in progress and cannot be reposted";
+            return NIXL_ERR_REPOST_ACTIVE;
+        }
+    }
+
+    nixl_opt_b_args_t opt;
+    if (req_hndl->hasNotif) {
+        opt.notifMsg = req_hndl->notifMsg;
+        opt.hasNotif = true;
+    }
+    if (extra_params) {
+        nixl_opt_b_args_t fresh;
+        carryNotif(extra_params, fresh);
+        req_hndl->hasNotif = opt.hasNotif = fresh.hasNotif;
+        if (fresh.hasNotif) req_hndl->notifMsg = opt.notifMsg = fresh.notifMsg;
+    }
+    if (opt.hasNotif && !req_hndl->engine->supportsNotif()) {
+        NIXL_ERROR_FUNC << "the selected backend '" << req_hndl->engine->getType() << "' does not support notifications";
+        return NIXL_ERR_BACKEND;
+    }
+
+    req_hndl->status = req_hndl->engine->postXfer(req_hndl->backendOp, req_hndl->initiatorDescs, req_hndl->targetDescs,
+                                                  req_hndl->remoteAgent, req_hndl->backendHandle, &opt);
+    req_hndl->postEnd = std::chrono::steady_clock::now();
+    req_hndl->telemetry.postDuration =
+        std::chrono::duration_cast<chrono_period_us_t>(req_hndl->postEnd - req_hndl->telemetry.startTime);
+    if (req_hndl->status == NIXL_SUCCESS) req_hndl->telemetry.xferDuration = req_hndl->telemetry.postDuration;
+    if (req_hndl->status < 0)
+        NIXL_ERROR_FUNC << "backend '" << req_hndl->engine->getType() << "' failed to post the transfer request with status "
+                        << req_hndl->status;
+    return req_hndl->status;
+}
+
+// reference: src/core/nixl_agent.cpp:1216-1260
+nixl_status_t
+nixlAgent::getXferStatus(nixlXferReqH *req_hndl) const {
+    if (!req_hndl) return NIXL_ERR_INVALID_PARAM;
+    std::shared_lock guard(data->lock);
+    // Only an in-flight request is re-checked; done or failed requests keep their status.
+    if (req_hndl->status == NIXL_IN_PROG) {
+        if (!data->remoteSections_.count(req_hndl->remoteAgent)) return NIXL_ERR_NOT_FOUND;
+        req_hndl->status = req_hndl->engine->checkXfer(req_hndl->backendHandle);
+        if (req_hndl->status == NIXL_SUCCESS)
+            req_hndl->telemetry.xferDuration = std::chrono::duration_cast<chrono_period_us_t>(
+                std::chrono::steady_clock::now() - req_hndl->telemetry.startTime);
+        else if (req_hndl->status < 0)
+            NIXL_ERROR_FUNC << "backend '" << req_hndl->engine->getType() << "' returned error status " << req_hndl->status;
+    }
+    return req_hndl->status;
+}
+
+// reference: src/core/nixl_agent.cpp:1262-1276
+nixl_status_t
+nixlAgent::getXferTelemetry(const nixlXferReqH *req_hndl, nixl_xfer_telem_t &telemetry) const {
+    if (!data->config_.captureTelemetry) {
+        NIXL_ERROR_FUNC << "cannot return values when telemetry is not enabled.";
+        return NIXL_ERR_NO_TELEMETRY;
+    }
+    if (req_hndl->status != NIXL_SUCCESS) return req_hndl->status;
+    telemetry = req_hndl->telemetry;
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:1278-1284
+nixl_status_t
+nixlAgent::queryXferBackend(const nixlXferReqH *req_hndl, nixlBackendH *&backend) const {
+    std::shared_lock guard(data->lock);
+    nixlAgentData::engineSlot *slot = data->slotOf(req_hndl->engine->getType());
+    backend = slot ? slot->handle.get() : nullptr;
+    return slot ? NIXL_SUCCESS : NIXL_ERR_NOT_FOUND;
+}
+
+// reference: src/core/nixl_agent.cpp:1286-1313
+nixl_status_t
+nixlAgent::releaseXferReq(nixlXferReqH *req_hndl) const {
+    if (!req_hndl) return NIXL_ERR_INVALID_PARAM;
+    std::shared_lock guard(data->lock);
+    if (req_hndl->status == NIXL_IN_PROG) {
+        req_hndl->status = req_hndl->engine->checkXfer(req_hndl->backendHandle);
+        if (req_hndl->status == NIXL_IN_PROG) {
+            // Ask the backend to abort; a backend that cannot must say so.
+            req_hndl->status = req_hndl->engine->releaseReqH(req_hndl->backendHandle);
+            if (req_hndl->status < 0) {
+                NIXL_ERROR_FUNC << "backend '" << req_hndl->engine->getType() << "' could not release an active request";
+                return NIXL_ERR_REPOST_ACTIVE;
+            }
+            req_hndl->backendHandle = nullptr;
+        }
+    }
+    delete req_hndl;
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:1315-1320
+nixl_status_t
+nixlAgent::releasedDlistH(nixlDlistH *dlist_hndl) const {
+    std::unique_lock guard(data->lock);
+    delete dlist_hndl;
+    return NIXL_SUCCESS;
+}
+
+// ---- outside the transfer path -----------------------------------------------------------
+
+nixl_status_t
+nixlAgent::prepMemView(const nixl_remote_dlist_t &, nixlMemViewH &, const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::prepMemView(const nixl_local_dlist_t &, nixlMemViewH &, const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+void
+nixlAgent::releaseMemView(nixlMemViewH) const {}
+
+nixl_status_t
+nixlAgent::getNotifs(nixl_notifs_t &, const nixl_opt_args_t *) {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::genNotif(const std::string &, const nixl_blob_t &, const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::getLocalMD(nixl_blob_t &) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::loadRemoteMD(const nixl_blob_t &, std::string &) {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::invalidateRemoteMD(const std::string &) {
+    return NIXL_ERR_NOT_SUPPORTED;
+}

@@ -1,0 +1,446 @@
+// extern "C" façade over nixlAgent (declared in include/nixl_amd_capi.h).
+#include "nixl_amd_capi.h"
+
+#include <exception>
+#include <thread>
+
+#include "agent_impl.h"
+
+struct nixl_capi_agent_s {
+    nixlAgent *inner;
+};
+struct nixl_capi_params_s {
+    nixl_b_params_t params;
+};
+struct nixl_capi_backend_s {
+    nixlBackendH *backend;
+};
+struct nixl_capi_opt_args_s {
+    nixl_opt_args_t args;
+};
+struct nixl_capi_xfer_dlist_s {
+    nixl_xfer_dlist_t *dlist;
+};
+struct nixl_capi_xfer_dlist_handle_s {
+    nixlDlistH *handle;
+};
+struct nixl_capi_reg_dlist_s {
+    nixl_reg_dlist_t *dlist;
+};
+struct nixl_capi_xfer_req_s {
+    nixlXferReqH *req;
+};
+
+namespace {
+
+thread_local int g_last_status = NIXL_SUCCESS;
+
+// Same folding as the reference wrapper: success, in-progress, not-found and
+// no-telemetry survive; every other error becomes "backend".
+nixl_capi_status_t
+fold(nixl_status_t st) {
+    g_last_status = st;
+    switch (st) {
+    case NIXL_SUCCESS: return NIXL_CAPI_SUCCESS;
+    case NIXL_IN_PROG: return NIXL_CAPI_IN_PROG;
+    case NIXL_ERR_NOT_FOUND: return NIXL_CAPI_ERROR_NOT_FOUND;
+    case NIXL_ERR_NO_TELEMETRY: return NIXL_CAPI_ERROR_NO_TELEMETRY;
+    default: return NIXL_CAPI_ERROR_BACKEND;
+    }
+}
+
+template<typename F>
+nixl_capi_status_t
+guarded(F &&f) {
+    try {
+        return f();
+    }
+    catch (const std::exception &e) {
+        std::cerr << "nixl_capi: exception: " << e.what() << std::endl;
+        return NIXL_CAPI_ERROR_EXCEPTION;
+    }
+    catch (...) {
+        return NIXL_CAPI_ERROR_EXCEPTION;
+    }
+}
+
+nixl_mem_t
+memOf(nixl_capi_mem_type_t t) {
+    return static_cast<nixl_mem_t>(t);
+}
+
+} // namespace
+
+extern "C" {
+
+int
+nixl_capi_last_nixl_status(void) {
+    return g_last_status;
+}
+
+nixl_capi_status_t
+nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent) {
+    if (!name || !agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlAgentConfig cfg(true);
+        *agent = new nixl_capi_agent_s{new nixlAgent(name, cfg)};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_create_configured_agent(const char *name, const nixl_capi_agent_config_t *cfg, nixl_capi_agent_t *agent) {
+    if (!name || !cfg || !agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlAgentConfig c(cfg->enable_prog_thread,
+                          cfg->enable_listen_thread,
+                          static_cast<uint16_t>(cfg->listen_port),
+                          static_cast<nixl_thread_sync_t>(cfg->thread_sync),
+                          cfg->num_workers,
+                          cfg->pthr_delay_us,
+                          cfg->lthr_delay_us,
+                          cfg->capture_telemetry);
+        *agent = new nixl_capi_agent_s{new nixlAgent(name, c)};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_agent(nixl_capi_agent_t agent) {
+    if (!agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        delete agent->inner;
+        delete agent;
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_create_params(nixl_capi_params_t *params) {
+    if (!params) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *params = new nixl_capi_params_s{};
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_params_add(nixl_capi_params_t params, const char *key, const char *value) {
+    if (!params || !key || !value) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    params->params[key] = value;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_params(nixl_capi_params_t params) {
+    if (!params) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete params;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_create_backend(nixl_capi_agent_t agent, const char *plugin_name, nixl_capi_params_t params, nixl_capi_backend_t *backend) {
+    if (!agent || !plugin_name || !backend) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        static const nixl_b_params_t none;
+        nixlBackendH *h = nullptr;
+        const nixl_status_t st = agent->inner->createBackend(plugin_name, params ? params->params : none, h);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *backend = new nixl_capi_backend_s{h};
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_backend(nixl_capi_backend_t backend) {
+    if (!backend) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete backend; // the engine itself belongs to the agent
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_create_opt_args(nixl_capi_opt_args_t *args) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *args = new nixl_capi_opt_args_s{};
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_opt_args(nixl_capi_opt_args_t args) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete args;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_add_backend(nixl_capi_opt_args_t args, nixl_capi_backend_t backend) {
+    if (!args || !backend) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.backends.push_back(backend->backend);
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_notif_msg(nixl_capi_opt_args_t args, const void *data, size_t len) {
+    if (!args || (!data && len)) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.notifMsg.assign(static_cast<const char *>(data), len);
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_has_notif(nixl_capi_opt_args_t args, bool has_notif) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.hasNotif = has_notif;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_skip_desc_merge(nixl_capi_opt_args_t args, bool skip_merge) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.skipDescMerge = skip_merge;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_create_xfer_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_xfer_dlist_t *dlist) {
+    if (!dlist || mem_type >= NIXL_CAPI_MEM_UNKNOWN) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *dlist = new nixl_capi_xfer_dlist_s{new nixl_xfer_dlist_t(memOf(mem_type))};
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_xfer_dlist(nixl_capi_xfer_dlist_t dlist) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete dlist->dlist;
+    delete dlist;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_add_desc(nixl_capi_xfer_dlist_t dlist, uintptr_t addr, size_t len, uint64_t dev_id) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    dlist->dlist->addDesc(nixlBasicDesc(addr, len, dev_id));
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_add_descs(nixl_capi_xfer_dlist_t dlist,
+                               const uint64_t *addrs,
+                               const uint64_t *lens,
+                               const uint64_t *dev_ids,
+                               size_t n) {
+    if (!dlist || (n && (!addrs || !lens))) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    dlist->dlist->reserve(static_cast<size_t>(dlist->dlist->descCount()) + n);
+    for (size_t i = 0; i < n; ++i)
+        dlist->dlist->emplace(static_cast<uintptr_t>(addrs[i]), static_cast<size_t>(lens[i]),
+                              dev_ids ? dev_ids[i] : uint64_t{0});
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_desc_count(nixl_capi_xfer_dlist_t dlist, size_t *count) {
+    if (!dlist || !count) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *count = static_cast<size_t>(dlist->dlist->descCount());
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_clear(nixl_capi_xfer_dlist_t dlist) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    dlist->dlist->clear();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_create_reg_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_reg_dlist_t *dlist) {
+    if (!dlist || mem_type >= NIXL_CAPI_MEM_UNKNOWN) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *dlist = new nixl_capi_reg_dlist_s{new nixl_reg_dlist_t(memOf(mem_type))};
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_reg_dlist(nixl_capi_reg_dlist_t dlist) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete dlist->dlist;
+    delete dlist;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_add_desc(nixl_capi_reg_dlist_t dlist, uintptr_t addr, size_t len, uint64_t dev_id, const void *metadata, size_t metadata_len) {
+    if (!dlist || (!metadata && metadata_len)) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    nixl_blob_t meta;
+    if (metadata_len) meta.assign(static_cast<const char *>(metadata), metadata_len);
+    dlist->dlist->addDesc(nixlBlobDesc(addr, len, dev_id, meta));
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_desc_count(nixl_capi_reg_dlist_t dlist, size_t *count) {
+    if (!dlist || !count) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *count = static_cast<size_t>(dlist->dlist->descCount());
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_register_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t dlist, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->registerMem(*dlist->dlist, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_deregister_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t dlist, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->deregisterMem(*dlist->dlist, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_prep_xfer_dlist(nixl_capi_agent_t agent, const char *agent_name, nixl_capi_xfer_dlist_t descs, nixl_capi_xfer_dlist_handle_t *dlist_hndl, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !agent_name || !descs || !dlist_hndl) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlDlistH *h = nullptr;
+        const nixl_status_t st = agent->inner->prepXferDlist(agent_name, *descs->dlist, h, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *dlist_hndl = new nixl_capi_xfer_dlist_handle_s{h};
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_release_xfer_dlist_handle(nixl_capi_agent_t agent, nixl_capi_xfer_dlist_handle_t dlist_handle) {
+    if (!agent || !dlist_handle) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        const nixl_status_t st = agent->inner->releasedDlistH(dlist_handle->handle);
+        delete dlist_handle;
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_handle_run_count(nixl_capi_xfer_dlist_handle_t h, size_t *runs) {
+    if (!h || !h->handle || !runs || h->handle->descs.empty()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *runs = static_cast<size_t>(h->handle->descs.begin()->second->descCount());
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_make_xfer_req(nixl_capi_agent_t agent,
+                        nixl_capi_xfer_op_t operation,
+                        nixl_capi_xfer_dlist_handle_t local_descs,
+                        const int *local_indices,
+                        size_t local_indices_count,
+                        nixl_capi_xfer_dlist_handle_t remote_descs,
+                        const int *remote_indices,
+                        size_t remote_indices_count,
+                        nixl_capi_xfer_req_t *req_hndl,
+                        nixl_capi_opt_args_t opt_args) {
+    if (!agent || !local_descs || !remote_descs || !req_hndl || (!local_indices && local_indices_count) ||
+        (!remote_indices && remote_indices_count))
+        return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        const std::vector<int> li(local_indices, local_indices + local_indices_count);
+        const std::vector<int> ri(remote_indices, remote_indices + remote_indices_count);
+        nixlXferReqH *req = nullptr;
+        const nixl_status_t st = agent->inner->makeXferReq(static_cast<nixl_xfer_op_t>(operation), local_descs->handle, li,
+                                                          remote_descs->handle, ri, req, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *req_hndl = new nixl_capi_xfer_req_s{req};
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_create_xfer_req(nixl_capi_agent_t agent,
+                          nixl_capi_xfer_op_t operation,
+                          nixl_capi_xfer_dlist_t local_descs,
+                          nixl_capi_xfer_dlist_t remote_descs,
+                          const char *remote_agent,
+                          nixl_capi_xfer_req_t *req_hndl,
+                          nixl_capi_opt_args_t opt_args) {
+    if (!agent || !local_descs || !remote_descs || !remote_agent || !req_hndl) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlXferReqH *req = nullptr;
+        const nixl_status_t st = agent->inner->createXferReq(static_cast<nixl_xfer_op_t>(operation), *local_descs->dlist,
+                                                            *remote_descs->dlist, remote_agent, req,
+                                                            opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *req_hndl = new nixl_capi_xfer_req_s{req};
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_post_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !req_hndl) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->postXferReq(req_hndl->req, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_get_xfer_status(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl) {
+    if (!agent || !req_hndl) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->getXferStatus(req_hndl->req)); });
+}
+
+nixl_capi_status_t
+nixl_capi_post_and_wait(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl) {
+    if (!agent || !req_hndl) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_status_t st = agent->inner->postXferReq(req_hndl->req, nullptr);
+        while (st == NIXL_IN_PROG) {
+            std::this_thread::yield();
+            st = agent->inner->getXferStatus(req_hndl->req);
+        }
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_get_xfer_telemetry(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_xfer_telemetry_t telemetry) {
+    if (!agent || !req_hndl || !telemetry) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_xfer_telem_t t{};
+        const nixl_status_t st = agent->inner->getXferTelemetry(req_hndl->req, t);
+        if (st != NIXL_SUCCESS) return fold(st);
+        telemetry->start_time_us = static_cast<uint64_t>(
+            std::chrono::duration_cast<std::chrono::microseconds>(t.startTime.time_since_epoch()).count());
+        telemetry->post_duration_us = static_cast<uint64_t>(t.postDuration.count());
+        telemetry->xfer_duration_us = static_cast<uint64_t>(t.xferDuration.count());
+        telemetry->total_bytes = t.totalBytes;
+        telemetry->desc_count = t.descCount;
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_req_desc_count(nixl_capi_xfer_req_t req, size_t *count, size_t *bytes) {
+    if (!req || !req->req) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    if (count) *count = req->req->telemetry.descCount;
+    if (bytes) *bytes = req->req->telemetry.totalBytes;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_req_get_desc(nixl_capi_xfer_req_t req, size_t i, uint64_t *local_addr, uint64_t *remote_addr, uint64_t *len) {
+    if (!req || !req->req || i >= static_cast<size_t>(req->req->initiatorDescs.descCount()))
+        return NIXL_CAPI_ERROR_INVALID_PARAM;
+    if (local_addr) *local_addr = req->req->initiatorDescs[i].addr;
+    if (remote_addr) *remote_addr = req->req->targetDescs[i].addr;
+    if (len) *len = req->req->initiatorDescs[i].len;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_release_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req) {
+    if (!agent || !req) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        const nixl_status_t st = agent->inner->releaseXferReq(req->req);
+        if (st == NIXL_SUCCESS) req->req = nullptr;
+        return fold(st);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_xfer_req(nixl_capi_xfer_req_t req) {
+    if (!req) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete req; // the inner request was handed back by nixl_capi_release_xfer_req
+    return NIXL_CAPI_SUCCESS;
+}
+
+} // extern "C"

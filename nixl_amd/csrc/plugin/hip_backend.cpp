@@ -1,0 +1,333 @@
+#include "hip_backend.h"
+
+#include <cstdlib>
+
+#include "backend/backend_plugin.h"
+#include "common/nixl_log.h"
+
+namespace {
+
+int
+paramInt(const nixl_b_params_t *params, const char *key, int fallback) {
+    if (!params) return fallback;
+    const auto it = params->find(key);
+    if (it == params->end()) return fallback;
+    char *end = nullptr;
+    const long v = std::strtol(it->second.c_str(), &end, 10);
+    if (end == it->second.c_str() || *end != '\0')
+        throw std::runtime_error(std::string("HIP backend: parameter '") + key +
+                                 "' is not an integer: " + it->second);
+    return static_cast<int>(v);
+}
+
+bool
+hipOk(hipError_t e, const char *what) {
+    if (e == hipSuccess) return true;
+    NIXL_ERROR << "HIP backend: " << what << " failed: " << hipGetErrorString(e);
+    return false;
+}
+
+} // namespace
+
+nixlHipReqH::~nixlHipReqH() {
+    (void)hipSetDevice(device);
+    if (plan) (void)nixl_amd_copy_plan_destroy(plan);
+    if (done) (void)hipEventDestroy(done);
+}
+
+nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
+    : nixlBackendEngine(init_params) {
+    const nixl_b_params_t *p = init_params->customParams;
+    tuning_.units_per_lane = paramInt(p, "units_per_lane", 0);
+    tuning_.nontemporal = paramInt(p, "nontemporal", 0);
+    tuning_.max_workgroups = paramInt(p, "max_workgroups", 0);
+    streamsPerDevice_ = paramInt(p, "num_streams", 1);
+    if (streamsPerDevice_ < 1 || streamsPerDevice_ > 16)
+        throw std::runtime_error("HIP backend: num_streams must be in [1, 16]");
+
+    const int n = nixl_amd_device_count();
+    if (n <= 0) {
+        NIXL_ERROR << "HIP backend: no HIP device visible (" << nixl_amd_last_error() << ")";
+        initErr = true;
+        return;
+    }
+    numDevices_ = n;
+    streams_.assign(static_cast<size_t>(n) * streamsPerDevice_, nullptr);
+}
+
+nixlHipEngine::~nixlHipEngine() {
+    reapRetired(true);
+    for (size_t i = 0; i < streams_.size(); ++i) {
+        if (!streams_[i]) continue;
+        (void)hipSetDevice(static_cast<int>(i / streamsPerDevice_));
+        (void)hipStreamSynchronize(streams_[i]);
+        (void)hipStreamDestroy(streams_[i]);
+    }
+}
+
+hipStream_t
+nixlHipEngine::pickStream(int device) const {
+    const unsigned slot = nextStream_.fetch_add(1, std::memory_order_relaxed) % streamsPerDevice_;
+    const size_t idx = static_cast<size_t>(device) * streamsPerDevice_ + slot;
+    std::lock_guard<std::mutex> lock(streamsMutex_);
+    if (!streams_[idx]) {
+        // Default priority on purpose; non-blocking so that the legacy default stream
+        // of the host application does not serialise against transfers.
+        if (!hipOk(hipStreamCreateWithFlags(&streams_[idx], hipStreamNonBlocking), "hipStreamCreateWithFlags"))
+            streams_[idx] = nullptr;
+    }
+    return streams_[idx];
+}
+
+void
+nixlHipEngine::reapRetired(bool wait) const {
+    std::lock_guard<std::mutex> lock(retiredMutex_);
+    size_t keep = 0;
+    for (nixlHipReqH *r : retired_) {
+        (void)hipSetDevice(r->device);
+        bool finished = true;
+        if (r->posted) {
+            if (wait)
+                (void)hipEventSynchronize(r->done);
+            else
+                finished = (hipEventQuery(r->done) != hipErrorNotReady);
+        }
+        if (finished)
+            delete r;
+        else
+            retired_[keep++] = r;
+    }
+    retired_.resize(keep);
+}
+
+nixl_status_t
+nixlHipEngine::registerMem(const nixlBlobDesc &mem, const nixl_mem_t &nixl_mem, nixlBackendMD *&out) {
+    out = nullptr;
+    if (nixl_mem != VRAM_SEG && nixl_mem != DRAM_SEG) return NIXL_ERR_NOT_SUPPORTED;
+    if (mem.len == 0 || mem.addr == 0) return NIXL_ERR_INVALID_PARAM;
+
+    hipPointerAttribute_t attr{};
+    const void *ptr = reinterpret_cast<const void *>(mem.addr);
+    if (hipPointerGetAttributes(&attr, ptr) != hipSuccess) {
+        (void)hipGetLastError(); // clear the sticky error left by the failed query
+        NIXL_ERROR << "HIP backend: address " << mem.addr << " is not known to the HIP runtime";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    int device = 0;
+    if (nixl_mem == VRAM_SEG) {
+        if (attr.type != hipMemoryTypeDevice) {
+            NIXL_ERROR << "HIP backend: VRAM_SEG registration of non-device memory";
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        if (static_cast<uint64_t>(attr.device) != mem.devId) {
+            NIXL_ERROR << "HIP backend: region lives on device " << attr.device << ", descriptor says "
+                       << mem.devId;
+            return NIXL_ERR_MISMATCH;
+        }
+        device = attr.device;
+    } else {
+        // Host memory is usable only if the runtime allocated it pinned (device-mapped);
+        // pageable or merely registered host memory is refused rather than staged.
+        if (attr.type != hipMemoryTypeHost) {
+            NIXL_ERROR << "HIP backend: DRAM_SEG registration requires hipHostMalloc memory";
+            return NIXL_ERR_NOT_SUPPORTED;
+        }
+        if (hipGetDevice(&device) != hipSuccess) return NIXL_ERR_BACKEND;
+    }
+    if (device < 0 || device >= numDevices_) return NIXL_ERR_INVALID_PARAM;
+
+    void *base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t *>(&base), &size,
+                              reinterpret_cast<hipDeviceptr_t>(const_cast<void *>(ptr))) == hipSuccess) {
+        const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+        if (mem.addr < b || mem.len > size || (mem.addr - b) > (size - mem.len)) {
+            NIXL_ERROR << "HIP backend: region [" << mem.addr << ", +" << mem.len
+                       << ") exceeds its allocation";
+            return NIXL_ERR_INVALID_PARAM;
+        }
+    } else {
+        (void)hipGetLastError();
+    }
+
+    out = new nixlHipMD(mem.addr, mem.len, device, nixl_mem);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::deregisterMem(nixlBackendMD *meta) {
+    delete static_cast<nixlHipMD *>(meta);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
+                        const nixl_meta_dlist_t &local,
+                        const nixl_meta_dlist_t &remote,
+                        const std::string &remote_agent,
+                        nixlBackendReqH *&handle,
+                        const nixl_opt_b_args_t *opt_args) const {
+    handle = nullptr;
+    reapRetired(false);
+
+    if (remote_agent != localAgent) {
+        NIXL_ERROR << "HIP backend: only loopback transfers are supported (agent '" << localAgent
+                   << "', remote '" << remote_agent << "')";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
+    if (opt_args && opt_args->hasNotif) return NIXL_ERR_NOT_SUPPORTED;
+    const int n = local.descCount();
+    if (n == 0 || n != remote.descCount()) {
+        NIXL_ERROR << "HIP backend: descriptor count mismatch (local " << n << ", remote "
+                   << remote.descCount() << ")";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    std::vector<nixl_amd_copy_desc_t> lowered(static_cast<size_t>(n));
+    int device = -1;
+    size_t bytes = 0;
+    for (int i = 0; i < n; ++i) {
+        const nixlMetaDesc &l = local[i];
+        const nixlMetaDesc &r = remote[i];
+        if (l.len != r.len) {
+            NIXL_ERROR << "HIP backend: length mismatch at descriptor " << i;
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        const auto *lmd = static_cast<const nixlHipMD *>(l.metadataP);
+        const auto *rmd = static_cast<const nixlHipMD *>(r.metadataP);
+        if (!lmd || !rmd || !lmd->contains(l.addr, l.len) || !rmd->contains(r.addr, r.len)) {
+            NIXL_ERROR << "HIP backend: descriptor " << i << " is outside its registered region";
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        // The kernel runs on the device that owns the VRAM side(s); two VRAM regions on
+        // different devices would need peer mappings, which this backend does not set up.
+        for (const nixlHipMD *md : {lmd, rmd}) {
+            if (md->mem != VRAM_SEG) continue;
+            if (device < 0) device = md->device;
+            if (md->device != device) {
+                NIXL_ERROR << "HIP backend: descriptors span devices " << device << " and " << md->device;
+                return NIXL_ERR_NOT_SUPPORTED;
+            }
+        }
+        const bool write = (operation == NIXL_WRITE);
+        lowered[i].src = write ? l.addr : r.addr;
+        lowered[i].dst = write ? r.addr : l.addr;
+        lowered[i].len = l.len;
+        bytes += l.len;
+    }
+    if (device < 0) device = static_cast<const nixlHipMD *>(local[0].metadataP)->device;
+
+    auto req = std::make_unique<nixlHipReqH>();
+    req->device = device;
+    req->bytes = bytes;
+    if (nixl_amd_copy_plan_create(lowered.data(), lowered.size(), device, &tuning_, &req->plan) !=
+        NIXL_AMD_OK) {
+        NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+        return NIXL_ERR_BACKEND;
+    }
+    if (!hipOk(hipSetDevice(device), "hipSetDevice") ||
+        !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
+        return NIXL_ERR_BACKEND;
+    req->stream = pickStream(device);
+    if (!req->stream) return NIXL_ERR_BACKEND;
+
+    handle = req.release();
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::postXfer(const nixl_xfer_op_t &,
+                        const nixl_meta_dlist_t &,
+                        const nixl_meta_dlist_t &,
+                        const std::string &,
+                        nixlBackendReqH *&handle,
+                        const nixl_opt_b_args_t *opt_args) const {
+    auto *req = static_cast<nixlHipReqH *>(handle);
+    if (!req || !req->plan) return NIXL_ERR_INVALID_PARAM;
+    if (opt_args && opt_args->hasNotif) return NIXL_ERR_NOT_SUPPORTED;
+    if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
+    if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
+
+    if (nixl_amd_copy_plan_launch(req->plan, req->stream) != NIXL_AMD_OK) {
+        NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+        return NIXL_ERR_BACKEND;
+    }
+    if (!hipOk(hipEventRecord(req->done, req->stream), "hipEventRecord")) return NIXL_ERR_BACKEND;
+    req->posted = true;
+    return NIXL_IN_PROG;
+}
+
+nixl_status_t
+nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
+    auto *req = static_cast<nixlHipReqH *>(handle);
+    if (!req) return NIXL_ERR_INVALID_PARAM;
+    if (!req->posted) return NIXL_SUCCESS; // nothing outstanding
+    if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
+    const hipError_t e = hipEventQuery(req->done);
+    if (e == hipSuccess) return NIXL_SUCCESS;
+    if (e == hipErrorNotReady) return NIXL_IN_PROG;
+    NIXL_ERROR << "HIP backend: transfer failed: " << hipGetErrorString(e);
+    return NIXL_ERR_BACKEND;
+}
+
+nixl_status_t
+nixlHipEngine::releaseReqH(nixlBackendReqH *handle) const {
+    auto *req = static_cast<nixlHipReqH *>(handle);
+    if (!req) return NIXL_SUCCESS;
+    (void)hipSetDevice(req->device);
+    if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) {
+        // A launched kernel cannot be cancelled; keep its plan alive until it has
+        // drained and free it from a later call, so that this call never blocks.
+        std::lock_guard<std::mutex> lock(retiredMutex_);
+        retired_.push_back(req);
+        return NIXL_SUCCESS;
+    }
+    delete req;
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::estimateXferCost(const nixl_xfer_op_t &,
+                                const nixl_meta_dlist_t &local,
+                                const nixl_meta_dlist_t &,
+                                const std::string &,
+                                nixlBackendReqH *const &handle,
+                                std::chrono::microseconds &duration,
+                                std::chrono::microseconds &err_margin,
+                                nixl_cost_t &method,
+                                const nixl_opt_args_t *) const {
+    size_t bytes = 0;
+    if (const auto *req = static_cast<const nixlHipReqH *>(handle)) {
+        bytes = req->bytes;
+    } else {
+        for (const auto &d : local)
+            bytes += d.len;
+    }
+    // Read + write of every byte at a conservative 4 TB/s of HBM traffic, plus launch latency.
+    const double us = 10.0 + (2.0 * static_cast<double>(bytes)) / 4.0e6;
+    duration = std::chrono::microseconds(static_cast<long>(us));
+    err_margin = std::chrono::microseconds(static_cast<long>(us * 0.5));
+    method = nixl_cost_t::ANALYTICAL_BACKEND;
+    return NIXL_SUCCESS;
+}
+
+// ---- plugin entry points -------------------------------------------------------------
+
+using hip_plugin_t = nixlBackendPluginCreator<nixlHipEngine>;
+
+extern "C" NIXL_PLUGIN_EXPORT nixlBackendPlugin *
+nixl_plugin_init() {
+    return hip_plugin_t::create(NIXL_PLUGIN_API_VERSION,
+                                "HIP",
+                                "0.1.0",
+                                {{"units_per_lane", "0"},
+                                 {"nontemporal", "0"},
+                                 {"max_workgroups", "0"},
+                                 {"num_streams", "1"}},
+                                {VRAM_SEG, DRAM_SEG});
+}
+
+extern "C" NIXL_PLUGIN_EXPORT void
+nixl_plugin_fini() {}

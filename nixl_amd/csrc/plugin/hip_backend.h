@@ -1,0 +1,153 @@
+// nixlHipEngine: a local-only NIXL backend for VRAM<->VRAM descriptor transfers on one
+// AMD GPU.  It fills the same slot as the reference's local backends (shape of
+// src/plugins/posix/posix_backend.h:78-158; request life-cycle split of
+// src/plugins/cuda_gds/gds_backend.cpp:159-391): prepXfer lowers the two descriptor
+// lists once into a device-resident copy plan, postXfer enqueues one kernel launch and
+// records an event, checkXfer polls the event, releaseReqH frees (or defers freeing if
+// the kernel is still running).
+#ifndef NIXL_AMD_HIP_BACKEND_H
+#define NIXL_AMD_HIP_BACKEND_H
+
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "backend/backend_engine.h"
+#include "nixl_amd_hip.h"
+
+// Registration record returned by registerMem and handed back in nixlMetaDesc::metadataP.
+class nixlHipMD : public nixlBackendMD {
+public:
+    nixlHipMD(uintptr_t addr_, size_t len_, int device_, nixl_mem_t mem_)
+        : nixlBackendMD(true),
+          addr(addr_),
+          len(len_),
+          device(device_),
+          mem(mem_) {}
+
+    const uintptr_t addr;
+    const size_t len;
+    const int device; // HIP device whose kernels may touch the region
+    const nixl_mem_t mem;
+
+    bool
+    contains(uintptr_t a, size_t l) const noexcept {
+        return a >= addr && l <= len && (a - addr) <= (len - l);
+    }
+};
+
+class nixlHipReqH : public nixlBackendReqH {
+public:
+    nixl_amd_copy_plan_t *plan = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t stream = nullptr;
+    int device = 0;
+    bool posted = false;
+    size_t bytes = 0;
+
+    ~nixlHipReqH() override;
+};
+
+class nixlHipEngine : public nixlBackendEngine {
+public:
+    explicit nixlHipEngine(const nixlBackendInitParams *init_params);
+    ~nixlHipEngine() override;
+
+    bool
+    supportsRemote() const override {
+        return false;
+    }
+
+    bool
+    supportsLocal() const override {
+        return true;
+    }
+
+    bool
+    supportsNotif() const override {
+        return false;
+    }
+
+    nixl_mem_list_t
+    getSupportedMems() const override {
+        return {VRAM_SEG, DRAM_SEG};
+    }
+
+    nixl_status_t
+    registerMem(const nixlBlobDesc &mem, const nixl_mem_t &nixl_mem, nixlBackendMD *&out) override;
+    nixl_status_t
+    deregisterMem(nixlBackendMD *meta) override;
+
+    nixl_status_t
+    connect(const std::string &) override {
+        return NIXL_SUCCESS;
+    }
+
+    nixl_status_t
+    disconnect(const std::string &) override {
+        return NIXL_SUCCESS;
+    }
+
+    nixl_status_t
+    unloadMD(nixlBackendMD *) override {
+        return NIXL_SUCCESS;
+    }
+
+    nixl_status_t
+    loadLocalMD(nixlBackendMD *input, nixlBackendMD *&output) override {
+        output = input;
+        return NIXL_SUCCESS;
+    }
+
+    nixl_status_t
+    prepXfer(const nixl_xfer_op_t &operation,
+             const nixl_meta_dlist_t &local,
+             const nixl_meta_dlist_t &remote,
+             const std::string &remote_agent,
+             nixlBackendReqH *&handle,
+             const nixl_opt_b_args_t *opt_args = nullptr) const override;
+    nixl_status_t
+    postXfer(const nixl_xfer_op_t &operation,
+             const nixl_meta_dlist_t &local,
+             const nixl_meta_dlist_t &remote,
+             const std::string &remote_agent,
+             nixlBackendReqH *&handle,
+             const nixl_opt_b_args_t *opt_args = nullptr) const override;
+    nixl_status_t
+    checkXfer(nixlBackendReqH *handle) const override;
+    nixl_status_t
+    releaseReqH(nixlBackendReqH *handle) const override;
+
+    nixl_status_t
+    estimateXferCost(const nixl_xfer_op_t &operation,
+                     const nixl_meta_dlist_t &local,
+                     const nixl_meta_dlist_t &remote,
+                     const std::string &remote_agent,
+                     nixlBackendReqH *const &handle,
+                     std::chrono::microseconds &duration,
+                     std::chrono::microseconds &err_margin,
+                     nixl_cost_t &method,
+                     const nixl_opt_args_t *extra_params = nullptr) const override;
+
+private:
+    hipStream_t
+    pickStream(int device) const;
+    void
+    reapRetired(bool wait) const;
+
+    int numDevices_ = 0;
+    int streamsPerDevice_ = 1;
+    nixl_amd_copy_tuning_t tuning_{};
+    // streams_[device * streamsPerDevice_ + i]; created lazily under streamsMutex_.
+    mutable std::vector<hipStream_t> streams_;
+    mutable std::mutex streamsMutex_;
+    mutable std::atomic<unsigned> nextStream_{0};
+    // Requests released while their kernel was still running; freed once it has finished.
+    mutable std::vector<nixlHipReqH *> retired_;
+    mutable std::mutex retiredMutex_;
+};
+
+#endif
