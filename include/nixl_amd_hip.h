@@ -47,9 +47,11 @@ typedef struct nixl_amd_copy_desc {
 
 /* Launch-shape knobs.  Zero in any field selects the built-in default. */
 typedef struct nixl_amd_copy_tuning {
-    int units_per_lane; /* 16-byte units one lane moves per chunk: 4, 8 or 16 */
+    int units_per_lane; /* 16-byte units one lane moves per chunk: 1, 2, 4, 8 or 16 */
     int nontemporal; /* 1 = non-temporal loads/stores, 2 = plain; 0 = default */
-    int max_workgroups; /* grid cap; waves loop over chunks beyond it */
+    int max_workgroups; /* grid cap of the mixed and byte-path kernels; waves loop beyond it */
+    int waves_per_workgroup; /* uniform-chunk kernel: 1, 2, 4, 8 or 16 */
+    int xcd_swizzle; /* 1 = each accelerator die walks a contiguous slice of the chunk list, 2 = off */
 } nixl_amd_copy_tuning_t;
 
 typedef struct nixl_amd_copy_plan nixl_amd_copy_plan_t;
@@ -87,16 +89,20 @@ int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan);
 
 /* Plan facts: total payload bytes, descriptors on the 128-bit path, descriptors on the
- * byte path, device bytes held by the plan's own arrays, workgroups per launch. */
+ * byte path, device bytes held by the plan's own arrays, and how the 128-bit stream was
+ * cut: chunks lying inside one descriptor (uniform) versus chunks crossing descriptor
+ * boundaries (mixed). */
 typedef struct nixl_amd_copy_plan_info {
     uint64_t payload_bytes;
     uint64_t vec_descs;
     uint64_t generic_descs;
     uint64_t plan_device_bytes;
     uint32_t vec_chunks;
-    uint32_t vec_workgroups;
+    uint32_t uniform_chunks;
+    uint32_t mixed_chunks;
     uint32_t generic_items;
     uint32_t units_per_lane;
+    uint32_t uniform_workgroups;
 } nixl_amd_copy_plan_info_t;
 
 int

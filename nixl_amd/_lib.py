@@ -36,14 +36,16 @@ class CopyDesc(Structure):
 
 
 class CopyTuning(Structure):
-    _fields_ = [("units_per_lane", c_int), ("nontemporal", c_int), ("max_workgroups", c_int)]
+    _fields_ = [("units_per_lane", c_int), ("nontemporal", c_int), ("max_workgroups", c_int),
+                ("waves_per_workgroup", c_int), ("xcd_swizzle", c_int)]
 
 
 class CopyPlanInfo(Structure):
     _fields_ = [("payload_bytes", c_uint64), ("vec_descs", c_uint64), ("generic_descs", c_uint64),
                 ("plan_device_bytes", c_uint64), ("vec_chunks", c_uint32),
-                ("vec_workgroups", c_uint32), ("generic_items", c_uint32),
-                ("units_per_lane", c_uint32)]
+                ("uniform_chunks", c_uint32), ("mixed_chunks", c_uint32),
+                ("generic_items", c_uint32), ("units_per_lane", c_uint32),
+                ("uniform_workgroups", c_uint32)]
 
 
 _kernels = None

@@ -3,15 +3,20 @@
 //
 // Data layout of a plan in HBM
 //   The 16-byte-aligned descriptors of a request are concatenated, in request order, into
-//   one virtual stream measured in 16-byte units.  The plan keeps, per descriptor j,
-//   src[j], dst[j] (byte addresses) and prefix[j] (first unit of j in the stream;
-//   prefix[n] = total units).  The stream is cut into chunks of 64*UPL units; one
-//   wavefront moves one chunk: lane l moves units chunk*64*UPL + k*64 + l, k < UPL, so
-//   every load/store instruction of a wave touches 1 KiB of consecutive bytes unless a
-//   descriptor boundary falls inside it.  span[c] = {first, last} descriptor touched by
-//   chunk c, computed on the host, so a wave never searches the whole prefix array.
+//   one virtual stream measured in 16-byte units.  The stream is cut into chunks of
+//   64*UPL units; one wavefront moves one chunk: lane l moves units k*64 + l of the chunk,
+//   k < UPL, so every load/store instruction of a wave touches 1 KiB of consecutive bytes
+//   unless a descriptor boundary falls inside it.  Chunks are classified on the host:
+//     * a full chunk that lies inside one descriptor becomes a 16-byte record
+//       {src address, dst address} in `uniform[]`; the uniform kernel reads its record
+//       with one scalar load and issues UPL 128-bit loads and UPL 128-bit stores per lane
+//       with wave-uniform base addresses — no search, no LDS, few registers;
+//     * any other chunk (it crosses descriptor boundaries, or it is the short last chunk)
+//       is listed by chunk index in `mixed[]`; the mixed kernel stages the descriptors the
+//       chunk touches (span[c] = {first, last}; src[j], dst[j], prefix[j] = first unit of
+//       descriptor j, prefix[n] = total) in a per-wave LDS slice and walks them.
 //   Descriptors that are not 16-byte aligned in src, dst and len are cut into byte-range
-//   work items handled by a second, byte-exact kernel.
+//   work items handled by a third, byte-exact kernel.
 //
 // What is equal to the reference: the bytes.  For every descriptor, in list order,
 // dst[0..len) = src[0..len), the result of the per-descriptor put/get loop at
@@ -46,18 +51,25 @@ fail(int code, const std::string &msg) {
     } while (0)
 
 constexpr int kWaveSize = 64;
-constexpr int kWavesPerWg = 4;
-constexpr int kThreadsPerWg = kWaveSize * kWavesPerWg;
+constexpr int kMixedWaves = 4; // waves per workgroup of the mixed and byte-path kernels
+constexpr int kMixedThreads = kWaveSize * kMixedWaves;
 constexpr uint32_t kGenericItemBytes = 16384; // byte-path work item size
 constexpr int kMaxLdsDescs = 64; // descriptors a wave stages in LDS for one chunk
+constexpr int kNumXcd = 8; // accelerator dies; workgroup i is dispatched to die i % 8
 
-struct StreamArgs {
+struct UniformRec {
+    uint64_t src;
+    uint64_t dst;
+};
+
+struct MixedArgs {
     const uint64_t *src; // [n]
     const uint64_t *dst; // [n]
     const uint64_t *prefix; // [n + 1], units
     const uint2 *span; // [n_chunks], {first desc, last desc}
+    const uint32_t *chunks; // [n_mixed] chunk indices
     uint64_t total_units;
-    uint32_t n_chunks;
+    uint32_t n_mixed;
 };
 
 struct GenericItem {
@@ -74,18 +86,16 @@ using gv4_ptr = __attribute__((address_space(1))) v4u *;
 using gv4_cptr = const __attribute__((address_space(1))) v4u *;
 
 template<bool NT>
-__device__ __forceinline__ uint4
-load16(const uint4 *p) {
-    gv4_cptr g = (gv4_cptr)(reinterpret_cast<uintptr_t>(p));
-    const v4u v = NT ? __builtin_nontemporal_load(g) : *g;
-    return make_uint4(v[0], v[1], v[2], v[3]);
+__device__ __forceinline__ v4u
+load16(uint64_t addr) {
+    gv4_cptr g = (gv4_cptr)(addr);
+    return NT ? __builtin_nontemporal_load(g) : *g;
 }
 
 template<bool NT>
 __device__ __forceinline__ void
-store16(uint4 *p, const uint4 &x) {
-    gv4_ptr g = (gv4_ptr)(reinterpret_cast<uintptr_t>(p));
-    const v4u v = {x.x, x.y, x.z, x.w};
+store16(uint64_t addr, const v4u &v) {
+    gv4_ptr g = (gv4_ptr)(addr);
     if constexpr (NT)
         __builtin_nontemporal_store(v, g);
     else
@@ -104,52 +114,63 @@ uniform64(uint64_t v) {
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// One wavefront per chunk of the virtual stream, 128-bit loads and stores.
+// Workgroups are handed to the 8 dies round-robin.  With the swizzle on, die x works
+// through one contiguous eighth of the record array instead of every eighth record.
+__device__ __forceinline__ uint32_t
+logical_workgroup(uint32_t n_wgs, bool swizzle) {
+    const uint32_t b = blockIdx.x;
+    if (!swizzle) return b;
+    const uint32_t per = (n_wgs + kNumXcd - 1) / kNumXcd;
+    return (b % kNumXcd) * per + b / kNumXcd; // may be >= n_wgs; caller checks
+}
+
+// One wavefront per full, single-descriptor chunk.
+template<int UPL, bool NT, int WAVES>
+__global__ void __launch_bounds__(kWaveSize *WAVES)
+copy_uniform_kernel(const UniformRec *recs, uint32_t n_recs, uint32_t n_wgs, int swizzle) {
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t wave = threadIdx.x / kWaveSize;
+    const uint32_t wg = logical_workgroup(n_wgs, swizzle != 0);
+    const uint32_t r = uniform(wg * WAVES + wave);
+    if (wg >= n_wgs || r >= n_recs) return;
+    const uint64_t s = uniform64(recs[r].src) + lane * 16u;
+    const uint64_t d = uniform64(recs[r].dst) + lane * 16u;
+    v4u v[UPL];
+#pragma unroll
+    for (int k = 0; k < UPL; ++k)
+        v[k] = load16<NT>(s + k * (kWaveSize * 16u));
+#pragma unroll
+    for (int k = 0; k < UPL; ++k)
+        store16<NT>(d + k * (kWaveSize * 16u), v[k]);
+}
+
+// One wavefront per chunk that crosses descriptor boundaries or is short.
 template<int UPL, bool NT>
-__global__ void __launch_bounds__(kThreadsPerWg)
-copy_stream_kernel(StreamArgs a) {
+__global__ void __launch_bounds__(kMixedThreads)
+copy_mixed_kernel(MixedArgs a) {
     constexpr uint32_t kChunkUnits = kWaveSize * UPL;
-    __shared__ uint64_t lds_prefix[kWavesPerWg][kMaxLdsDescs + 1];
-    __shared__ uint64_t lds_src[kWavesPerWg][kMaxLdsDescs];
-    __shared__ uint64_t lds_dst[kWavesPerWg][kMaxLdsDescs];
+    __shared__ uint64_t lds_prefix[kMixedWaves][kMaxLdsDescs + 1];
+    __shared__ uint64_t lds_src[kMixedWaves][kMaxLdsDescs];
+    __shared__ uint64_t lds_dst[kMixedWaves][kMaxLdsDescs];
 
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = threadIdx.x / kWaveSize;
-    const uint32_t n_waves = gridDim.x * kWavesPerWg;
+    const uint32_t n_waves = gridDim.x * kMixedWaves;
 
-    for (uint32_t c = uniform(blockIdx.x * kWavesPerWg + wave); c < a.n_chunks; c += n_waves) {
+    for (uint32_t m = uniform(blockIdx.x * kMixedWaves + wave); m < a.n_mixed; m += n_waves) {
+        const uint32_t c = uniform(a.chunks[m]);
         const uint2 sp = a.span[c];
         const uint32_t j0 = uniform(sp.x);
         const uint32_t j1 = uniform(sp.y);
         const uint64_t u0 = static_cast<uint64_t>(c) * kChunkUnits;
-        const uint64_t remaining = a.total_units - u0; // > 0 because c < n_chunks
-        const uint32_t n_units =
-            remaining < kChunkUnits ? static_cast<uint32_t>(remaining) : kChunkUnits;
-
-        if (j0 == j1) {
-            // The whole chunk lies inside one descriptor: wave-uniform base addresses.
-            const uint64_t off = (u0 - uniform64(a.prefix[j0])) * 16u;
-            const uint4 *s = reinterpret_cast<const uint4 *>(uniform64(a.src[j0]) + off);
-            uint4 *d = reinterpret_cast<uint4 *>(uniform64(a.dst[j0]) + off);
-            if (n_units == kChunkUnits) {
-                uint4 v[UPL];
-#pragma unroll
-                for (int k = 0; k < UPL; ++k)
-                    v[k] = load16<NT>(s + k * kWaveSize + lane);
-#pragma unroll
-                for (int k = 0; k < UPL; ++k)
-                    store16<NT>(d + k * kWaveSize + lane, v[k]);
-            } else {
-                for (uint32_t i = lane; i < n_units; i += kWaveSize)
-                    store16<NT>(d + i, load16<NT>(s + i));
-            }
-            continue;
-        }
-
+        const uint64_t remaining = a.total_units - u0; // > 0: the host lists only real chunks
+        const uint32_t n_units = remaining < kChunkUnits ? static_cast<uint32_t>(remaining) : kChunkUnits;
         const uint32_t nd = j1 - j0 + 1;
+
         if (nd <= kMaxLdsDescs) {
             // Stage this chunk's descriptors in the wave's LDS slice, then each lane walks
-            // forward through them as its unit index grows by 64 per step.
+            // forward through them as its unit index grows by 64 per step.  Only this
+            // wave touches the slice, and a wave's LDS operations complete in order.
             __builtin_amdgcn_wave_barrier();
             if (lane < nd) {
                 lds_prefix[wave][lane] = a.prefix[j0 + lane];
@@ -162,32 +183,31 @@ copy_stream_kernel(StreamArgs a) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
             uint32_t jj = 0;
-            const uint4 *sp_[UPL];
-            uint4 *dp_[UPL];
-            uint4 v[UPL];
+            uint64_t sa[UPL], da[UPL];
+            v4u v[UPL];
 #pragma unroll
             for (int k = 0; k < UPL; ++k) {
                 const uint32_t i = k * kWaveSize + lane;
-                sp_[k] = nullptr;
-                dp_[k] = nullptr;
+                sa[k] = 0;
+                da[k] = 0;
                 if (i < n_units) {
                     const uint64_t u = u0 + i;
                     while (jj + 1 < nd && lds_prefix[wave][jj + 1] <= u)
                         ++jj;
                     const uint64_t off = (u - lds_prefix[wave][jj]) * 16u;
-                    sp_[k] = reinterpret_cast<const uint4 *>(lds_src[wave][jj] + off);
-                    dp_[k] = reinterpret_cast<uint4 *>(lds_dst[wave][jj] + off);
+                    sa[k] = lds_src[wave][jj] + off;
+                    da[k] = lds_dst[wave][jj] + off;
                 }
             }
 #pragma unroll
             for (int k = 0; k < UPL; ++k)
-                if (sp_[k]) v[k] = load16<NT>(sp_[k]);
+                if (sa[k]) v[k] = load16<NT>(sa[k]);
 #pragma unroll
             for (int k = 0; k < UPL; ++k)
-                if (dp_[k]) store16<NT>(dp_[k], v[k]);
+                if (da[k]) store16<NT>(da[k], v[k]);
             __builtin_amdgcn_wave_barrier();
         } else {
-            // Many tiny descriptors in one chunk: bisect the global prefix array per unit.
+            // More than 64 tiny descriptors in one chunk: bisect the global prefix array.
             for (uint32_t i = lane; i < n_units; i += kWaveSize) {
                 const uint64_t u = u0 + i;
                 uint32_t lo = j0, hi = j1;
@@ -199,9 +219,7 @@ copy_stream_kernel(StreamArgs a) {
                         hi = mid - 1;
                 }
                 const uint64_t off = (u - a.prefix[lo]) * 16u;
-                const uint4 *s = reinterpret_cast<const uint4 *>(a.src[lo] + off);
-                uint4 *d = reinterpret_cast<uint4 *>(a.dst[lo] + off);
-                store16<NT>(d, load16<NT>(s));
+                store16<NT>(a.dst[lo] + off, load16<NT>(a.src[lo] + off));
             }
         }
     }
@@ -212,12 +230,12 @@ struct __attribute__((packed, aligned(1))) unaligned16 {
 };
 
 // One wavefront per byte-range work item; correct for any alignment and length.
-__global__ void __launch_bounds__(kThreadsPerWg)
+__global__ void __launch_bounds__(kMixedThreads)
 copy_generic_kernel(const GenericItem *items, uint32_t n_items) {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = threadIdx.x / kWaveSize;
-    const uint32_t n_waves = gridDim.x * kWavesPerWg;
-    for (uint32_t it = uniform(blockIdx.x * kWavesPerWg + wave); it < n_items; it += n_waves) {
+    const uint32_t n_waves = gridDim.x * kMixedWaves;
+    for (uint32_t it = uniform(blockIdx.x * kMixedWaves + wave); it < n_items; it += n_waves) {
         const uint64_t src = uniform64(items[it].src);
         const uint64_t dst = uniform64(items[it].dst);
         const uint32_t len = uniform(items[it].len);
@@ -248,25 +266,65 @@ copy_generic_kernel(const GenericItem *items, uint32_t n_items) {
     }
 }
 
+template<int UPL, bool NT>
+void
+launch_uniform(int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz) {
+    switch (waves) {
+    case 1: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 1>), grid, dim3(64), 0, s, recs, n, n_wgs, swz); break;
+    case 2: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 2>), grid, dim3(128), 0, s, recs, n, n_wgs, swz); break;
+    case 4: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 4>), grid, dim3(256), 0, s, recs, n, n_wgs, swz); break;
+    case 8: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 8>), grid, dim3(512), 0, s, recs, n, n_wgs, swz); break;
+    default: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 16>), grid, dim3(1024), 0, s, recs, n, n_wgs, swz); break;
+    }
+}
+
+template<bool NT>
+void
+launch_uniform_upl(int upl, int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz) {
+    switch (upl) {
+    case 1: launch_uniform<1, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    case 2: launch_uniform<2, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    case 4: launch_uniform<4, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    case 8: launch_uniform<8, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    default: launch_uniform<16, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    }
+}
+
+template<bool NT>
+void
+launch_mixed_upl(int upl, dim3 grid, hipStream_t s, const MixedArgs &a) {
+    const dim3 block(kMixedThreads);
+    switch (upl) {
+    case 1: hipLaunchKernelGGL((copy_mixed_kernel<1, NT>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((copy_mixed_kernel<2, NT>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((copy_mixed_kernel<4, NT>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((copy_mixed_kernel<8, NT>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((copy_mixed_kernel<16, NT>), grid, block, 0, s, a); break;
+    }
+}
+
 } // namespace
 
 struct nixl_amd_copy_plan {
     int device = 0;
-    int upl = 8;
+    int upl = 1;
     bool nt = true;
+    int waves = 1;
+    int swizzle = 0;
     uint32_t max_wgs = 0;
     // device arrays
     void *arena = nullptr;
     size_t arena_bytes = 0;
-    StreamArgs stream_args{};
+    const UniformRec *uniform_recs = nullptr;
+    uint32_t n_uniform = 0;
+    uint32_t uniform_wgs = 0;
+    MixedArgs mixed_args{};
+    uint32_t mixed_wgs = 0;
     const GenericItem *generic_items = nullptr;
     uint32_t n_generic = 0;
-    uint32_t vec_wgs = 0;
     uint32_t generic_wgs = 0;
-    // facts
     nixl_amd_copy_plan_info_t info{};
-    // timing events (lazily created)
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr; // timing events, created on first use
 };
 
 extern "C" {
@@ -295,16 +353,22 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     if (!descs && n) return fail(NIXL_AMD_ERR_INVALID, "plan_create: descs is null");
     if (n >= (1ull << 32)) return fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: more than 2^32-1 descriptors");
 
-    int upl = 8, nt = 1;
+    // Defaults from a sweep on MI355X: the smallest chunk (one 128-bit load and store per
+    // lane, one wave per workgroup) with non-temporal accesses gave the highest HBM rate.
+    int upl = 1, nt = 1, waves = 1, swizzle = 0;
     uint32_t max_wgs = 0;
     if (tuning) {
         if (tuning->units_per_lane) upl = tuning->units_per_lane;
         if (tuning->nontemporal) nt = tuning->nontemporal;
         if (tuning->max_workgroups > 0) max_wgs = static_cast<uint32_t>(tuning->max_workgroups);
+        if (tuning->waves_per_workgroup) waves = tuning->waves_per_workgroup;
+        if (tuning->xcd_swizzle) swizzle = tuning->xcd_swizzle == 1 ? 1 : 0;
     }
-    if (upl != 4 && upl != 8 && upl != 16)
-        return fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 4, 8 or 16");
+    if (upl != 1 && upl != 2 && upl != 4 && upl != 8 && upl != 16)
+        return fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 1, 2, 4, 8 or 16");
     if (nt != 1 && nt != 2) return fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0, 1 or 2");
+    if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16)
+        return fail(NIXL_AMD_ERR_INVALID, "plan_create: waves_per_workgroup must be 1, 2, 4, 8 or 16");
 
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
@@ -352,6 +416,9 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     const uint32_t n_chunks = static_cast<uint32_t>(n_chunks64);
 
     std::vector<uint2> span(n_chunks);
+    std::vector<UniformRec> uni;
+    std::vector<uint32_t> mixed;
+    uni.reserve(n_chunks);
     {
         size_t j = 0;
         for (uint32_t c = 0; c < n_chunks; ++c) {
@@ -363,32 +430,45 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             while (vprefix[jl + 1] <= last)
                 ++jl;
             span[c] = make_uint2(static_cast<uint32_t>(j), static_cast<uint32_t>(jl));
+            if (j == jl && last - first + 1 == chunk_units) {
+                const uint64_t off = (first - vprefix[j]) * 16u;
+                uni.push_back(UniformRec{vsrc[j] + off, vdst[j] + off});
+            } else {
+                mixed.push_back(c);
+            }
         }
     }
 
     // ---- one device arena for all plan arrays --------------------------------------
     auto align256 = [](size_t x) { return (x + 255) & ~size_t(255); };
-    const size_t off_src = 0;
-    const size_t off_dst = off_src + align256(nv * 8);
-    const size_t off_prefix = off_dst + align256(nv * 8);
-    const size_t off_span = off_prefix + align256((nv + 1) * 8);
-    const size_t off_items = off_span + align256(size_t(n_chunks) * sizeof(uint2));
+    const bool need_desc_arrays = !mixed.empty();
+    const size_t off_uni = 0;
+    const size_t off_src = off_uni + align256(uni.size() * sizeof(UniformRec));
+    const size_t off_dst = off_src + (need_desc_arrays ? align256(nv * 8) : 0);
+    const size_t off_prefix = off_dst + (need_desc_arrays ? align256(nv * 8) : 0);
+    const size_t off_span = off_prefix + (need_desc_arrays ? align256((nv + 1) * 8) : 0);
+    const size_t off_mixed = off_span + (need_desc_arrays ? align256(size_t(n_chunks) * sizeof(uint2)) : 0);
+    const size_t off_items = off_mixed + align256(mixed.size() * sizeof(uint32_t));
     const size_t total = off_items + align256(items.size() * sizeof(GenericItem));
 
     auto *plan = new nixl_amd_copy_plan();
     plan->device = device;
     plan->upl = upl;
     plan->nt = (nt == 1);
+    plan->waves = waves;
+    plan->swizzle = swizzle;
     plan->max_wgs = max_wgs;
 
-    if (total > 0 && (nv > 0 || !items.empty())) {
+    if (total > 0) {
         std::vector<uint8_t> host(total, 0);
-        if (nv) {
+        if (!uni.empty()) std::memcpy(host.data() + off_uni, uni.data(), uni.size() * sizeof(UniformRec));
+        if (need_desc_arrays) {
             std::memcpy(host.data() + off_src, vsrc.data(), nv * 8);
             std::memcpy(host.data() + off_dst, vdst.data(), nv * 8);
+            std::memcpy(host.data() + off_prefix, vprefix.data(), (nv + 1) * 8);
+            std::memcpy(host.data() + off_span, span.data(), size_t(n_chunks) * sizeof(uint2));
+            std::memcpy(host.data() + off_mixed, mixed.data(), mixed.size() * sizeof(uint32_t));
         }
-        std::memcpy(host.data() + off_prefix, vprefix.data(), (nv + 1) * 8);
-        if (n_chunks) std::memcpy(host.data() + off_span, span.data(), size_t(n_chunks) * sizeof(uint2));
         if (!items.empty())
             std::memcpy(host.data() + off_items, items.data(), items.size() * sizeof(GenericItem));
         hipError_t e = hipMalloc(&plan->arena, total);
@@ -404,32 +484,38 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         }
         plan->arena_bytes = total;
         auto *base = static_cast<uint8_t *>(plan->arena);
-        plan->stream_args.src = reinterpret_cast<const uint64_t *>(base + off_src);
-        plan->stream_args.dst = reinterpret_cast<const uint64_t *>(base + off_dst);
-        plan->stream_args.prefix = reinterpret_cast<const uint64_t *>(base + off_prefix);
-        plan->stream_args.span = reinterpret_cast<const uint2 *>(base + off_span);
+        plan->uniform_recs = reinterpret_cast<const UniformRec *>(base + off_uni);
+        plan->mixed_args.src = reinterpret_cast<const uint64_t *>(base + off_src);
+        plan->mixed_args.dst = reinterpret_cast<const uint64_t *>(base + off_dst);
+        plan->mixed_args.prefix = reinterpret_cast<const uint64_t *>(base + off_prefix);
+        plan->mixed_args.span = reinterpret_cast<const uint2 *>(base + off_span);
+        plan->mixed_args.chunks = reinterpret_cast<const uint32_t *>(base + off_mixed);
         plan->generic_items = reinterpret_cast<const GenericItem *>(base + off_items);
     }
-    plan->stream_args.total_units = units;
-    plan->stream_args.n_chunks = n_chunks;
+    plan->n_uniform = static_cast<uint32_t>(uni.size());
+    plan->mixed_args.total_units = units;
+    plan->mixed_args.n_mixed = static_cast<uint32_t>(mixed.size());
     plan->n_generic = static_cast<uint32_t>(items.size());
 
-    auto wgs_for = [&](uint32_t waves) {
-        uint32_t w = (waves + kWavesPerWg - 1) / kWavesPerWg;
-        if (plan->max_wgs && w > plan->max_wgs) w = plan->max_wgs;
+    auto wgs_for = [&](uint32_t n_waves, uint32_t waves_per_wg, bool cap) {
+        uint32_t w = (n_waves + waves_per_wg - 1) / waves_per_wg;
+        if (cap && plan->max_wgs && w > plan->max_wgs) w = plan->max_wgs;
         return w;
     };
-    plan->vec_wgs = wgs_for(n_chunks);
-    plan->generic_wgs = wgs_for(plan->n_generic);
+    plan->uniform_wgs = wgs_for(plan->n_uniform, static_cast<uint32_t>(waves), false);
+    plan->mixed_wgs = wgs_for(plan->mixed_args.n_mixed, kMixedWaves, true);
+    plan->generic_wgs = wgs_for(plan->n_generic, kMixedWaves, true);
 
     plan->info.payload_bytes = payload;
     plan->info.vec_descs = nv;
     plan->info.generic_descs = n_generic_descs;
     plan->info.plan_device_bytes = plan->arena_bytes;
     plan->info.vec_chunks = n_chunks;
-    plan->info.vec_workgroups = plan->vec_wgs;
+    plan->info.uniform_chunks = plan->n_uniform;
+    plan->info.mixed_chunks = plan->mixed_args.n_mixed;
     plan->info.generic_items = plan->n_generic;
     plan->info.units_per_lane = static_cast<uint32_t>(upl);
+    plan->info.uniform_workgroups = plan->uniform_wgs;
     *out = plan;
     return NIXL_AMD_OK;
 }
@@ -439,24 +525,28 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
     if (!plan) return fail(NIXL_AMD_ERR_INVALID, "plan_launch: plan is null");
     HIP_TRY(hipSetDevice(plan->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (plan->vec_wgs) {
-        const dim3 grid(plan->vec_wgs), block(kThreadsPerWg);
-        const StreamArgs &a = plan->stream_args;
-#define LAUNCH_STREAM(UPL_, NT_) hipLaunchKernelGGL((copy_stream_kernel<UPL_, NT_>), grid, block, 0, s, a)
-        if (plan->nt) {
-            if (plan->upl == 4) LAUNCH_STREAM(4, true);
-            else if (plan->upl == 8) LAUNCH_STREAM(8, true);
-            else LAUNCH_STREAM(16, true);
-        } else {
-            if (plan->upl == 4) LAUNCH_STREAM(4, false);
-            else if (plan->upl == 8) LAUNCH_STREAM(8, false);
-            else LAUNCH_STREAM(16, false);
-        }
-#undef LAUNCH_STREAM
+    if (plan->uniform_wgs) {
+        // With the die swizzle the grid is rounded up to a multiple of 8 so that every
+        // die owns an equally long slice; surplus workgroups exit at once.
+        uint32_t grid = plan->uniform_wgs;
+        if (plan->swizzle) grid = ((grid + kNumXcd - 1) / kNumXcd) * kNumXcd;
+        if (plan->nt)
+            launch_uniform_upl<true>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
+                                     plan->uniform_wgs, plan->swizzle);
+        else
+            launch_uniform_upl<false>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
+                                      plan->uniform_wgs, plan->swizzle);
+        HIP_TRY(hipGetLastError());
+    }
+    if (plan->mixed_wgs) {
+        if (plan->nt)
+            launch_mixed_upl<true>(plan->upl, dim3(plan->mixed_wgs), s, plan->mixed_args);
+        else
+            launch_mixed_upl<false>(plan->upl, dim3(plan->mixed_wgs), s, plan->mixed_args);
         HIP_TRY(hipGetLastError());
     }
     if (plan->generic_wgs) {
-        hipLaunchKernelGGL(copy_generic_kernel, dim3(plan->generic_wgs), dim3(kThreadsPerWg), 0, s,
+        hipLaunchKernelGGL(copy_generic_kernel, dim3(plan->generic_wgs), dim3(kMixedThreads), 0, s,
                            plan->generic_items, plan->n_generic);
         HIP_TRY(hipGetLastError());
     }

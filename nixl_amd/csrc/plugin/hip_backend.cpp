@@ -41,9 +41,25 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     tuning_.units_per_lane = paramInt(p, "units_per_lane", 0);
     tuning_.nontemporal = paramInt(p, "nontemporal", 0);
     tuning_.max_workgroups = paramInt(p, "max_workgroups", 0);
+    tuning_.waves_per_workgroup = paramInt(p, "waves_per_workgroup", 0);
+    tuning_.xcd_swizzle = paramInt(p, "xcd_swizzle", 0);
     streamsPerDevice_ = paramInt(p, "num_streams", 1);
     if (streamsPerDevice_ < 1 || streamsPerDevice_ > 16)
         throw std::runtime_error("HIP backend: num_streams must be in [1, 16]");
+    if (p) {
+        // "stream" carries a hipStream_t of the application, as an integer.  Transfers are
+        // then enqueued there, ordered with the application's own work on that stream, and
+        // the application may bracket them with its own events.
+        const auto it = p->find("stream");
+        if (it != p->end() && !it->second.empty()) {
+            char *end = nullptr;
+            const unsigned long long v = std::strtoull(it->second.c_str(), &end, 0);
+            if (end == it->second.c_str() || *end != '\0')
+                throw std::runtime_error("HIP backend: parameter 'stream' is not an integer: " + it->second);
+            externalStream_ = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(v));
+            useExternalStream_ = true;
+        }
+    }
 
     const int n = nixl_amd_device_count();
     if (n <= 0) {
@@ -67,6 +83,7 @@ nixlHipEngine::~nixlHipEngine() {
 
 hipStream_t
 nixlHipEngine::pickStream(int device) const {
+    if (useExternalStream_) return externalStream_;
     const unsigned slot = nextStream_.fetch_add(1, std::memory_order_relaxed) % streamsPerDevice_;
     const size_t idx = static_cast<size_t>(device) * streamsPerDevice_ + slot;
     std::lock_guard<std::mutex> lock(streamsMutex_);
@@ -231,7 +248,7 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
         !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
         return NIXL_ERR_BACKEND;
     req->stream = pickStream(device);
-    if (!req->stream) return NIXL_ERR_BACKEND;
+    if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
 
     handle = req.release();
     return NIXL_SUCCESS;
@@ -325,7 +342,10 @@ nixl_plugin_init() {
                                 {{"units_per_lane", "0"},
                                  {"nontemporal", "0"},
                                  {"max_workgroups", "0"},
-                                 {"num_streams", "1"}},
+                                 {"waves_per_workgroup", "0"},
+                                 {"xcd_swizzle", "0"},
+                                 {"num_streams", "1"},
+                                 {"stream", ""}},
                                 {VRAM_SEG, DRAM_SEG});
 }
 

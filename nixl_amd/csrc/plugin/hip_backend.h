@@ -140,6 +140,8 @@ private:
 
     int numDevices_ = 0;
     int streamsPerDevice_ = 1;
+    bool useExternalStream_ = false; // launches go to the application's stream (may be the null stream)
+    hipStream_t externalStream_ = nullptr;
     nixl_amd_copy_tuning_t tuning_{};
     // streams_[device * streamsPerDevice_ + i]; created lazily under streamsMutex_.
     mutable std::vector<hipStream_t> streams_;

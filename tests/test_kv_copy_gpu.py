@@ -1,0 +1,356 @@
+"""GPU parity tests for the descriptor-transfer half: the copy kernels through their C ABI
+and the HIP backend plugin through the agent, against the CPU oracle (per-descriptor
+memcpy) and through size-independent properties at full configuration sizes."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import kv_oracle as ko
+from nixl_amd import _lib, nixl_agent, nixl_agent_config
+from nixl_amd import agent as ag
+
+pytestmark = pytest.mark.gpu
+
+
+def _plan(descs, tuning=None):
+    lib = _lib.kernels()
+    arr = (_lib.CopyDesc * len(descs))(*[_lib.CopyDesc(int(s), int(d), int(n)) for s, d, n in descs])
+    plan = ctypes.c_void_p()
+    t = ctypes.byref(_lib.CopyTuning(*tuning)) if tuning else None
+    rc = lib.nixl_amd_copy_plan_create(arr, len(descs), 0, t, ctypes.byref(plan))
+    assert rc == 0, _lib.kernels_error()
+    return plan
+
+
+def _run_plan(torch, plan):
+    lib = _lib.kernels()
+    torch.cuda.synchronize()
+    assert lib.nixl_amd_copy_plan_launch(plan, None) == 0, _lib.kernels_error()
+    torch.cuda.synchronize()
+
+
+def _check_against_oracle(torch, cuda, mem_bytes, src_off, dst_off, lens, tuning=None, seed=0):
+    rng = np.random.default_rng(seed)
+    host = rng.integers(0, 256, mem_bytes, dtype=np.uint8)
+    dev = torch.from_numpy(host.copy()).to(cuda)
+    base = dev.data_ptr()
+    plan = _plan([(base + s, base + d, n) for s, d, n in zip(src_off, dst_off, lens)], tuning)
+    info = _lib.CopyPlanInfo()
+    _lib.kernels().nixl_amd_copy_plan_query(plan, ctypes.byref(info))
+    _run_plan(torch, plan)
+    want = ko.copy_descs(host, src_off, dst_off, lens)
+    got = dev.cpu().numpy()
+    assert _lib.kernels().nixl_amd_copy_plan_destroy(plan) == 0
+    assert np.array_equal(got, want), f"first mismatch at byte {int(np.argmax(got != want))}"
+    return info
+
+
+def _disjoint_layout(rng, lens, align, region):
+    """Random non-overlapping offsets for the given lengths inside [0, region)."""
+    order = rng.permutation(len(lens))
+    sizes = np.array([((int(lens[i]) + align - 1) // align + 1) * align for i in order], dtype=np.int64)
+    starts = np.concatenate([[0], np.cumsum(sizes)])
+    assert starts[-1] <= region
+    offs = np.empty(len(lens), dtype=np.int64)
+    offs[order] = starts[:-1]
+    return offs
+
+
+@pytest.mark.parametrize("upl", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("nt", [1, 2])
+def test_aligned_descriptors_match_oracle(cuda, upl, nt):
+    import torch
+    rng = np.random.default_rng(upl * 10 + nt)
+    # sizes straddling every chunk boundary case: sub-wave, exactly one chunk, several chunks
+    lens = [16, 32, 512, 1008, 1024, 4096, 8192, 8208, 16384, 32768, 65536 + 48, 16 * upl * 64, 16 * upl * 64 - 16]
+    lens += [int(x) * 16 for x in rng.integers(1, 600, 200)]
+    half = 8 << 20
+    so = _disjoint_layout(rng, lens, 16, half)
+    do = _disjoint_layout(rng, lens, 16, half) + half
+    info = _check_against_oracle(torch, cuda, 2 * half, so, do, lens, (upl, nt, 0, 0, 0), seed=upl)
+    assert info.vec_descs == len(lens) and info.generic_descs == 0
+    assert info.payload_bytes == sum(lens)
+
+
+def test_ragged_small_descriptors_match_oracle(cuda):
+    # BASELINE config 3 in miniature: sizes log-uniform in [512, 4096] rounded to 16.
+    import torch
+    rng = np.random.default_rng(33)
+    n = 20000
+    lens = (np.exp(rng.uniform(np.log(512), np.log(4096), n)).astype(np.int64) // 16) * 16
+    half = 96 << 20
+    so = _disjoint_layout(rng, lens, 16, half)
+    do = _disjoint_layout(rng, lens, 16, half) + half
+    _check_against_oracle(torch, cuda, 2 * half, so, do, lens, seed=5)
+
+
+def test_many_tiny_descriptors_in_one_chunk(cuda):
+    # 16-byte descriptors: more than 64 descriptors fall into one 8 KiB chunk, which takes
+    # the bisection path of the kernel.
+    import torch
+    rng = np.random.default_rng(4)
+    lens = [16] * 3000 + [48] * 100
+    half = 1 << 20
+    so = _disjoint_layout(rng, lens, 16, half)
+    do = _disjoint_layout(rng, lens, 16, half) + half
+    _check_against_oracle(torch, cuda, 2 * half, so, do, lens, seed=6)
+
+
+def test_unaligned_brute_force(cuda):
+    # every length 1..80 with every src/dst residue mod 16 in turn, plus long odd spans
+    import torch
+    src_off, dst_off, lens = [], [], []
+    pos_s, pos_d = 0, 1 << 20
+    k = 0
+    for n in list(range(1, 81)) + [255, 1000, 4097, 16385, 40001]:
+        for _ in range(4):
+            sa, da = k % 16, (k // 16 + k) % 16
+            k += 7
+            src_off.append(pos_s + sa)
+            dst_off.append(pos_d + da)
+            lens.append(n)
+            pos_s += ((n + 31) // 16 + 1) * 16
+            pos_d += ((n + 31) // 16 + 1) * 16
+    assert pos_s <= (1 << 20)
+    info = _check_against_oracle(torch, cuda, 2 << 20, src_off, dst_off, lens, seed=8)
+    assert info.generic_descs > 0
+
+
+def test_zero_length_and_empty(cuda):
+    import torch
+    dev = torch.zeros(4096, dtype=torch.uint8, device=cuda)
+    plan = _plan([(dev.data_ptr(), dev.data_ptr() + 2048, 0)])
+    info = _lib.CopyPlanInfo()
+    _lib.kernels().nixl_amd_copy_plan_query(plan, ctypes.byref(info))
+    assert info.payload_bytes == 0 and info.vec_chunks == 0
+    _run_plan(torch, plan)
+    _lib.kernels().nixl_amd_copy_plan_destroy(plan)
+    # null address / bad tuning are rejected on the host, before any launch
+    lib = _lib.kernels()
+    out = ctypes.c_void_p()
+    bad = (_lib.CopyDesc * 1)(_lib.CopyDesc(0, dev.data_ptr(), 16))
+    assert lib.nixl_amd_copy_plan_create(bad, 1, 0, None, ctypes.byref(out)) == -1
+    ok = (_lib.CopyDesc * 1)(_lib.CopyDesc(dev.data_ptr(), dev.data_ptr() + 16, 16))
+    assert lib.nixl_amd_copy_plan_create(ok, 1, 0, ctypes.byref(_lib.CopyTuning(5, 0, 0, 0, 0)), ctypes.byref(out)) == -1
+    assert lib.nixl_amd_copy_plan_create(ok, 1, 99, None, ctypes.byref(out)) == -1
+
+
+# ---- through the agent and the plugin --------------------------------------------------------
+
+@pytest.fixture()
+def hip_agent(cuda):
+    a = nixl_agent("agent", nixl_agent_config(backends=("HIP",)))
+    yield a
+    a.close()
+
+
+def _wait(a, req):
+    st = a.transfer(req)
+    assert st in ("DONE", "PROC")
+    while st == "PROC":
+        st = a.check_xfer_state(req)
+    assert st == "DONE"
+
+
+def _descs(t, offs, lens):
+    offs = np.asarray(offs, dtype=np.uint64)
+    return np.stack([np.uint64(t.data_ptr()) + offs, np.asarray(lens, dtype=np.uint64), np.zeros_like(offs)], 1)
+
+
+def test_prepared_lists_three_requests(hip_agent, cuda):
+    # Shape of test/nixl/agent_example.cpp:375-531 (sideXferTest): 32 x 1 KiB buffers per
+    # side, both sides prepared once, three requests with different index vectors off the
+    # same handles; every destination byte must be 0xbb (check_buf, :28-34).
+    import torch
+    a = hip_agent
+    n, ln = 32, 1024
+    src = torch.full((n * ln,), 0xBB, dtype=torch.uint8, device=cuda)
+    dst = torch.zeros(n * ln, dtype=torch.uint8, device=cuda)
+    a.register_memory([src, dst])
+    offs = np.arange(n) * ln
+    hl = a.prep_xfer_dlist("", _descs(src, offs, [ln] * n), "VRAM")
+    hr = a.prep_xfer_dlist("agent", _descs(dst, offs, [ln] * n), "VRAM")
+    torch.cuda.synchronize()
+    lo, hi = np.arange(16), np.arange(16, 32)
+    r1 = a.make_prepped_xfer("WRITE", hl, lo, hr, lo)
+    _wait(a, r1)
+    assert bool((dst[:16 * ln] == 0xBB).all()) and bool((dst[16 * ln:] == 0).all())
+    src[16 * ln:] = 0
+    torch.cuda.synchronize()
+    r2 = a.make_prepped_xfer("READ", hl, hi, hr, lo)  # local[16..31] <- remote[0..15]
+    _wait(a, r2)
+    assert bool((src == 0xBB).all())
+    r3 = a.make_prepped_xfer("WRITE", hl, hi, hr, hi)
+    _wait(a, r3)
+    assert bool((dst == 0xBB).all())
+    for h in (r1, r2, r3, hl, hr):
+        h.release()
+
+
+def test_write_zero_read_roundtrip_and_repost(hip_agent, cuda):
+    # transfer_handler round trip (test/gtest/plugins/transfer_handler.h:182-209 with
+    # memory_handler.h:42-58): WRITE, clear the source, READ back, expect the increasing
+    # pattern 0x11+i.  Then the repost rule of test/unit/plugins/posix/nixl_posix_test.cpp:
+    # 714-770: the same handles posted again after the source changed deliver the new bytes.
+    import torch
+    a = hip_agent
+    n = 1 << 20
+    pattern = (torch.arange(n, device=cuda) + 0x11).to(torch.uint8)
+    src = pattern.clone()
+    dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
+    reg = a.register_memory([src, dst])
+    # split_buf: four 16-byte entries at the start, then the rest in one descriptor
+    offs = [0, 16, 32, 48, 64]
+    lens = [16, 16, 16, 16, n - 64]
+    ld = a.get_xfer_descs(_descs(src, offs, lens), "VRAM")
+    rd = a.get_xfer_descs(_descs(dst, offs, lens), "VRAM")
+    torch.cuda.synchronize()
+    w = a.initialize_xfer("WRITE", ld, rd, "agent")
+    r = a.initialize_xfer("READ", ld, rd, "agent")
+    assert w.desc_count() == (5, n)  # createXferReq does not merge
+    _wait(a, w)
+    assert torch.equal(dst, pattern)
+    src.zero_()
+    torch.cuda.synchronize()
+    _wait(a, r)
+    assert torch.equal(src, pattern)
+    src.fill_(0x5A)
+    torch.cuda.synchronize()
+    _wait(a, w)  # repost of the same handle
+    assert bool((dst == 0x5A).all())
+    a.deregister_memory(reg)  # before releasing the requests, as the reference test does
+    w.release()
+    r.release()
+
+
+def test_plugin_rejects_what_it_cannot_do(hip_agent, cuda):
+    import torch
+    a = hip_agent
+    t = torch.zeros(4096, dtype=torch.uint8, device=cuda)
+    # wrong device id in the registration descriptor
+    with pytest.raises(ag.NixlError):
+        a.register_memory(np.array([[t.data_ptr(), 4096, 3]], dtype=np.uint64), "VRAM")
+    # an address HIP does not know
+    host = np.zeros(4096, np.uint8)
+    with pytest.raises(ag.NixlError):
+        a.register_memory(np.array([[host.ctypes.data, 4096, 0]], dtype=np.uint64), "VRAM")
+    a.register_memory([t])
+    # notifications are not supported by a local-only backend
+    ld = a.get_xfer_descs(_descs(t, [0], [16]), "VRAM")
+    rd = a.get_xfer_descs(_descs(t, [2048], [16]), "VRAM")
+    with pytest.raises(ag.NixlError) as e:
+        a.initialize_xfer("WRITE", ld, rd, "agent", notif_msg=b"n")
+    assert e.value.status == ag.NIXL_ERR_BACKEND
+
+
+def test_release_while_in_flight_does_not_block_or_corrupt(hip_agent, cuda):
+    import torch
+    a = hip_agent
+    n = 256 << 20
+    src = torch.full((n,), 7, dtype=torch.uint8, device=cuda)
+    dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
+    a.register_memory([src, dst])
+    torch.cuda.synchronize()
+    req = a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(src, [0], [n]), "VRAM"),
+                            a.get_xfer_descs(_descs(dst, [0], [n]), "VRAM"), "agent")
+    a.transfer(req)
+    req.release()  # may still be running: the backend must keep the plan alive
+    torch.cuda.synchronize()
+    assert bool((dst == 7).all())
+
+
+def test_config2_llama3_kv_gather_scatter_full_size(hip_agent, cuda):
+    # BASELINE config 2 at full size: pool [32 layers][K,V][8192 blocks][32 KiB] of bf16
+    # N(0,1); gather 1024 random blocks into contiguous staging (65536 descriptors), then
+    # scatter to a seeded permutation of destination block ids in a second pool.  Checked
+    # through properties: staging equals the torch gather of the source pool, the
+    # destination blocks equal the source blocks, untouched destination blocks keep their
+    # canary, and a checksum of the moved bytes is preserved.
+    import torch
+    a = hip_agent
+    layers, pool_blocks, blk = 32, 8192, 32768
+    n_sel = 1024
+    lk = layers * 2
+    gen = torch.Generator(device=cuda)
+    gen.manual_seed(1234)
+    src_pool = torch.empty((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=cuda)
+    for i in range(lk):
+        src_pool[i] = torch.randn((pool_blocks, blk // 2), generator=gen, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+    dst_pool = torch.full((lk, pool_blocks, blk // 2), -7.0, dtype=torch.bfloat16, device=cuda)
+    staging = torch.zeros((n_sel, lk, blk // 2), dtype=torch.bfloat16, device=cuda)
+    a.register_memory([src_pool, dst_pool, staging])
+
+    rng = np.random.default_rng(99)
+    sel = rng.choice(pool_blocks, n_sel, replace=False)
+    dst_ids = rng.permutation(pool_blocks)[:n_sel]
+    n_desc = n_sel * lk
+    lens = np.full(n_desc, blk, dtype=np.uint64)
+    zeros = np.zeros(n_desc, dtype=np.uint64)
+    src_addrs = ko.kv_block_descs(src_pool.data_ptr(), layers, pool_blocks, blk, sel)
+    dst_addrs = ko.kv_block_descs(dst_pool.data_ptr(), layers, pool_blocks, blk, dst_ids)
+    stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
+    h_src = a.prep_xfer_dlist("", np.stack([src_addrs, lens, zeros], 1), "VRAM")
+    h_stg_r = a.prep_xfer_dlist("agent", np.stack([stg_addrs, lens, zeros], 1), "VRAM")
+    h_stg_l = a.prep_xfer_dlist("", np.stack([stg_addrs, lens, zeros], 1), "VRAM")
+    h_dst = a.prep_xfer_dlist("agent", np.stack([dst_addrs, lens, zeros], 1), "VRAM")
+    idx = np.arange(n_desc)
+    gather = a.make_prepped_xfer("WRITE", h_src, idx, h_stg_r, idx)
+    scatter = a.make_prepped_xfer("WRITE", h_stg_l, idx, h_dst, idx)
+    assert gather.desc_count() == (n_desc, n_desc * blk)
+    torch.cuda.synchronize()
+    _wait(a, gather)
+    _wait(a, scatter)
+
+    sel_t = torch.from_numpy(sel).to(cuda)
+    dst_t = torch.from_numpy(dst_ids).to(cuda)
+    want_staging = src_pool[:, sel_t, :].permute(1, 0, 2)
+    assert torch.equal(staging.view(torch.int16), want_staging.contiguous().view(torch.int16))
+    assert torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16))
+    untouched = torch.ones(pool_blocks, dtype=torch.bool, device=cuda)
+    untouched[dst_t] = False
+    assert bool((dst_pool[:, untouched, :] == -7.0).all())
+    moved_sum = src_pool[:, sel_t, :].view(torch.int16).to(torch.int64).sum()
+    assert int(dst_pool[:, dst_t, :].view(torch.int16).to(torch.int64).sum()) == int(moved_sum)
+    for h in (gather, scatter, h_src, h_stg_r, h_stg_l, h_dst):
+        h.release()
+
+
+def test_config3_small_descriptor_stress_full_size(hip_agent, cuda):
+    # BASELINE config 3: 262144 descriptors, sizes log-uniform in [512 B, 4 KiB] rounded to
+    # 16 B, random 16 B-aligned offsets in two 4 GiB buffers, destinations non-overlapping.
+    # Verified exactly against a torch gather/scatter of the same spans done with 16-byte
+    # elements, and by a canary (0xC3) over every destination byte no descriptor covers.
+    import torch
+    a = hip_agent
+    n = 262144
+    buf_bytes = 4 << 30
+    rng = np.random.default_rng(2025)
+    lens = (np.exp(rng.uniform(np.log(512), np.log(4096), n)).astype(np.int64) // 16) * 16
+    src = torch.randint(0, 256, (buf_bytes,), dtype=torch.uint8, device=cuda)
+    dst = torch.full((buf_bytes,), 0xC3, dtype=torch.uint8, device=cuda)
+    a.register_memory([src, dst])
+    so = rng.integers(0, (buf_bytes - 4096) // 16, n) * 16
+    # non-overlapping destinations: shuffled slots of 4 KiB + random slack inside a slot
+    slots = rng.permutation(buf_bytes // 8192)[:n] * 8192
+    do = slots + (rng.integers(0, (8192 - 4096) // 16, n) * 16)
+    zeros = np.zeros(n, dtype=np.uint64)
+    hl = a.prep_xfer_dlist("", np.stack([np.uint64(src.data_ptr()) + so.astype(np.uint64), lens.astype(np.uint64), zeros], 1), "VRAM")
+    hr = a.prep_xfer_dlist("agent", np.stack([np.uint64(dst.data_ptr()) + do.astype(np.uint64), lens.astype(np.uint64), zeros], 1), "VRAM")
+    req = a.make_prepped_xfer("WRITE", hl, np.arange(n), hr, np.arange(n))
+    torch.cuda.synchronize()
+    _wait(a, req)
+
+    units = lens // 16
+    starts = np.concatenate([[0], np.cumsum(units)])
+    owner = np.repeat(np.arange(n), units)
+    within = np.arange(starts[-1]) - starts[owner]
+    s_unit = torch.from_numpy(so[owner] // 16 + within).to(cuda)
+    d_unit = torch.from_numpy(do[owner] // 16 + within).to(cuda)
+    src16 = src.view(torch.int64).view(-1, 2)
+    expect = torch.full((buf_bytes,), 0xC3, dtype=torch.uint8, device=cuda)
+    expect.view(torch.int64).view(-1, 2)[d_unit] = src16[s_unit]
+    diff = int((dst.view(torch.int64) != expect.view(torch.int64)).sum())
+    assert diff == 0, f"{diff} of {buf_bytes // 8} 8-byte words differ"
+    for h in (req, hl, hr):
+        h.release()
