@@ -1,0 +1,228 @@
+/*
+ * C ABI of the expert-parallel (EP) dispatch / combine kernels (libnixl_amd_kernels.so).
+ *
+ * These entry points stand where the reference's kernel launchers stand — plain functions
+ * taking raw pointers, sizes and a stream (examples/device/ep/csrc/kernels/api.cuh:63-72,
+ * 81-203,211-238) — with one change of shape: the reference launches one rank's kernel per
+ * process and moves data between processes; here every rank of the job is a region of one
+ * GPU's HBM, so each call processes ALL virtual ranks and every array carries a leading
+ * rank dimension.  `rank`, the RDMA buffers, `next_clean`, `phases`, time-outs and the
+ * device-side NIXL context of the reference signatures have no meaning on one GPU and are
+ * gone.  Results are what the reference kernels deliver, in their canonical order (segments
+ * by source rank ascending, tokens ascending), bit for bit.
+ *
+ * Notation: R ranks, E experts (E % R == 0), El = E / R, T tokens per rank as laid out,
+ * K top-k, H hidden, M = num_max_dispatch_tokens_per_rank, N = R * M.
+ * `stream` is a hipStream_t passed as void*.  All pointers are device pointers unless
+ * stated otherwise.  Return value: 0 or a negative nixl_amd_status (nixl_amd_hip.h);
+ * nixl_amd_last_error() has the text.  Arguments are validated on the host before any
+ * launch; nothing falls back to a CPU path.
+ */
+#ifndef NIXL_AMD_EP_H
+#define NIXL_AMD_EP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Bytes of scratch the low-latency dispatch needs (per-(rank, expert) send counts and
+ * per-(token, k) positions).  Reference: `workspace` of ep_kernels::dispatch,
+ * kernels/nixl_ep_ll.cu:423-426. */
+size_t
+nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk);
+
+/*
+ * Low-latency dispatch for all ranks.  Replaces ep_kernels::dispatch
+ * (kernels/api.cuh:211-224; kernel kernels/nixl_ep_ll.cu:71-395; host
+ * csrc/nixl_ep.cpp:1030-1143).
+ *   x                      [R][T][H] bf16
+ *   topk_idx               [R][T][K] int32, -1 = no selection; the K entries of one token
+ *                          must be distinct (as a top-k selection is)
+ *   num_tokens_per_rank    [R] int32 tokens present on each rank (<= T), or NULL = T
+ *   mask_buffer            [R][R] int32 or NULL; tokens travel a -> b only if neither
+ *                          mask[a][b] nor mask[b][a] is set (kernels/nixl_ep_ll.cu:197,266,319)
+ *   packed_recv_x          [R][El][N][H]    fp8 e4m3 (use_fp8) or bf16
+ *   packed_recv_x_scales   [R][El][H/128][N] float, or with use_ue8m0 [R][El][H/512][N]
+ *                          int32 words of four exponent bytes; NULL unless use_fp8
+ *   packed_recv_src_info   [R][El][N] int32
+ *   packed_recv_layout_range [R][El][R] int64: count | begin << 32
+ *   packed_recv_count      [R][El] int32
+ *   cumulative_local_expert_recv_stats [R][El] int32 or NULL; incremented by the counts
+ * Rows at or beyond packed_recv_count are not written.
+ */
+int
+nixl_amd_ep_ll_dispatch(void *packed_recv_x,
+                        void *packed_recv_x_scales,
+                        int *packed_recv_src_info,
+                        int64_t *packed_recv_layout_range,
+                        int *packed_recv_count,
+                        const int *mask_buffer,
+                        int *cumulative_local_expert_recv_stats,
+                        const void *x,
+                        const int32_t *topk_idx,
+                        const int *num_tokens_per_rank,
+                        int num_tokens,
+                        int hidden,
+                        int num_max_dispatch_tokens_per_rank,
+                        int num_topk,
+                        int num_ranks,
+                        int num_experts,
+                        int use_fp8,
+                        int round_scale,
+                        int use_ue8m0,
+                        void *workspace,
+                        size_t workspace_bytes,
+                        void *stream);
+
+/*
+ * Low-latency combine for all ranks.  Replaces ep_kernels::combine (kernels/api.cuh:226-238;
+ * kernel kernels/nixl_ep_ll.cu:618-1017): combined_x[r][t] = bf16( sum over k, in top-k
+ * order, of float(x[row(r,t,k)]) * topk_weights[r][t][k] ) with fused multiply-adds in
+ * fp32, skipping idx < 0 and masked ranks.  row(r,t,k) is located through the dispatch
+ * handle (src_info, layout_range), so any valid permutation inside a segment is accepted.
+ *   x             [R][El][N][H] bf16 (expert outputs in packed_recv_x layout)
+ *   combined_x    [R][T][H] bf16
+ * The LogFMT payload codec of the reference is not implemented: use_logfmt must be 0.
+ */
+int
+nixl_amd_ep_ll_combine(void *combined_x,
+                       const void *x,
+                       const int32_t *topk_idx,
+                       const float *topk_weights,
+                       const int *src_info,
+                       const int64_t *layout_range,
+                       const int *mask_buffer,
+                       const int *num_tokens_per_rank,
+                       int num_tokens,
+                       int hidden,
+                       int num_max_dispatch_tokens_per_rank,
+                       int num_topk,
+                       int num_ranks,
+                       int num_experts,
+                       int use_logfmt,
+                       void *stream);
+
+/*
+ * Token counts per rank and per expert and the token-in-rank matrix, for all source ranks.
+ * Replaces layout::get_dispatch_layout (kernels/api.cuh:63-72; kernels/layout.cu:31-153).
+ *   topk_idx               [R][T][K] int32
+ *   num_tokens_per_rank    [R src][R] int32
+ *   num_tokens_per_expert  [R src][E] int32
+ *   is_token_in_rank       [R src][T][R] bool (1 byte)
+ */
+int
+nixl_amd_ep_get_dispatch_layout(const int32_t *topk_idx,
+                                int *num_tokens_per_rank,
+                                int *num_tokens_per_expert,
+                                uint8_t *is_token_in_rank,
+                                int num_tokens,
+                                int num_topk,
+                                int num_ranks,
+                                int num_experts,
+                                void *stream);
+
+/*
+ * Normal-mode count exchange.  Replaces the arithmetic of ht::notify_dispatch
+ * (kernels/api.cuh:81-113; kernels/nixl_ep_ht.cu:257-314,324-374).
+ *   recv_gbl_rank_prefix_sum [R dst][R src] int32, inclusive over source ranks
+ *   recv_expert_count        [R dst][El] int32, rounded up to expert_alignment
+ *   gbl_channel_prefix_matrix [R src][R dst][C] int32, inclusive over channels; channel c
+ *                            covers tokens [c * ceil(T/C), (c+1) * ceil(T/C))
+ *   send_head                [R src][T][R dst] int32: position of the token inside the
+ *                            (src -> dst) segment, -1 if it does not go there
+ */
+int
+nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
+                               const int *num_tokens_per_expert,
+                               int *recv_gbl_rank_prefix_sum,
+                               int *recv_expert_count,
+                               int *gbl_channel_prefix_matrix,
+                               int *send_head,
+                               int num_tokens,
+                               int num_ranks,
+                               int num_experts,
+                               int num_channels,
+                               int expert_alignment,
+                               void *stream);
+
+/*
+ * Normal-mode dispatch (bf16 rows).  Result contract of ht::dispatch
+ * (kernels/api.cuh:115-160; kernels/nixl_ep_ht.cu:1109-1243): destination d's rows start at
+ * recv_row_offset[d] in the concatenated outputs and are ordered by source rank, then by
+ * source token index; top-k indices are rebased to d's local experts (-1 elsewhere) and
+ * weights of non-local selections are zero.
+ *   recv_row_offset  [R + 1] int64 device array (exclusive prefix of per-destination totals)
+ *   recv_x           [total][H] bf16;  recv_topk_idx [total][K];  recv_topk_weights [total][K]
+ *   recv_src_meta    [total][2] int32 = {source rank, source token}
+ */
+int
+nixl_amd_ep_ht_dispatch(void *recv_x,
+                        int32_t *recv_topk_idx,
+                        float *recv_topk_weights,
+                        int32_t *recv_src_meta,
+                        const void *x,
+                        const int32_t *topk_idx,
+                        const float *topk_weights,
+                        const uint8_t *is_token_in_rank,
+                        const int *recv_gbl_rank_prefix_sum,
+                        const int *send_head,
+                        const int64_t *recv_row_offset,
+                        int num_tokens,
+                        int hidden,
+                        int num_topk,
+                        int num_ranks,
+                        int num_experts,
+                        void *stream);
+
+/*
+ * Normal-mode combine.  Replaces ht::combine with one reduction stage
+ * (kernels/api.cuh:176-203; combine_token, kernels/nixl_ep_ht.cu:1682-1737):
+ * combined_x[r][t] = bf16( float(bias_0) + float(bias_1) + sum over destination ranks that
+ * hold the token, ascending, of float(x[row]) ); no weights are applied to x;
+ * combined_topk_weights[r][t][k] = sum over those ranks of topk_weights[row][k].
+ * bias_0, bias_1, topk_weights and combined_topk_weights may be NULL.
+ */
+int
+nixl_amd_ep_ht_combine(void *combined_x,
+                       float *combined_topk_weights,
+                       const void *x,
+                       const float *topk_weights,
+                       const void *bias_0,
+                       const void *bias_1,
+                       const uint8_t *is_token_in_rank,
+                       const int *recv_gbl_rank_prefix_sum,
+                       const int *send_head,
+                       const int64_t *recv_row_offset,
+                       int num_tokens,
+                       int hidden,
+                       int num_topk,
+                       int num_ranks,
+                       void *stream);
+
+/*
+ * Router: for every token the K largest logits (descending, ties to the lower expert
+ * index) and the softmax over those K logits in fp32.  No counterpart in the reference,
+ * whose callers pass top-k indices in (examples/device/ep/tests/elastic/elastic.py:153-158).
+ *   logits [num_tokens][E] float;  topk_idx [num_tokens][K] int32;  topk_weights float
+ */
+int
+nixl_amd_ep_router_topk(const float *logits,
+                        int32_t *topk_idx,
+                        float *topk_weights,
+                        int num_tokens,
+                        int num_experts,
+                        int num_topk,
+                        void *stream);
+
+/* Element-wise fp32 -> e4m3 codes with the kernels' own encoder (round-to-nearest-even,
+ * saturating); exists so that the encoder can be checked exhaustively. */
+int
+nixl_amd_ep_f32_to_e4m3(const float *in, uint8_t *out, size_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NIXL_AMD_EP_H */

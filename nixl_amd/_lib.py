@@ -77,6 +77,42 @@ def kernels_error():
     return kernels().nixl_amd_last_error().decode()
 
 
+_EP_SIGS = {
+    "nixl_amd_ep_ll_dispatch": [c_void_p] * 10 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p],
+    "nixl_amd_ep_ll_combine": [c_void_p] * 8 + [c_int] * 7 + [c_void_p],
+    "nixl_amd_ep_get_dispatch_layout": [c_void_p] * 4 + [c_int] * 4 + [c_void_p],
+    "nixl_amd_ep_ht_notify_dispatch": [c_void_p] * 6 + [c_int] * 5 + [c_void_p],
+    "nixl_amd_ep_ht_dispatch": [c_void_p] * 11 + [c_int] * 5 + [c_void_p],
+    "nixl_amd_ep_ht_combine": [c_void_p] * 10 + [c_int] * 4 + [c_void_p],
+    "nixl_amd_ep_router_topk": [c_void_p] * 3 + [c_int] * 3 + [c_void_p],
+    "nixl_amd_ep_f32_to_e4m3": [c_void_p, c_void_p, c_size_t, c_void_p],
+}
+
+_ep = None
+
+
+def ep_kernels():
+    """The expert-parallel entry points of libnixl_amd_kernels.so (include/nixl_amd_ep.h)."""
+    global _ep
+    if _ep is not None:
+        return _ep
+    lib = kernels()
+    for name, args in _EP_SIGS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    lib.nixl_amd_ep_ll_workspace_bytes.argtypes = [c_int] * 4
+    lib.nixl_amd_ep_ll_workspace_bytes.restype = c_size_t
+    _ep = lib
+    return lib
+
+
+def kernel_symbols():
+    return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create",
+                   "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
+                   "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
+
+
 # ---------------------------------------------------------------------------------------
 # Agent C API (include/nixl_amd_capi.h)
 # ---------------------------------------------------------------------------------------

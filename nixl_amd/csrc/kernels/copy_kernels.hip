@@ -22,35 +22,14 @@
 // dst[0..len) = src[0..len), the result of the per-descriptor put/get loop at
 // src/plugins/ucx/ucx_backend.cpp:1216-1244.  Descriptors of one request must not
 // overlap each other's destination ranges (the reference's puts are unordered too).
-#include <hip/hip_runtime.h>
-
 #include <algorithm>
-#include <cstdio>
 #include <cstring>
-#include <string>
 #include <vector>
 
-#include "nixl_amd_hip.h"
+#include "common.h"
 
 namespace {
 
-thread_local std::string g_last_error;
-
-int
-fail(int code, const std::string &msg) {
-    g_last_error = msg;
-    return code;
-}
-
-#define HIP_TRY(expr)                                                                      \
-    do {                                                                                   \
-        hipError_t e_ = (expr);                                                            \
-        if (e_ != hipSuccess)                                                              \
-            return fail(NIXL_AMD_ERR_HIP,                                                  \
-                        std::string(#expr) + ": " + hipGetErrorString(e_));                \
-    } while (0)
-
-constexpr int kWaveSize = 64;
 constexpr int kMixedWaves = 4; // waves per workgroup of the mixed and byte-path kernels
 constexpr int kMixedThreads = kWaveSize * kMixedWaves;
 constexpr uint32_t kGenericItemBytes = 16384; // byte-path work item size
@@ -100,18 +79,6 @@ store16(uint64_t addr, const v4u &v) {
         __builtin_nontemporal_store(v, g);
     else
         *g = v;
-}
-
-__device__ __forceinline__ uint32_t
-uniform(uint32_t v) {
-    return __builtin_amdgcn_readfirstlane(v);
-}
-
-__device__ __forceinline__ uint64_t
-uniform64(uint64_t v) {
-    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
-    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-    return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
 // Workgroups are handed to the 8 dies round-robin.  With the swizzle on, die x works
@@ -329,29 +296,16 @@ struct nixl_amd_copy_plan {
 
 extern "C" {
 
-const char *
-nixl_amd_last_error(void) {
-    return g_last_error.c_str();
-}
-
-int
-nixl_amd_device_count(void) {
-    int n = 0;
-    hipError_t e = hipGetDeviceCount(&n);
-    if (e != hipSuccess) return fail(NIXL_AMD_ERR_NO_DEVICE, hipGetErrorString(e));
-    return n;
-}
-
 int
 nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
                           size_t n,
                           int device,
                           const nixl_amd_copy_tuning_t *tuning,
                           nixl_amd_copy_plan_t **out) {
-    if (!out) return fail(NIXL_AMD_ERR_INVALID, "plan_create: out is null");
+    if (!out) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: out is null");
     *out = nullptr;
-    if (!descs && n) return fail(NIXL_AMD_ERR_INVALID, "plan_create: descs is null");
-    if (n >= (1ull << 32)) return fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: more than 2^32-1 descriptors");
+    if (!descs && n) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: descs is null");
+    if (n >= (1ull << 32)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: more than 2^32-1 descriptors");
 
     // Defaults from a sweep on MI355X: the smallest chunk (one 128-bit load and store per
     // lane, one wave per workgroup) with non-temporal accesses gave the highest HBM rate.
@@ -365,15 +319,15 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         if (tuning->xcd_swizzle) swizzle = tuning->xcd_swizzle == 1 ? 1 : 0;
     }
     if (upl != 1 && upl != 2 && upl != 4 && upl != 8 && upl != 16)
-        return fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 1, 2, 4, 8 or 16");
-    if (nt != 1 && nt != 2) return fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0, 1 or 2");
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 1, 2, 4, 8 or 16");
+    if (nt != 1 && nt != 2) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0, 1 or 2");
     if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16)
-        return fail(NIXL_AMD_ERR_INVALID, "plan_create: waves_per_workgroup must be 1, 2, 4, 8 or 16");
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: waves_per_workgroup must be 1, 2, 4, 8 or 16");
 
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
-        return fail(NIXL_AMD_ERR_NO_DEVICE, "plan_create: no HIP device");
-    if (device < 0 || device >= ndev) return fail(NIXL_AMD_ERR_INVALID, "plan_create: bad device index");
+        return nixl_amd_fail(NIXL_AMD_ERR_NO_DEVICE, "plan_create: no HIP device");
+    if (device < 0 || device >= ndev) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: bad device index");
     HIP_TRY(hipSetDevice(device));
 
     // ---- host-side lowering ------------------------------------------------------
@@ -387,9 +341,9 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         const nixl_amd_copy_desc_t &d = descs[i];
         if (d.len == 0) continue;
         if (d.src == 0 || d.dst == 0)
-            return fail(NIXL_AMD_ERR_INVALID, "plan_create: null address in descriptor " + std::to_string(i));
+            return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: null address in descriptor " + std::to_string(i));
         if (d.src + d.len < d.src || d.dst + d.len < d.dst)
-            return fail(NIXL_AMD_ERR_INVALID, "plan_create: address range wraps in descriptor " + std::to_string(i));
+            return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: address range wraps in descriptor " + std::to_string(i));
         payload += d.len;
         if (((d.src | d.dst | d.len) & 15u) == 0) {
             vsrc.push_back(d.src);
@@ -412,7 +366,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     const uint64_t chunk_units = static_cast<uint64_t>(kWaveSize) * upl;
     const uint64_t n_chunks64 = (units + chunk_units - 1) / chunk_units;
     if (n_chunks64 >= (1ull << 32) || items.size() >= (1ull << 32))
-        return fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: request too large for 32-bit chunk index");
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: request too large for 32-bit chunk index");
     const uint32_t n_chunks = static_cast<uint32_t>(n_chunks64);
 
     std::vector<uint2> span(n_chunks);
@@ -474,13 +428,13 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         hipError_t e = hipMalloc(&plan->arena, total);
         if (e != hipSuccess) {
             delete plan;
-            return fail(NIXL_AMD_ERR_HIP, std::string("hipMalloc(plan arena): ") + hipGetErrorString(e));
+            return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipMalloc(plan arena): ") + hipGetErrorString(e));
         }
         e = hipMemcpy(plan->arena, host.data(), total, hipMemcpyHostToDevice);
         if (e != hipSuccess) {
             (void)hipFree(plan->arena);
             delete plan;
-            return fail(NIXL_AMD_ERR_HIP, std::string("hipMemcpy(plan arena): ") + hipGetErrorString(e));
+            return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipMemcpy(plan arena): ") + hipGetErrorString(e));
         }
         plan->arena_bytes = total;
         auto *base = static_cast<uint8_t *>(plan->arena);
@@ -522,7 +476,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
 
 int
 nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
-    if (!plan) return fail(NIXL_AMD_ERR_INVALID, "plan_launch: plan is null");
+    if (!plan) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_launch: plan is null");
     HIP_TRY(hipSetDevice(plan->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (plan->uniform_wgs) {
@@ -561,13 +515,13 @@ nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan) {
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     hipError_t e = plan->arena ? hipFree(plan->arena) : hipSuccess;
     delete plan;
-    if (e != hipSuccess) return fail(NIXL_AMD_ERR_HIP, std::string("hipFree(plan arena): ") + hipGetErrorString(e));
+    if (e != hipSuccess) return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipFree(plan arena): ") + hipGetErrorString(e));
     return NIXL_AMD_OK;
 }
 
 int
 nixl_amd_copy_plan_query(const nixl_amd_copy_plan_t *plan, nixl_amd_copy_plan_info_t *info) {
-    if (!plan || !info) return fail(NIXL_AMD_ERR_INVALID, "plan_query: null argument");
+    if (!plan || !info) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_query: null argument");
     *info = plan->info;
     return NIXL_AMD_OK;
 }
@@ -575,7 +529,7 @@ nixl_amd_copy_plan_query(const nixl_amd_copy_plan_t *plan, nixl_amd_copy_plan_in
 int
 nixl_amd_copy_plan_time(nixl_amd_copy_plan_t *plan, void *stream, int iters, float *ms_per_launch) {
     if (!plan || !ms_per_launch || iters <= 0)
-        return fail(NIXL_AMD_ERR_INVALID, "plan_time: bad argument");
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_time: bad argument");
     HIP_TRY(hipSetDevice(plan->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (!plan->ev0) HIP_TRY(hipEventCreate(&plan->ev0));

@@ -1,0 +1,479 @@
+// Normal-mode ("high-throughput") expert-parallel kernels and the router, for all virtual
+// ranks of one GPU, with their C ABI (declared in include/nixl_amd_ep.h).
+//
+// The reference streams token rows through RDMA and NVLink ring queues, forwarding them hop
+// by hop (kernels/nixl_ep_ht.cu:472-1245).  None of that exists when every rank is a region
+// of the same HBM; what remains is the result: destination rows ordered by source rank then
+// source token, rebased top-k indices, and the unweighted fp32 reduction on the way back.
+// Positions come from prefix sums instead of queue heads:
+//   row(r, t, d) = recv_row_offset[d] + recv_rank_prefix[d][r - 1] + send_head[r][t][d].
+//
+// HBM traffic: dispatch reads every source row once (2H) and writes it once per destination
+// rank that holds one of its experts; combine reads those rows once and writes 2H per token.
+#include <cstdint>
+
+#include "common.h"
+#include "ep_common.h"
+#include "nixl_amd_ep.h"
+
+namespace {
+
+constexpr int kScanThreads = 1024;
+
+// Exclusive prefix of `v` over the workgroup (blockDim.x == kScanThreads); `total` gets the sum.
+__device__ __forceinline__ int
+block_exclusive_scan(int v, int *wave_sums, int &total) {
+    const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+    }
+    __syncthreads(); // wave_sums may still be read from a previous call
+    if (lane == kWaveSize - 1) wave_sums[wave] = incl;
+    __syncthreads();
+    constexpr int kWaves = kScanThreads / kWaveSize;
+    int before = 0, sum = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        const int s = wave_sums[w];
+        if (w < wave) before += s;
+        sum += s;
+    }
+    total = sum;
+    return before + incl - v;
+}
+
+// ---- layout (kernels/layout.cu:31-138) ----------------------------------------------------
+// grid = R source ranks; LDS: E + R counters.
+__global__ void __launch_bounds__(kScanThreads)
+layout_kernel(const int32_t *__restrict__ topk_idx,
+              int *__restrict__ per_rank,
+              int *__restrict__ per_expert,
+              uint8_t *__restrict__ in_rank,
+              int T,
+              int K,
+              int R,
+              int E) {
+    extern __shared__ int counters[]; // [E] experts, then [R] ranks
+    const int src = blockIdx.x, El = E / R;
+    for (int i = threadIdx.x; i < E + R; i += blockDim.x)
+        counters[i] = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < T; t += blockDim.x) {
+        const int32_t *sel = topk_idx + (static_cast<size_t>(src) * T + t) * K;
+        uint8_t *flags = in_rank + (static_cast<size_t>(src) * T + t) * R;
+        for (int d = 0; d < R; ++d)
+            flags[d] = 0;
+        for (int k = 0; k < K; ++k) {
+            const int e = sel[k];
+            if (e < 0 || e >= E) continue;
+            atomicAdd(&counters[e], 1);
+            flags[e / El] = 1;
+        }
+        for (int d = 0; d < R; ++d)
+            if (flags[d]) atomicAdd(&counters[E + d], 1);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < E; i += blockDim.x)
+        per_expert[static_cast<size_t>(src) * E + i] = counters[i];
+    for (int i = threadIdx.x; i < R; i += blockDim.x)
+        per_rank[static_cast<size_t>(src) * R + i] = counters[E + i];
+}
+
+// ---- notify, part 1: per source rank, positions inside each (src -> dst) segment and the
+// per-channel prefix (kernels/nixl_ep_ht.cu:324-373) ----------------------------------------
+__global__ void __launch_bounds__(kScanThreads)
+ht_scan_kernel(const uint8_t *__restrict__ in_rank,
+               int *__restrict__ send_head,
+               int *__restrict__ channel_prefix,
+               int T,
+               int R,
+               int C) {
+    __shared__ int wave_sums[kScanThreads / kWaveSize];
+    const int src = blockIdx.x;
+    const int per_thread = (T + kScanThreads - 1) / kScanThreads;
+    const int t0 = min(static_cast<int>(threadIdx.x) * per_thread, T), t1 = min(t0 + per_thread, T);
+    const int per_channel = (T + C - 1) / C;
+    for (int d = 0; d < R; ++d) {
+        int mine = 0;
+        for (int t = t0; t < t1; ++t)
+            mine += in_rank[(static_cast<size_t>(src) * T + t) * R + d];
+        int total;
+        int pos = block_exclusive_scan(mine, wave_sums, total);
+        for (int t = t0; t < t1; ++t) {
+            const bool hit = in_rank[(static_cast<size_t>(src) * T + t) * R + d] != 0;
+            send_head[(static_cast<size_t>(src) * T + t) * R + d] = hit ? pos : -1;
+            pos += hit;
+            // `pos` is now the number of hits in tokens [0, t]; a channel's inclusive prefix
+            // is that number at the channel's last token.
+            if ((t + 1) % per_channel == 0 || t + 1 == T) {
+                const int c = t / per_channel;
+                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = pos;
+            }
+        }
+        // channels that start at or beyond T are empty: they repeat the grand total
+        if (threadIdx.x == 0)
+            for (int c = (T + per_channel - 1) / per_channel; c < C; ++c)
+                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = total;
+    }
+}
+
+// ---- notify, part 2: receive-side prefix over source ranks and aligned per-expert counts
+// (kernels/nixl_ep_ht.cu:295-314) -------------------------------------------------------------
+__global__ void
+ht_prefix_kernel(const int *__restrict__ channel_prefix,
+                 const int *__restrict__ per_expert,
+                 int *__restrict__ recv_rank_prefix,
+                 int *__restrict__ recv_expert_count,
+                 int R,
+                 int E,
+                 int C,
+                 int alignment) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < R) {
+        const int d = i;
+        int sum = 0;
+        for (int r = 0; r < R; ++r) {
+            sum += channel_prefix[(static_cast<size_t>(r) * R + d) * C + (C - 1)];
+            recv_rank_prefix[d * R + r] = sum;
+        }
+    }
+    if (i < E) {
+        int n = 0;
+        for (int r = 0; r < R; ++r)
+            n += per_expert[static_cast<size_t>(r) * E + i];
+        recv_expert_count[i] = (n + alignment - 1) / alignment * alignment;
+    }
+}
+
+struct HtDims {
+    int R, T, H, K, E;
+};
+
+__device__ __forceinline__ long long
+recv_row(const int *prefix, const int *send_head, const long long *row_offset, const HtDims &d, int r, int t, int dst) {
+    const int seg = r == 0 ? 0 : prefix[dst * d.R + r - 1];
+    return row_offset[dst] + seg + send_head[(static_cast<size_t>(r) * d.T + t) * d.R + dst];
+}
+
+// ---- dispatch (result of kernels/nixl_ep_ht.cu:1109-1243) -------------------------------------
+// grid = R*T; block = H/8 lanes rounded up to whole waves (16 bytes of a row per lane).
+__global__ void __launch_bounds__(1024)
+ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
+                   int32_t *__restrict__ recv_topk_idx,
+                   float *__restrict__ recv_topk_weights,
+                   int32_t *__restrict__ recv_src_meta,
+                   const uint16_t *__restrict__ x,
+                   const int32_t *__restrict__ topk_idx,
+                   const float *__restrict__ topk_weights,
+                   const uint8_t *__restrict__ in_rank,
+                   const int *__restrict__ prefix,
+                   const int *__restrict__ send_head,
+                   const long long *__restrict__ row_offset,
+                   HtDims d) {
+    const int tid = threadIdx.x;
+    const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
+    const size_t tok = static_cast<size_t>(r) * d.T + t;
+    const int El = d.E / d.R;
+    const bool active = tid < d.H / 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (active) v = ld16_nt(reinterpret_cast<const uint4 *>(x + tok * d.H) + tid);
+    int sel = -1;
+    float w = 0.f;
+    if (tid < d.K && topk_idx) {
+        sel = topk_idx[tok * d.K + tid];
+        w = topk_weights ? topk_weights[tok * d.K + tid] : 0.f;
+    }
+    for (int dst = 0; dst < d.R; ++dst) {
+        if (!in_rank[tok * d.R + dst]) continue; // uniform over the workgroup
+        const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+        if (active) st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(row) * d.H) + tid, v);
+        if (tid < d.K && recv_topk_idx) {
+            const bool local = sel >= dst * El && sel < (dst + 1) * El;
+            recv_topk_idx[row * d.K + tid] = local ? sel - dst * El : -1;
+            if (recv_topk_weights) recv_topk_weights[row * d.K + tid] = local ? w : 0.f;
+        }
+        if (tid == 0 && recv_src_meta) {
+            recv_src_meta[row * 2] = r;
+            recv_src_meta[row * 2 + 1] = t;
+        }
+    }
+}
+
+// ---- combine (combine_token, kernels/nixl_ep_ht.cu:1682-1737) -----------------------------------
+__global__ void __launch_bounds__(1024)
+ht_combine_kernel(uint16_t *__restrict__ combined,
+                  float *__restrict__ combined_w,
+                  const uint16_t *__restrict__ x,
+                  const float *__restrict__ topk_weights,
+                  const uint16_t *__restrict__ bias0,
+                  const uint16_t *__restrict__ bias1,
+                  const uint8_t *__restrict__ in_rank,
+                  const int *__restrict__ prefix,
+                  const int *__restrict__ send_head,
+                  const long long *__restrict__ row_offset,
+                  HtDims d) {
+    const int tid = threadIdx.x;
+    const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
+    const size_t tok = static_cast<size_t>(r) * d.T + t;
+    const bool active = tid < d.H / 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (active) {
+        uint4 b0 = make_uint4(0, 0, 0, 0), b1 = b0;
+        if (bias0) b0 = ld16_nt(reinterpret_cast<const uint4 *>(bias0 + tok * d.H) + tid);
+        if (bias1) b1 = ld16_nt(reinterpret_cast<const uint4 *>(bias1 + tok * d.H) + tid);
+        const uint32_t u0[4] = {b0.x, b0.y, b0.z, b0.w}, u1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            acc[2 * c] = bf16_lo_to_f32(u0[c]) + bf16_lo_to_f32(u1[c]);
+            acc[2 * c + 1] = bf16_hi_to_f32(u0[c]) + bf16_hi_to_f32(u1[c]);
+        }
+    }
+    float wsum = 0.f;
+    for (int dst = 0; dst < d.R; ++dst) {
+        if (!in_rank[tok * d.R + dst]) continue;
+        const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+        if (active) {
+            const uint4 v = ld16_nt(reinterpret_cast<const uint4 *>(x + static_cast<size_t>(row) * d.H) + tid);
+            const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                acc[2 * c] += bf16_lo_to_f32(u[c]);
+                acc[2 * c + 1] += bf16_hi_to_f32(u[c]);
+            }
+        }
+        if (topk_weights && tid < d.K) wsum += topk_weights[row * d.K + tid];
+    }
+    if (active) {
+        uint4 out;
+        out.x = f32_to_bf16(acc[0]) | (f32_to_bf16(acc[1]) << 16);
+        out.y = f32_to_bf16(acc[2]) | (f32_to_bf16(acc[3]) << 16);
+        out.z = f32_to_bf16(acc[4]) | (f32_to_bf16(acc[5]) << 16);
+        out.w = f32_to_bf16(acc[6]) | (f32_to_bf16(acc[7]) << 16);
+        st16_nt(reinterpret_cast<uint4 *>(combined + tok * d.H) + tid, out);
+    }
+    if (combined_w && tid < d.K) combined_w[tok * d.K + tid] = wsum;
+}
+
+// ---- router -----------------------------------------------------------------------------------------
+// One wave per token; lane l holds experts l, l + 64, ...  K rounds of a wave-wide argmax
+// (larger value wins, equal values go to the lower expert index).
+constexpr int kRouterMaxPerLane = 16; // E <= 1024
+
+__global__ void __launch_bounds__(256)
+router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, float *__restrict__ topk_w, int n_tokens, int E, int K) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int token = blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
+    if (token >= n_tokens) return;
+    float v[kRouterMaxPerLane];
+    unsigned taken = 0;
+#pragma unroll
+    for (int j = 0; j < kRouterMaxPerLane; ++j) {
+        const int e = j * kWaveSize + lane;
+        v[j] = e < E ? logits[static_cast<size_t>(token) * E + e] : 0.f;
+        if (e >= E) taken |= 1u << j;
+    }
+    float sel_v[16];
+    int sel_i[16];
+    for (int k = 0; k < K; ++k) {
+        float best = 0.f;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < kRouterMaxPerLane; ++j) {
+            const int e = j * kWaveSize + lane;
+            if (!((taken >> j) & 1u) && (best_e == 0x7fffffff || v[j] > best)) {
+                best = v[j];
+                best_e = e;
+            }
+        }
+#pragma unroll
+        for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(best, off);
+            const int oe = __shfl_xor(best_e, off);
+            const bool mine_valid = best_e != 0x7fffffff, other_valid = oe != 0x7fffffff;
+            if (other_valid && (!mine_valid || ov > best || (ov == best && oe < best_e))) {
+                best = ov;
+                best_e = oe;
+            }
+        }
+        if ((best_e & (kWaveSize - 1)) == lane) taken |= 1u << (best_e / kWaveSize);
+        sel_v[k] = best;
+        sel_i[k] = best_e;
+    }
+    if (lane == 0) {
+        const float top = sel_v[0];
+        float ex[16], sum = 0.f;
+        for (int k = 0; k < K; ++k) {
+            ex[k] = expf(sel_v[k] - top);
+            sum += ex[k];
+        }
+        for (int k = 0; k < K; ++k) {
+            topk_idx[static_cast<size_t>(token) * K + k] = sel_i[k];
+            topk_w[static_cast<size_t>(token) * K + k] = ex[k] / sum;
+        }
+    }
+}
+
+int
+round_up_wave(int n) {
+    return (n + kWaveSize - 1) / kWaveSize * kWaveSize;
+}
+
+int
+check_ht(const char *who, int T, int H, int K, int R, int E) {
+    auto bad = [&](const std::string &why) { return nixl_amd_fail(NIXL_AMD_ERR_INVALID, std::string(who) + ": " + why); };
+    if (R <= 0 || R > 1024) return bad("num_ranks must be in [1, 1024]");
+    if (E <= 0 || E % R != 0) return bad("num_experts must be a positive multiple of num_ranks");
+    if (T <= 0) return bad("num_tokens must be positive");
+    if (K < 0 || K > 16) return bad("num_topk must be at most 16");
+    if (H % 8 != 0 || H < 0 || H > 8192) return bad("hidden must be a multiple of 8, at most 8192");
+    if (static_cast<long long>(R) * T > (1ll << 30)) return bad("num_ranks * num_tokens too large");
+    return NIXL_AMD_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int
+nixl_amd_ep_get_dispatch_layout(const int32_t *topk_idx,
+                                int *num_tokens_per_rank,
+                                int *num_tokens_per_expert,
+                                uint8_t *is_token_in_rank,
+                                int num_tokens,
+                                int num_topk,
+                                int num_ranks,
+                                int num_experts,
+                                void *stream) {
+    const int rc = check_ht("get_dispatch_layout", num_tokens, 0, num_topk, num_ranks, num_experts);
+    if (rc) return rc;
+    if (!topk_idx || !num_tokens_per_rank || !num_tokens_per_expert || !is_token_in_rank)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "get_dispatch_layout: null pointer argument");
+    const size_t lds = static_cast<size_t>(num_experts + num_ranks) * sizeof(int);
+    if (lds > 48 * 1024) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "get_dispatch_layout: too many experts");
+    hipLaunchKernelGGL(layout_kernel, dim3(num_ranks), dim3(kScanThreads), lds, static_cast<hipStream_t>(stream), topk_idx,
+                       num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk, num_ranks,
+                       num_experts);
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
+                               const int *num_tokens_per_expert,
+                               int *recv_gbl_rank_prefix_sum,
+                               int *recv_expert_count,
+                               int *gbl_channel_prefix_matrix,
+                               int *send_head,
+                               int num_tokens,
+                               int num_ranks,
+                               int num_experts,
+                               int num_channels,
+                               int expert_alignment,
+                               void *stream) {
+    const int rc = check_ht("ht_notify_dispatch", num_tokens, 0, 0, num_ranks, num_experts);
+    if (rc) return rc;
+    if (num_channels <= 0 || expert_alignment <= 0)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_notify_dispatch: num_channels and expert_alignment must be positive");
+    if (!is_token_in_rank || !num_tokens_per_expert || !recv_gbl_rank_prefix_sum || !recv_expert_count ||
+        !gbl_channel_prefix_matrix || !send_head)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_notify_dispatch: null pointer argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(ht_scan_kernel, dim3(num_ranks), dim3(kScanThreads), 0, s, is_token_in_rank, send_head,
+                       gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
+    HIP_TRY(hipGetLastError());
+    const int n = num_experts > num_ranks ? num_experts : num_ranks;
+    hipLaunchKernelGGL(ht_prefix_kernel, dim3((n + 255) / 256), dim3(256), 0, s, gbl_channel_prefix_matrix,
+                       num_tokens_per_expert, recv_gbl_rank_prefix_sum, recv_expert_count, num_ranks, num_experts,
+                       num_channels, expert_alignment);
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_ht_dispatch(void *recv_x,
+                        int32_t *recv_topk_idx,
+                        float *recv_topk_weights,
+                        int32_t *recv_src_meta,
+                        const void *x,
+                        const int32_t *topk_idx,
+                        const float *topk_weights,
+                        const uint8_t *is_token_in_rank,
+                        const int *recv_gbl_rank_prefix_sum,
+                        const int *send_head,
+                        const int64_t *recv_row_offset,
+                        int num_tokens,
+                        int hidden,
+                        int num_topk,
+                        int num_ranks,
+                        int num_experts,
+                        void *stream) {
+    const int rc = check_ht("ht_dispatch", num_tokens, hidden, num_topk, num_ranks, num_experts);
+    if (rc) return rc;
+    if (hidden == 0) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: hidden must be positive");
+    if (!recv_x || !x || !is_token_in_rank || !recv_gbl_rank_prefix_sum || !send_head || !recv_row_offset)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: null pointer argument");
+    if (recv_topk_idx && !topk_idx) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: recv_topk_idx without topk_idx");
+    const HtDims d{num_ranks, num_tokens, hidden, num_topk, num_experts};
+    hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens), dim3(round_up_wave(hidden / 8)),
+                       0, static_cast<hipStream_t>(stream), static_cast<uint16_t *>(recv_x), recv_topk_idx, recv_topk_weights,
+                       recv_src_meta, static_cast<const uint16_t *>(x), topk_idx, topk_weights, is_token_in_rank,
+                       recv_gbl_rank_prefix_sum, send_head, reinterpret_cast<const long long *>(recv_row_offset), d);
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_ht_combine(void *combined_x,
+                       float *combined_topk_weights,
+                       const void *x,
+                       const float *topk_weights,
+                       const void *bias_0,
+                       const void *bias_1,
+                       const uint8_t *is_token_in_rank,
+                       const int *recv_gbl_rank_prefix_sum,
+                       const int *send_head,
+                       const int64_t *recv_row_offset,
+                       int num_tokens,
+                       int hidden,
+                       int num_topk,
+                       int num_ranks,
+                       void *stream) {
+    const int rc = check_ht("ht_combine", num_tokens, hidden, num_topk, num_ranks, num_ranks);
+    if (rc) return rc;
+    if (hidden == 0) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_combine: hidden must be positive");
+    if (!combined_x || !x || !is_token_in_rank || !recv_gbl_rank_prefix_sum || !send_head || !recv_row_offset)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_combine: null pointer argument");
+    const HtDims d{num_ranks, num_tokens, hidden, num_topk, num_ranks};
+    hipLaunchKernelGGL(ht_combine_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens), dim3(round_up_wave(hidden / 8)),
+                       0, static_cast<hipStream_t>(stream), static_cast<uint16_t *>(combined_x), combined_topk_weights,
+                       static_cast<const uint16_t *>(x), topk_weights, static_cast<const uint16_t *>(bias_0),
+                       static_cast<const uint16_t *>(bias_1), is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                       reinterpret_cast<const long long *>(recv_row_offset), d);
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_router_topk(const float *logits,
+                        int32_t *topk_idx,
+                        float *topk_weights,
+                        int num_tokens,
+                        int num_experts,
+                        int num_topk,
+                        void *stream) {
+    if (!logits || !topk_idx || !topk_weights) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "router_topk: null pointer argument");
+    if (num_tokens < 0 || num_experts <= 0 || num_experts > kRouterMaxPerLane * kWaveSize)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "router_topk: num_experts must be in [1, 1024]");
+    if (num_topk <= 0 || num_topk > 16 || num_topk > num_experts)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "router_topk: num_topk must be in [1, min(16, num_experts)]");
+    if (num_tokens == 0) return NIXL_AMD_OK;
+    hipLaunchKernelGGL(router_kernel, dim3((num_tokens + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), logits,
+                       topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+} // extern "C"

@@ -310,6 +310,21 @@ oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const flo
     return 0;
 }
 
+/* The reduction of one token on explicit rows: out = bf16(sum_k float(rows[k]) * w[k]) in
+ * top-k order, fused (use_fma) or as separate multiply and add.  Lets a test check single
+ * tokens of a large run without building the whole world on the CPU. */
+void
+oracle_weighted_sum_rows(const uint16_t *rows, const float *w, int K, int H, int use_fma, uint16_t *out) {
+    for (int h = 0; h < H; ++h) {
+        float acc = 0.0f;
+        for (int k = 0; k < K; ++k) {
+            const float v = oracle_bf16_to_f32(rows[(size_t)k * H + h]);
+            acc = use_fma ? fmaf(v, w[k], acc) : acc + v * w[k];
+        }
+        out[h] = oracle_f32_to_bf16(acc);
+    }
+}
+
 /* ---- normal mode ----------------------------------------------------------------------- */
 
 /* kernels/layout.cu:31-138: tokens per expert, tokens per rank (a token counts once per

@@ -49,6 +49,8 @@ int oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const
                       const int32_t *mask, int R, int T, int H, int K, int E, int M, int use_fma,
                       uint16_t *combined, int threads);
 
+void oracle_weighted_sum_rows(const uint16_t *rows, const float *w, int K, int H, int use_fma, uint16_t *out);
+
 /* normal (high-throughput) mode */
 void oracle_dispatch_layout(const int32_t *topk_idx, int T, int K, int R, int E, int32_t *num_tokens_per_rank,
                             int32_t *num_tokens_per_expert, uint8_t *is_token_in_rank);

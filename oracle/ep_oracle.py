@@ -36,6 +36,7 @@ def lib():
         L.oracle_ll_dispatch.restype = _I
         L.oracle_ll_combine.argtypes = [_P] * 7 + [_I] * 7 + [_P, _I]
         L.oracle_ll_combine.restype = _I
+        L.oracle_weighted_sum_rows.argtypes = [_P, _P, _I, _I, _I, _P]
         L.oracle_dispatch_layout.argtypes = [_P, _I, _I, _I, _I, _P, _P, _P]
         L.oracle_ht_notify.argtypes = [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P]
         L.oracle_ht_dispatch.argtypes = [_P] * 5 + [_I] * 5 + [_P] * 7
@@ -137,6 +138,15 @@ def ll_combine(expert_out, topk_idx, topk_weights, src_info, layout_range, num_e
                                  _p(nt), _p(mk), R, T, H, K, num_experts, max_tok, int(use_fma), _p(out), threads)
     if rc != 0:
         raise ValueError(f"oracle_ll_combine rejected the arguments ({rc})")
+    return out
+
+
+def weighted_sum_rows(rows, weights, use_fma=True):
+    """rows [K,H] bf16 bits, weights [K] -> bf16 bits [H] of sum_k rows[k] * weights[k]."""
+    rows = _c(rows, np.uint16)
+    weights = _c(weights, np.float32)
+    out = np.zeros(rows.shape[1], np.uint16)
+    lib().oracle_weighted_sum_rows(_p(rows), _p(weights), rows.shape[0], rows.shape[1], int(use_fma), _p(out))
     return out
 
 

@@ -1,0 +1,511 @@
+"""GPU parity tests for the expert-parallel half: the HIP kernels through their C ABI
+(include/nixl_amd_ep.h) and through the host-side Buffer, against the CPU oracle on seeded
+inputs, on the reference tests' own data pattern, and through size-independent properties
+at the full BASELINE sizes."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ep_oracle as eo
+from nixl_amd import _lib
+from nixl_amd.ep import Buffer, EPError
+
+pytestmark = pytest.mark.gpu
+
+
+def bits16(t):
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def calc_diff(x, y):
+    # examples/device/ep/tests/utils.py:63-67
+    x, y = x.double() + 1, y.double() + 1
+    return float(1 - 2 * (x * y).sum() / (x * x + y * y).sum())
+
+
+def make_world(seed, R, T, H, K, E, drop=0.1, scale=1.0):
+    rng = np.random.default_rng(seed)
+    x = torch.from_numpy(rng.standard_normal((R, T, H)).astype(np.float32) * scale).to(torch.bfloat16)
+    scores = rng.standard_normal((R, T, E))
+    topk = np.argsort(-scores, axis=2)[:, :, :K].astype(np.int32)
+    topk[rng.random((R, T, K)) < drop] = -1
+    w = np.abs(rng.standard_normal((R, T, K))).astype(np.float32)
+    return x, topk, w
+
+
+def raw_ll_dispatch(cuda, x, topk, E, M, use_fp8, round_scale=False, use_ue8m0=False, num_tokens=None, mask=None,
+                    stats=None, fill=0x55):
+    """Call the C ABI directly on buffers pre-filled with `fill`."""
+    k = _lib.ep_kernels()
+    R, T, H = x.shape
+    K = topk.shape[2]
+    El, N = E // R, R * M
+    dev = lambda a, dt: None if a is None else torch.from_numpy(np.ascontiguousarray(a, dtype=dt)).to(cuda)
+    xd = x.to(cuda)
+    td = dev(topk, np.int32)
+    ntd, md = dev(num_tokens, np.int32), dev(mask, np.int32)
+    recv_x = torch.full((R, El, N, H * (1 if use_fp8 else 2)), fill, dtype=torch.uint8, device=cuda)
+    scales = None
+    if use_fp8:
+        scales = torch.full((R, El, (H // 512 if use_ue8m0 else H // 128), N, 4), fill, dtype=torch.uint8, device=cuda)
+    src_info = torch.full((R, El, N, 4), fill, dtype=torch.uint8, device=cuda)
+    layout = torch.zeros((R, El, R), dtype=torch.int64, device=cuda)
+    count = torch.zeros((R, El), dtype=torch.int32, device=cuda)
+    ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K) + 16, dtype=torch.uint8, device=cuda)
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    rc = k.nixl_amd_ep_ll_dispatch(p(recv_x), p(scales), p(src_info), p(layout), p(count), p(md), p(stats), p(xd), p(td),
+                                   p(ntd), T, H, M, K, R, E, int(use_fp8), int(round_scale), int(use_ue8m0), p(ws),
+                                   ws.numel(), None)
+    torch.cuda.synchronize()
+    return rc, dict(recv_x=recv_x.cpu().numpy(), scales=None if scales is None else scales.cpu().numpy(),
+                    src_info=src_info.cpu().numpy(), layout_range=layout.cpu().numpy(), recv_count=count.cpu().numpy())
+
+
+def assert_dispatch_equal(got, want, use_fp8, use_ue8m0=False, fill=0x55):
+    assert np.array_equal(got["recv_count"], want["recv_count"])
+    assert np.array_equal(got["layout_range"], want["layout_range"])
+    R, El = want["recv_count"].shape
+    wx = want["recv_x"].view(np.uint8).reshape(got["recv_x"].shape)
+    wsi = want["src_info"].view(np.uint8).reshape(got["src_info"].shape)
+    assert np.array_equal(got["recv_x"], wx)  # includes: rows past recv_count keep the fill byte
+    assert np.array_equal(got["src_info"], wsi)
+    if use_fp8:
+        ws = want["scales"].view(np.uint8).reshape(got["scales"].shape)
+        assert np.array_equal(got["scales"], ws)
+
+
+# ---- encoder -------------------------------------------------------------------------------------
+
+def test_fp8_encoder_exhaustive(cuda):
+    codes = np.arange(65536, dtype=np.uint16)
+    x = eo.bf16_to_f32(codes)
+    rng = np.random.default_rng(1)
+    amax = np.concatenate([[1e-4, 1.0, 3.0, 448.0, 0.37], np.abs(rng.standard_normal(27)) * 4 + 1e-3]).astype(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        v = (x[None, :] * (np.float32(448.0) / amax)[:, None]).astype(np.float32).reshape(-1)
+    extra = np.array([np.inf, -np.inf, np.nan, -np.nan, 448.0, 463.9, 464.0, 1e30, 2.0 ** -10, 3 * 2.0 ** -10, 2.0 ** -9 * 7.5],
+                     np.float32)
+    rnd = rng.integers(0, 2 ** 32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    v = np.concatenate([v, extra, rnd])
+    vin = torch.from_numpy(v).to(cuda)
+    out = torch.empty(v.size, dtype=torch.uint8, device=cuda)
+    rc = _lib.ep_kernels().nixl_amd_ep_f32_to_e4m3(ctypes.c_void_p(vin.data_ptr()), ctypes.c_void_p(out.data_ptr()), v.size, None)
+    assert rc == 0, _lib.kernels_error()
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), eo.f32_to_e4m3(v))
+
+
+# ---- low-latency dispatch ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("use_fp8,round_scale,use_ue8m0", [(False, False, False), (True, False, False), (True, True, False), (True, True, True)])
+@pytest.mark.parametrize("shape", [(4, 12, 512, 3, 8, 16), (2, 130, 1024, 8, 64, 130), (8, 5, 2560, 4, 16, 8)])
+def test_ll_dispatch_matches_oracle(cuda, shape, use_fp8, round_scale, use_ue8m0):
+    R, T, H, K, E, M = shape
+    if use_fp8 and H % 512:
+        pytest.skip("fp8 needs hidden % 512 == 0")
+    x, topk, _ = make_world(hash(shape) % 1000 + use_fp8, R, T, H, K, E, scale=3.0)
+    nt = np.full(R, T, np.int32)
+    nt[1] = T // 2
+    nt[-1] = 0
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, use_fp8, round_scale, use_ue8m0, num_tokens=nt)
+    assert rc == 0, _lib.kernels_error()
+    want = eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, use_fp8, round_scale, use_ue8m0, num_tokens=nt, fill=0x55)
+    assert_dispatch_equal(got, want, use_fp8, use_ue8m0)
+
+
+def test_ll_dispatch_extreme_values(cuda):
+    # zeros (amax floor 1e-4), huge and tiny magnitudes, a constant row, negative zero
+    R, T, H, K, E, M = 2, 8, 512, 2, 4, 8
+    x, topk, _ = make_world(7, R, T, H, K, E, drop=0.0)
+    x[0, 0] = 0
+    x[0, 1] = 3.0e38
+    x[0, 2] = 1.0e-38
+    x[0, 3] = -0.0
+    x[0, 4] = 1.0
+    x[1, 0, ::2] = 1.0e-5
+    x[1, 1] = torch.arange(H).to(torch.bfloat16) - 256
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, True)
+    assert rc == 0
+    assert_dispatch_equal(got, eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, True, fill=0x55), True)
+
+
+def test_ll_dispatch_mask_and_stats(cuda):
+    R, T, H, K, E, M = 4, 16, 512, 4, 16, 16
+    x, topk, _ = make_world(11, R, T, H, K, E, drop=0.0)
+    mask = np.zeros((R, R), np.int32)
+    mask[:, 2] = 1
+    mask[2, :] = 1
+    stats = torch.full((R, E // R), 5, dtype=torch.int32, device=cuda)
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, True, mask=mask, stats=stats)
+    assert rc == 0
+    want = eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, True, mask=mask, fill=0x55)
+    assert_dispatch_equal(got, want, True)
+    assert np.array_equal(stats.cpu().numpy(), want["recv_count"] + 5)  # elastic.py:266-269
+    assert got["recv_count"][2].sum() == 0
+
+
+def test_ll_dispatch_rejects_bad_arguments(cuda):
+    x, topk, _ = make_world(1, 2, 4, 512, 2, 4)
+    assert raw_ll_dispatch(cuda, x, topk, 4, 2, True)[0] == -1  # T > max tokens per rank
+    assert raw_ll_dispatch(cuda, x, topk, 3, 4, True)[0] == -1  # experts do not divide over ranks
+    assert raw_ll_dispatch(cuda, x, topk, 4, 4, False, use_ue8m0=True)[0] == -1
+    x2, topk2, _ = make_world(1, 2, 4, 384, 2, 4)
+    assert raw_ll_dispatch(cuda, x2, topk2, 4, 4, True)[0] == -1  # fp8 needs hidden % 512 == 0
+    buf = Buffer(2, device=cuda)
+    with pytest.raises(EPError):
+        buf.dispatch(x.to(cuda).float(), torch.from_numpy(topk).to(cuda), 4, 4)
+    with pytest.raises(EPError):
+        Buffer(2, low_latency_mode=False, device=cuda).dispatch(x.to(cuda), torch.from_numpy(topk).to(cuda), 4, 4)
+
+
+# ---- low-latency combine -------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(4, 12, 512, 3, 8, 16), (2, 130, 1024, 8, 64, 130), (8, 5, 2560, 4, 16, 8), (2, 9, 7168, 8, 16, 16)])
+def test_ll_combine_matches_oracle(cuda, shape):
+    R, T, H, K, E, M = shape
+    x, topk, w = make_world(5 + R, R, T, H, K, E)
+    nt = np.full(R, T, np.int32)
+    nt[0] = max(T - 3, 0)
+    buf = Buffer(R, device=cuda)
+    td = torch.from_numpy(topk).to(cuda)
+    wd = torch.from_numpy(w).to(cuda)
+    ntd = torch.from_numpy(nt).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False, num_tokens_per_rank=ntd)
+    # expert f_e(x) = x * (1 + 0.001 e) in bf16, only on the rows that exist
+    El = E // R
+    factor = (1 + 0.001 * torch.arange(E, device=cuda, dtype=torch.float32)).view(R, El, 1, 1)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, (rx.float() * factor).to(torch.bfloat16), torch.zeros_like(rx))
+    comb = torch.full((R, T, H), 7.0, dtype=torch.bfloat16, device=cuda)
+    out, _, _ = buf.combine(y, td, wd, handle, out=comb, num_tokens_per_rank=ntd)
+    torch.cuda.synchronize()
+    assert out is comb
+    si, lr = handle[0].cpu().numpy(), handle[1].cpu().numpy()
+    want = eo.ll_combine(bits16(y).reshape(R, El, R * M, H), topk, w, si, lr, E, M, num_tokens=nt, use_fma=True)
+    got = bits16(comb).reshape(R, T, H)
+    for r in range(R):
+        assert np.array_equal(got[r, :nt[r]], want[r, :nt[r]])
+        assert np.all(got[r, nt[r]:] == 0x40E0)  # rows of absent tokens keep the caller's 7.0
+    # within one bf16 ulp of the unfused (multiply, then add) evaluation
+    alt = eo.ll_combine(bits16(y).reshape(R, El, R * M, H), topk, w, si, lr, E, M, num_tokens=nt, use_fma=False)
+    a, b = eo.bf16_to_f32(got), eo.bf16_to_f32(alt)
+    for r in range(R):
+        ulp = np.maximum(np.abs(b[r, :nt[r]]), 2.0 ** -126) * 2.0 ** -7
+        assert np.all(np.abs(a[r, :nt[r]] - b[r, :nt[r]]) <= ulp)
+
+
+def test_ll_combine_follows_src_info_not_position(cuda):
+    R, T, H, K, E, M = 2, 70, 512, 2, 4, 70
+    x, topk, w = make_world(21, R, T, H, K, E, drop=0.0)
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    base, _, _ = buf.combine(rx.clone(), td, wd, handle)
+    si, lr = handle[0].clone(), handle[1].cpu().numpy()
+    rx2 = rx.clone()
+    rng = np.random.default_rng(0)
+    for d in range(R):
+        for le in range(E // R):
+            for r in range(R):
+                n, b = int(lr[d, le, r] & 0xFFFFFFFF), int(lr[d, le, r] >> 32)
+                p = torch.from_numpy(rng.permutation(n)).to(cuda)
+                rx2[d, le, b:b + n] = rx[d, le, b:b + n][p]
+                si[d, le, b:b + n] = handle[0][d, le, b:b + n][p]
+    out, _, _ = buf.combine(rx2, td, wd, (si, handle[1], handle[2], handle[3]))
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+
+
+def test_ll_masked_rank_drops_out_of_dispatch_and_combine(cuda):
+    # examples/device/ep/tests/elastic/elastic.py:359-383: after a rank is masked its tokens
+    # vanish from every count and its experts no longer contribute to combine.
+    R, T, H, K, E, M = 4, 16, 512, 4, 16, 16
+    x, topk, w = make_world(31, R, T, H, K, E, drop=0.0)
+    buf = Buffer(R, device=cuda)
+    buf.update_mask_buffer(1, True)
+    status = torch.zeros(R, dtype=torch.int32, device=cuda)
+    buf.query_mask_buffer(status)
+    assert status.tolist() == [0, 1, 0, 0]
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    out, _, _ = buf.combine(torch.where(torch.isfinite(rx.float()), rx, torch.zeros_like(rx)), td, wd, handle)
+    torch.cuda.synchronize()
+    El = E // R
+    alive = torch.tensor([0, 2, 3])
+    for e in range(E):
+        want = 0 if e // El == 1 else int((torch.from_numpy(topk)[alive] == e).sum())
+        assert int(cnt[e // El, e % El]) == want
+    keep = torch.from_numpy((topk // El != 1) & (topk >= 0))
+    wsum = (torch.from_numpy(w) * keep).sum(2)
+    for r in (0, 2, 3):
+        assert calc_diff(x[r].float() * wsum[r].unsqueeze(1), out[r].float().cpu()) < 1e-5
+    buf.clean_mask_buffer()
+    buf.query_mask_buffer(status)
+    assert status.sum().item() == 0
+
+
+def test_reference_elastic_pattern_fp8_and_bf16(cuda):
+    # The data of examples/device/ep/tests/elastic/elastic.py:131-134,153-175 and its checks
+    # (:263-318, :377-387) with 4 virtual ranks, 32 experts, top-8 and 64 tokens.
+    R, T, H, K, E, M = 4, 64, 2048, 8, 32, 64
+    El = E // R
+    g = torch.Generator().manual_seed(0)
+    x = torch.ones((R, T, H), dtype=torch.bfloat16) * (torch.arange(R).view(R, 1, 1) - 128).to(torch.bfloat16)
+    x[:, :, -128:] = torch.arange(T).to(torch.bfloat16).view(1, T, 1)
+    scores = torch.randn((R, T, E), generator=g).abs() + 1
+    topk = torch.topk(scores, K, dim=-1, largest=True, sorted=True)[1].to(torch.int32)
+    for r in range(R):
+        for _ in range(10):
+            topk[r, int(torch.randint(0, T, (1,), generator=g)), int(torch.randint(0, K, (1,), generator=g))] = -1
+    w = torch.randn((R, T, K), generator=g).abs()
+    buf = Buffer(R, device=cuda)
+    xd, td, wd = x.to(cuda), topk.to(cuda), w.to(cuda)
+    for use_fp8 in (False, True):
+        stats = torch.zeros((R, El), dtype=torch.int32, device=cuda)
+        recv, cnt, handle, event, hook = buf.dispatch(xd, td, M, E, cumulative_local_expert_recv_stats=stats,
+                                                      use_fp8=use_fp8, async_finish=True)
+        event.current_stream_wait()
+        torch.cuda.synchronize()
+        if use_fp8:
+            q, sc = recv[0], recv[1].contiguous()
+            assert sc.shape == (R, El, R * M, H // 128)
+            # cast back through bf16 like per_token_cast_back (tests/utils.py:80-89)
+            deq = (q.float().view(R, El, R * M, H // 128, 128) * sc.unsqueeze(-1)).view(R, El, R * M, H)
+            deq = deq.to(torch.bfloat16).float()
+        else:
+            deq = recv.float()
+        for rank in range(R):
+            for i in range(El):
+                e = rank * El + i
+                n = int(cnt[rank, i])
+                assert int(stats[rank, i]) == n
+                lr = handle[1][rank, i]
+                assert n == int((lr & 0xFFFFFFFF).sum()) == int((topk == e).sum())
+                if n == 0:
+                    continue
+                rx = deq[rank, i, :n]
+                assert torch.equal(rx[:, :-128].amin(dim=-1), rx[:, :-128].amax(dim=-1))
+                src = handle[0][rank, i, :n]
+                assert float((rx[:, -128:] - src.view(-1, 1) % T).abs().sum()) == 0 or use_fp8
+                if use_fp8:
+                    assert calc_diff(rx[:, -1], src.float()) < 0.007
+                for j in range(R):
+                    b, c = int(lr[j] >> 32), int(lr[j] & 0xFFFFFFFF)
+                    assert c == int((topk[j] == e).sum())
+                    assert float((rx[b:b + c, :-128] - (j - 128)).abs().sum()) == 0
+        # identity experts: combined == x * sum of valid weights
+        y = deq.to(torch.bfloat16)
+        y = torch.where(torch.isfinite(y.float()), y, torch.zeros_like(y))
+        comb, _, _ = buf.combine(y, td, wd, handle)
+        torch.cuda.synchronize()
+        ref = xd.float() * (wd * (td >= 0)).sum(2, keepdim=True)
+        assert calc_diff(ref, comb.float()) < (9e-4 if use_fp8 else 1e-5)
+
+
+def test_config4_full_size_properties(cuda):
+    # BASELINE config 4: 32 virtual ranks x 128 tokens x hidden 7168, 256 experts, top-8 by
+    # the router from N(0,1) logits, fp8 dispatch, expert f_e = dequant(x) * (1 + 0.001 e) in
+    # bf16, weighted combine.  Checked by: counts against a histogram, every delivered row
+    # against the oracle's cast of its source token (sampled) and against a torch
+    # re-quantisation (all rows, dequantised error bound), combine against the closed form
+    # on sampled tokens (bit-exact) and against x * sum(w * f) globally.
+    R, T, H, K, E, M = 32, 128, 7168, 8, 256, 128
+    El, N = E // R, R * M
+    g = torch.Generator(device=cuda).manual_seed(4)
+    x = torch.randn((R, T, H), generator=g, device=cuda).to(torch.bfloat16)
+    logits = torch.randn((R, T, E), generator=g, device=cuda)
+    buf = Buffer(R, device=cuda)
+    topk, w = buf.route(logits, K)
+    (q, sc_t), cnt, handle, _, _ = buf.dispatch(x, topk, M, E, use_fp8=True)
+    torch.cuda.synchronize()
+    src_info, layout = handle[0], handle[1]
+    hist = torch.bincount(topk.view(-1).long(), minlength=E).view(R, El)
+    assert torch.equal(cnt.long(), hist)
+    assert torch.equal((layout & 0xFFFFFFFF).sum(-1), hist)
+    # segments: begin = exclusive prefix of counts over source ranks
+    counts = layout & 0xFFFFFFFF
+    begins = layout >> 32
+    assert torch.equal(begins, torch.cumsum(counts, -1) - counts)
+    per_src = torch.stack([torch.bincount(topk[r].view(-1).long(), minlength=E) for r in range(R)], 1).view(R, El, R)
+    assert torch.equal(counts, per_src)
+    sc = sc_t.contiguous()  # [R, El, N, G]
+    rng = np.random.default_rng(0)
+    xb = bits16(x).reshape(R, T, H)
+    qh = q.view(torch.uint8)
+    lr = layout.cpu().numpy()
+    for _ in range(48):
+        e = int(rng.integers(0, E))
+        d, le = divmod(e, El)
+        n = int(cnt[d, le])
+        if n == 0:
+            continue
+        i = int(rng.integers(0, n))
+        seg_begin = lr[d, le] >> 32
+        r = int(np.searchsorted(seg_begin + (lr[d, le] & 0xFFFFFFFF), i, side="right"))
+        t = int(src_info[d, le, i])
+        assert e in topk[r, t].tolist()
+        want_q, want_s = eo.cast_row_fp8(xb[r, t])
+        assert np.array_equal(qh[d, le, i].cpu().numpy(), want_q)
+        assert np.array_equal(sc[d, le, i].cpu().numpy(), want_s)
+    # expert step and combine
+    valid = (torch.arange(N, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1))
+    y = torch.zeros((R, El, N, H), dtype=torch.bfloat16, device=cuda)
+    for d in range(R):
+        deq = (q[d].float().view(El, N, H // 128, 128) * sc[d].unsqueeze(-1)).view(El, N, H)
+        f = (1 + 0.001 * (d * El + torch.arange(El, device=cuda, dtype=torch.float32))).view(El, 1, 1)
+        y[d] = torch.where(valid[d].unsqueeze(-1), (deq.to(torch.bfloat16).float() * f).to(torch.bfloat16), y[d])
+    comb, _, _ = buf.combine(y, topk, w, handle)
+    torch.cuda.synchronize()
+    fw = (w * (1 + 0.001 * topk.float())).sum(-1, keepdim=True)
+    assert calc_diff(x.float() * fw, comb.float()) < 9e-4
+    si_h = src_info.cpu().numpy()
+    tk, wk = topk.cpu().numpy(), w.cpu().numpy()
+    for _ in range(24):
+        r, t = int(rng.integers(0, R)), int(rng.integers(0, T))
+        rows = []
+        for k in range(K):
+            e = int(tk[r, t, k])
+            d, le = divmod(e, El)
+            b, n = int(lr[d, le, r] >> 32), int(lr[d, le, r] & 0xFFFFFFFF)
+            i = b + int(np.nonzero(si_h[d, le, b:b + n] == t)[0][0])
+            rows.append(bits16(y[d, le, i]))
+        assert np.array_equal(bits16(comb[r, t]), eo.weighted_sum_rows(np.stack(rows), wk[r, t]))
+
+
+# ---- normal mode -------------------------------------------------------------------------------------------
+
+def zipf_topk(rng, R, T, K, E, s=1.2):
+    """Skewed router for BASELINE config 5: K distinct experts per token drawn from a Zipf(s)
+    law over a seeded permutation of the experts (Gumbel top-k = sampling without
+    replacement), softmax weights of the drawn scores."""
+    perm = rng.permutation(E)
+    p = 1.0 / np.arange(1, E + 1) ** s
+    logp = np.log(p / p.sum())[np.argsort(perm)]
+    keys = logp[None, None, :] + rng.gumbel(size=(R, T, E))
+    topk = np.argsort(-keys, axis=2)[:, :, :K].astype(np.int32)
+    sel = np.take_along_axis(keys, topk, 2)
+    w = np.exp(sel - sel.max(2, keepdims=True))
+    return topk, (w / w.sum(2, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("shape", [(4, 37, 256, 4, 16, 5, 8), (8, 300, 1024, 8, 64, 10, 1), (2, 1500, 512, 2, 4, 3, 4)])
+def test_ht_pipeline_matches_oracle(cuda, shape):
+    R, T, H, K, E, C, align = shape
+    x, topk, w = make_world(3 * R, R, T, H, K, E)
+    buf = Buffer(R, low_latency_mode=False, device=cuda)
+    xd, td, wd = x.to(cuda), torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(td, E)
+    torch.cuda.synchronize()
+    lay = [eo.dispatch_layout(topk[r], R, E) for r in range(R)]
+    assert np.array_equal(per_rank.cpu().numpy(), np.stack([l[0] for l in lay]))
+    assert np.array_equal(per_expert.cpu().numpy(), np.stack([l[1] for l in lay]))
+    o_in_rank = np.stack([l[2] for l in lay])
+    assert np.array_equal(in_rank.cpu().numpy().astype(np.uint8), o_in_rank)
+    recv_x, recv_idx, recv_w, per_expert_list, handle, _ = buf.ht_dispatch(
+        xd, num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert, topk_idx=td,
+        topk_weights=wd, expert_alignment=align, num_channels=C)
+    torch.cuda.synchronize()
+    o_prefix, o_counts, o_chan = eo.ht_notify(o_in_rank, np.stack([l[1] for l in lay]), C, align)
+    _, prefix, chan, meta, send_head, row_offset = handle
+    assert np.array_equal(prefix.cpu().numpy(), o_prefix)
+    assert np.array_equal(chan.cpu().numpy(), o_chan)
+    assert per_expert_list == o_counts.tolist()
+    o = eo.ht_dispatch(bits16(x).reshape(R, T, H), topk, w, o_in_rank, o_prefix, E)
+    assert np.array_equal(row_offset.cpu().numpy(), o["row_offset"])
+    assert np.array_equal(send_head.cpu().numpy(), o["send_head"])
+    assert np.array_equal(bits16(recv_x).reshape(-1, H), o["recv_x"])
+    assert np.array_equal(recv_idx.cpu().numpy(), o["recv_topk_idx"])
+    assert np.array_equal(recv_w.cpu().numpy(), o["recv_topk_weights"])
+    assert np.array_equal(meta.cpu().numpy(), np.stack([o["recv_src_rank"], o["recv_src_token"]], 1))
+    b0 = torch.from_numpy(np.random.default_rng(1).standard_normal((R, T, H)).astype(np.float32)).to(torch.bfloat16)
+    b1 = torch.from_numpy(np.random.default_rng(2).standard_normal((R, T, H)).astype(np.float32)).to(torch.bfloat16)
+    for bias in (None, b0.to(cuda), (b0.to(cuda), b1.to(cuda))):
+        comb, comb_w, _ = buf.ht_combine(recv_x, handle, topk_weights=recv_w, bias=bias)
+        torch.cuda.synchronize()
+        ob0 = None if bias is None else bits16(b0).reshape(R, T, H)
+        ob1 = bits16(b1).reshape(R, T, H) if isinstance(bias, tuple) else None
+        want, want_w = eo.ht_combine(o["recv_x"], o["recv_topk_weights"], o_in_rank, o_prefix, o["send_head"],
+                                     o["row_offset"], ob0, ob1)
+        assert np.array_equal(bits16(comb).reshape(R, T, H), want)
+        assert np.array_equal(comb_w.cpu().numpy(), want_w)
+
+
+def test_config5_full_size_properties(cuda):
+    # BASELINE config 5: 8 virtual ranks x 4096 tokens x 7168, 256 experts, top-8, Zipf(1.2)
+    # expert popularity; bf16 dispatch with counts and prefix layout; combine of per-rank
+    # partial sums y_d[t] = bf16(sum over local selected experts of w * f_e(x)).
+    R, T, H, K, E, C = 8, 4096, 7168, 8, 256, 10
+    El = E // R
+    rng = np.random.default_rng(5)
+    topk, w = zipf_topk(rng, R, T, K, E)
+    g = torch.Generator(device=cuda).manual_seed(5)
+    x = torch.randn((R, T, H), generator=g, device=cuda).to(torch.bfloat16)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    buf = Buffer(R, low_latency_mode=False, device=cuda)
+    per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(td, E)
+    # tests/test_ht.py:99-152
+    assert torch.equal(per_expert.long(), torch.stack([torch.bincount(td[r].view(-1).long(), minlength=E) for r in range(R)]))
+    rank_of = td // El
+    want_in = torch.zeros((R, T, R), dtype=torch.bool, device=cuda).scatter_(2, rank_of.long(), True)
+    assert torch.equal(in_rank, want_in)
+    assert torch.equal(per_rank.long(), want_in.sum(1))
+    recv_x, recv_idx, recv_w, per_expert_list, handle, _ = buf.ht_dispatch(
+        x, num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert, topk_idx=td,
+        topk_weights=wd, num_channels=C)
+    torch.cuda.synchronize()
+    _, prefix, chan, meta, send_head, row_offset = handle
+    assert torch.equal(prefix.long(), torch.cumsum(want_in.sum(1).t(), 1))  # [dst][src], test_ht.py:166-172
+    assert recv_x.shape[0] == int(want_in.sum())
+    assert per_expert_list == per_expert.sum(0).view(R, El).tolist()  # test_ht.py:223-229
+    # every received row is its source row; rows are ordered by (source rank, token)
+    src_r, src_t = meta[:, 0].long(), meta[:, 1].long()
+    assert torch.equal(recv_x.view(torch.int16), x[src_r, src_t].view(torch.int16))
+    for d in range(R):
+        lo, hi = int(row_offset[d]), int(row_offset[d + 1])
+        key = src_r[lo:hi] * T + src_t[lo:hi]
+        assert bool((key[1:] > key[:-1]).all())
+        ridx = recv_idx[lo:hi]
+        assert bool(((ridx == -1) | ((ridx >= 0) & (ridx < El))).all())  # test_ht.py:236-244
+        assert torch.equal(torch.bincount(ridx[ridx >= 0].long(), minlength=El), per_expert.sum(0)[d * El:(d + 1) * El].long())
+        assert bool((recv_w[lo:hi][ridx < 0] == 0).all())
+    # expert step on each destination: partial weighted sum over its local experts
+    f = 1 + 0.001 * (torch.arange(R, device=cuda).repeat_interleave(torch.diff(row_offset)).view(-1, 1) * El + recv_idx.clamp(min=0)).float()
+    coef = (recv_w * f * (recv_idx >= 0)).sum(1, keepdim=True)
+    y = (recv_x.float() * coef).to(torch.bfloat16)
+    comb, comb_w, _ = buf.ht_combine(y, handle, topk_weights=recv_w)
+    torch.cuda.synchronize()
+    assert torch.allclose(comb_w, wd, rtol=0, atol=1e-7)  # test_ht.py:309-323
+    ref = x.float() * (wd * (1 + 0.001 * td.float())).sum(-1, keepdim=True)
+    assert calc_diff(ref, comb.float()) < 5e-5
+    # exact check of the reduction on sampled tokens: ascending destination order, fp32 adds
+    yb = y.view(torch.int16)
+    for _ in range(16):
+        r, t = int(rng.integers(0, R)), int(rng.integers(0, T))
+        acc = np.zeros(H, np.float32)
+        for d in range(R):
+            if not bool(in_rank[r, t, d]):
+                continue
+            row = int(row_offset[d]) + (0 if r == 0 else int(prefix[d, r - 1])) + int(send_head[r, t, d])
+            acc = acc + eo.bf16_to_f32(yb[row].cpu().numpy().view(np.uint16))
+        assert np.array_equal(bits16(comb[r, t]), eo.f32_to_bf16(acc))
+
+
+# ---- router ---------------------------------------------------------------------------------------------------
+
+def test_router_matches_oracle(cuda):
+    rng = np.random.default_rng(40)
+    for T, E, K in ((200, 256, 8), (33, 7, 3), (5, 1024, 16), (64, 64, 1)):
+        logits = rng.standard_normal((T, E)).astype(np.float32)
+        logits[0, :] = 0.0
+        if E > 9:
+            logits[1, 5] = logits[1, 9] = 7.0
+        buf = Buffer(2, device=cuda)
+        idx, w = buf.route(torch.from_numpy(logits).to(cuda), K)
+        torch.cuda.synchronize()
+        oi, ow = eo.router(logits, K)
+        assert np.array_equal(idx.cpu().numpy(), oi)
+        # weights: exp() of the device and of libm may differ in the last place
+        assert np.allclose(w.cpu().numpy(), ow, rtol=2e-6, atol=0)
+    with pytest.raises(EPError):
+        buf.route(torch.zeros((4, 2000), device=cuda), 2)
