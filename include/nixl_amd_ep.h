@@ -28,11 +28,17 @@
 extern "C" {
 #endif
 
-/* Bytes of scratch the low-latency dispatch needs (per-(rank, expert) send counts and
- * per-(token, k) positions).  Reference: `workspace` of ep_kernels::dispatch,
- * kernels/nixl_ep_ll.cu:423-426. */
+/* Launch-shape knob of the low-latency kernels (no reference counterpart): the largest
+ * workgroup, in lanes, of the dispatch and combine kernels; a multiple of 64 in [64, 1024],
+ * or 0 to leave a value unchanged.  Process-wide; not thread-safe against running calls. */
+int
+nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes);
+
+/* Bytes of scratch the low-latency dispatch needs (per-(rank, expert) send counts,
+ * per-(token, k) rows, per-token scales); the scratch must be 4-byte aligned.  Reference:
+ * `workspace` of ep_kernels::dispatch, kernels/nixl_ep_ll.cu:423-426. */
 size_t
-nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk);
+nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk, int hidden);
 
 /*
  * Low-latency dispatch for all ranks.  Replaces ep_kernels::dispatch
@@ -51,6 +57,10 @@ nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, i
  *   packed_recv_layout_range [R][El][R] int64: count | begin << 32
  *   packed_recv_count      [R][El] int32
  *   cumulative_local_expert_recv_stats [R][El] int32 or NULL; incremented by the counts
+ *   row_map                [R][T][K] int32 or NULL (no reference counterpart): receives, for
+ *                          every selection, its row in the flattened [R*El*N] row space of
+ *                          packed_recv_x, or -1.  Passing it on to the combine call saves
+ *                          that call its search through src_info.
  * Rows at or beyond packed_recv_count are not written.
  */
 int
@@ -73,6 +83,7 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                         int use_fp8,
                         int round_scale,
                         int use_ue8m0,
+                        int *row_map,
                         void *workspace,
                         size_t workspace_bytes,
                         void *stream);
@@ -85,6 +96,8 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
  * handle (src_info, layout_range), so any valid permutation inside a segment is accepted.
  *   x             [R][El][N][H] bf16 (expert outputs in packed_recv_x layout)
  *   combined_x    [R][T][H] bf16
+ *   row_map       [R][T][K] int32 as written by the dispatch call that produced this
+ *                 handle, or NULL to locate rows through src_info / layout_range
  * The LogFMT payload codec of the reference is not implemented: use_logfmt must be 0.
  */
 int
@@ -96,6 +109,7 @@ nixl_amd_ep_ll_combine(void *combined_x,
                        const int64_t *layout_range,
                        const int *mask_buffer,
                        const int *num_tokens_per_rank,
+                       const int *row_map,
                        int num_tokens,
                        int hidden,
                        int num_max_dispatch_tokens_per_rank,

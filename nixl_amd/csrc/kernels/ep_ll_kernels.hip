@@ -4,16 +4,22 @@
 // What the reference does per rank with three passes over the payload (cast into a send
 // buffer, K message copies into per-(expert, source rank) receive slots, repack into the
 // per-expert contiguous output; kernels/nixl_ep_ll.cu:134-393) is done here in two
-// launches, because every "remote" slot is an address in the same HBM:
+// launches that touch the payload once, because every "remote" slot is an address in the
+// same HBM:
 //   1. ll_layout_kernel    one workgroup per source rank builds, in LDS, one bitmask of
 //                          tokens per expert and derives count[r][e] and the position of
 //                          every (token, k) inside its (r, e) segment;
 //   2. ll_dispatch_kernel  one workgroup per token reads its bf16 row once, quantises it in
 //                          registers and writes it straight to its K final rows of
-//                          packed_recv_x (and the scales column-major, src_info); the row
-//                          index is begin[e][r] + position with begin = sum of counts of
-//                          lower source ranks.  Extra workgroups write layout_range,
-//                          recv_count and the statistics.
+//                          packed_recv_x (row = e * N + sum of the lower source ranks'
+//                          counts for e + position), plus src_info and the token's H/128
+//                          scales (once, contiguous);
+//   3. ll_scales_kernel    workgroups per expert scan the per-rank counts into layout_range,
+//                          recv_count and the statistics, and copy each received row's
+//                          scales into the column-major scales array with coalesced stores
+//                          (writing them from step 2 would be one isolated 4-byte store per
+//                          scale).
+// Steps 1 and 3 move a few megabytes; step 2 moves the payload.
 // The order this produces is the canonical one among those the reference's atomics allow:
 // segments by source rank ascending, tokens ascending inside a segment.
 //
@@ -23,6 +29,7 @@
 // Combine is one launch: one workgroup per token locates its K rows through the dispatch
 // handle, reads them once and accumulates in fp32 with fused multiply-adds in top-k order
 // (kernels/nixl_ep_ll.cu:959-1012).  Traffic per token: read K * 2H, write 2H.
+#include <algorithm>
 #include <cstdint>
 
 #include "common.h"
@@ -103,82 +110,65 @@ ll_layout_kernel(const int32_t *__restrict__ topk_idx,
     }
 }
 
-// ---- 2. cast + scatter ------------------------------------------------------------------
+// ---- 2. cast + scatter ----------------------------------------------------------------------------
 
 struct DispatchArgs {
     uint8_t *recv_x;
-    void *recv_scales;
     int *src_info;
-    long long *layout_range;
-    int *recv_count;
-    int *stats;
+    float *token_scales; // [R][T][H/128] inverse scales, one row per source token
     const uint16_t *x;
     const int32_t *topk_idx;
     const int *num_tokens_per_rank;
-    const int *send_count;
-    const int *pos;
+    const int *send_count; // [R][E]
+    const int *rows; // [R][T][K] position inside the (r, e) segment, -1 if none
+    int *rows_out; // [R][T][K] final row e * N + begin + position, -1 if none
     LlDims d;
     int round_scale;
-    int use_ue8m0;
+    int parts; // workgroups per token; each covers blockDim.x of the token's H/16 lanes
 };
 
-// grid = R metadata workgroups followed by R*T token workgroups; block = H/16 lanes rounded
-// up to whole waves.  Each lane owns 16 consecutive channels (32 bytes of bf16, 16 bytes of
-// fp8), so a 128-channel scale group is 8 neighbouring lanes.
+// grid = R*T*parts workgroups.  A token's row is H/16 "lanes" of 16 consecutive channels
+// (32 bytes of bf16, 16 bytes of fp8), so a 128-channel scale group is 8 neighbouring
+// lanes; a workgroup covers blockDim.x of them (a multiple of 64).
 template<bool FP8>
 __global__ void __launch_bounds__(1024)
 ll_dispatch_kernel(DispatchArgs a) {
     const LlDims d = a.d;
     const int tid = threadIdx.x;
-    __shared__ long long row_of_k[kMaxTopk]; // e * N + slot, or -1
-
-    if (blockIdx.x < static_cast<unsigned>(d.R)) {
-        // Metadata role for source rank r: (count, begin) of every expert's segment r.
-        const int r = blockIdx.x;
-        for (int e = tid; e < d.E; e += blockDim.x) {
-            int begin = 0;
-            for (int q = 0; q < r; ++q)
-                begin += a.send_count[q * d.E + e];
-            const int n = a.send_count[r * d.E + e];
-            a.layout_range[static_cast<size_t>(e) * d.R + r] =
-                static_cast<long long>(static_cast<unsigned>(n)) | (static_cast<long long>(begin) << 32);
-            if (r == d.R - 1) {
-                a.recv_count[e] = begin + n;
-                if (a.stats) a.stats[e] += begin + n;
-            }
-        }
-        return;
-    }
-
-    const int token = blockIdx.x - d.R;
+    __shared__ int row_of_k[kMaxTopk]; // e * N + slot, or -1
+    const int token = blockIdx.x / a.parts, part = blockIdx.x % a.parts;
     const int r = token / d.T, t = token % d.T;
     const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
     if (t >= nt) return;
 
-    if (tid < d.K) {
-        const int p = a.pos[(static_cast<size_t>(r) * d.T + t) * d.K + tid];
-        long long row = -1;
-        if (p >= 0) {
-            const int e = a.topk_idx[(static_cast<size_t>(r) * d.T + t) * d.K + tid];
-            int begin = 0;
-            for (int q = 0; q < r; ++q)
-                begin += a.send_count[q * d.E + e];
-            row = static_cast<long long>(e) * d.N + begin + p;
-        }
-        row_of_k[tid] = row;
+    // Final row of selection k: e * N + (tokens the lower source ranks send to e) + position.
+    // Half a wave per selection: its 32 lanes fetch the lower ranks' counts in parallel.
+    for (int k = tid >> 5; k < d.K; k += blockDim.x >> 5) {
+        const int q0 = tid & 31;
+        const size_t sel = (static_cast<size_t>(r) * d.T + t) * d.K + k;
+        const int p = a.rows[sel];
+        const int e = a.topk_idx[sel];
+        int partial = 0;
+        if (p >= 0)
+            for (int q = q0; q < r; q += 32)
+                partial += a.send_count[q * d.E + e];
+        partial += __shfl_xor(partial, 16);
+        partial += __shfl_xor(partial, 8);
+        partial += __shfl_xor(partial, 4);
+        partial += __shfl_xor(partial, 2);
+        partial += __shfl_xor(partial, 1);
+        if (q0 == 0) row_of_k[k] = p >= 0 ? e * d.N + partial + p : -1;
     }
-
-    const int lanes = d.H / 16;
-    const bool active = tid < lanes;
+    const int lane = part * blockDim.x + tid; // lane of the token's row
+    const bool active = lane < d.H / 16;
     uint4 raw0 = make_uint4(0, 0, 0, 0), raw1 = raw0;
     if (active) {
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.x + (static_cast<size_t>(r) * d.T + t) * d.H) + tid * 2;
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.x + (static_cast<size_t>(r) * d.T + t) * d.H) + lane * 2;
         raw0 = ld16_nt(src);
         raw1 = ld16_nt(src + 1);
     }
 
     uint4 q = make_uint4(0, 0, 0, 0);
-    float scale_inv = 0.f;
     if constexpr (FP8) {
         const uint32_t w[8] = {raw0.x, raw0.y, raw0.z, raw0.w, raw1.x, raw1.y, raw1.z, raw1.w};
         float v[16];
@@ -193,8 +183,10 @@ ll_dispatch_kernel(DispatchArgs a) {
         amax = fmaxf(amax, __shfl_xor(amax, 1));
         amax = fmaxf(amax, __shfl_xor(amax, 2));
         amax = fmaxf(amax, __shfl_xor(amax, 4));
-        float scale;
+        float scale, scale_inv;
         fp8_scales(amax, a.round_scale != 0, scale, scale_inv);
+        if (active && (lane & 7) == 0)
+            a.token_scales[(static_cast<size_t>(r) * d.T + t) * (d.H / 128) + (lane >> 3)] = scale_inv;
         uint32_t out[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -204,31 +196,129 @@ ll_dispatch_kernel(DispatchArgs a) {
         q = make_uint4(out[0], out[1], out[2], out[3]);
     }
     __syncthreads();
+    // Publish the rows (combine reads them back as its row map).  They go to an array of
+    // their own: the other workgroups of this token may still be reading the positions.
+    if (part == 0 && tid < d.K) a.rows_out[(static_cast<size_t>(r) * d.T + t) * d.K + tid] = row_of_k[tid];
 
-    const int G = d.H / 128;
     for (int k = 0; k < d.K; ++k) {
-        const long long row = row_of_k[k];
+        const int row = row_of_k[k];
         if (row < 0) continue;
-        if (tid == 0) a.src_info[row] = t;
+        if (lane == 0) a.src_info[row] = t;
         if (!active) continue;
         if constexpr (FP8) {
-            uint4 *dst = reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H) + tid;
-            st16_nt(dst, q);
-            if ((tid & 7) == 0) {
-                const int g = tid >> 3;
-                const long long e = row / d.N, slot = row % d.N;
-                if (!a.use_ue8m0) {
-                    static_cast<float *>(a.recv_scales)[(static_cast<size_t>(e) * G + g) * d.N + slot] = scale_inv;
-                } else {
-                    uint8_t *base = static_cast<uint8_t *>(a.recv_scales) + static_cast<size_t>(e) * (G / 4) * d.N * 4;
-                    base[(static_cast<size_t>(g / 4) * d.N + slot) * 4 + (g & 3)] =
-                        static_cast<uint8_t>(__float_as_uint(scale_inv) >> 23);
+            st16_nt(reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H) + lane, q);
+        } else {
+            uint4 *dst = reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H * 2) + lane * 2;
+            st16_nt(dst, raw0);
+            st16_nt(dst + 1, raw1);
+        }
+    }
+}
+
+// ---- 3. receive-side metadata and scales, column-major per expert ----------------------------------------------------------------
+
+struct ScalesArgs {
+    void *recv_scales; // null: metadata only
+    const float *token_scales;
+    const int *src_info;
+    const int *send_count; // [R][E]
+    long long *layout_range;
+    int *recv_count;
+    int *stats;
+    LlDims d;
+    int use_ue8m0;
+};
+
+// grid = E * kScaleParts workgroups.  Every workgroup of expert e scans the R per-rank
+// counts into segment ends (part 0 also writes them out as layout_range, recv_count and the
+// statistics); workgroup (e, part) then copies scale groups part, part + kScaleParts, ... of
+// every received row of expert e.  A thread owns row `slot`
+// (= tid, tid + 256, ...): it finds the row's source rank from the segment ends, then
+// gathers that token's scales (contiguous per token) and writes them at stride N, so that
+// for each scale group the threads of a wave write consecutive addresses (the column-major
+// layout of csrc/nixl_ep.cpp:1093-1100, kernels/nixl_ep_ll.cu:372-391).
+constexpr int kScaleParts = 4;
+constexpr int kScaleBatch = 8;
+
+__global__ void __launch_bounds__(kLayoutThreads)
+ll_scales_kernel(ScalesArgs a) {
+    extern __shared__ int seg_end[]; // [R] end of each source rank's segment of expert e
+    const LlDims d = a.d;
+    const int e = blockIdx.x / kScaleParts, part = blockIdx.x % kScaleParts, tid = threadIdx.x;
+    const int G = d.H / 128;
+    if (!a.recv_scales && part != 0) return; // metadata only: one workgroup per expert is enough
+    // the first row's source token is fetched before its validity is known (always in bounds)
+    int t_next = a.src_info[static_cast<size_t>(e) * d.N + min(tid, d.N - 1)];
+    for (int r = tid; r < d.R; r += kLayoutThreads)
+        seg_end[r] = a.send_count[r * d.E + e];
+    __syncthreads();
+    if (tid < kWaveSize) {
+        // inclusive scan of the R counts by one wave, 64 ranks per step
+        int carry = 0;
+        for (int r0 = 0; r0 < d.R; r0 += kWaveSize) {
+            const int r = r0 + tid;
+            const int n_r = r < d.R ? seg_end[r] : 0;
+            int incl = n_r;
+#pragma unroll
+            for (int off = 1; off < kWaveSize; off <<= 1) {
+                const int up = __shfl_up(incl, off);
+                if (tid >= off) incl += up;
+            }
+            incl += carry;
+            if (r < d.R) {
+                seg_end[r] = incl;
+                if (part == 0)
+                    a.layout_range[static_cast<size_t>(e) * d.R + r] =
+                        static_cast<long long>(static_cast<unsigned>(n_r)) | (static_cast<long long>(incl - n_r) << 32);
+            }
+            carry = __shfl(incl, kWaveSize - 1);
+        }
+        if (part == 0 && tid == 0) {
+            a.recv_count[e] = carry;
+            if (a.stats) a.stats[e] += carry;
+        }
+    }
+    __syncthreads();
+    if (!a.recv_scales) return;
+    const int n = seg_end[d.R - 1];
+    for (int slot = tid; slot < n; slot += kLayoutThreads) {
+        const int t = t_next;
+        if (slot + kLayoutThreads < n) t_next = a.src_info[static_cast<size_t>(e) * d.N + slot + kLayoutThreads];
+        int lo = 0, hi = d.R - 1; // first rank whose segment ends beyond `slot`
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (seg_end[mid] > slot)
+                hi = mid;
+            else
+                lo = mid + 1;
+        }
+        const float *__restrict__ src = a.token_scales + (static_cast<size_t>(lo) * d.T + t) * G;
+        if (!a.use_ue8m0) {
+            float *__restrict__ dst = static_cast<float *>(a.recv_scales) + static_cast<size_t>(e) * G * d.N + slot;
+            for (int g0 = part; g0 < G; g0 += kScaleParts * kScaleBatch) {
+                float v[kScaleBatch];
+#pragma unroll
+                for (int j = 0; j < kScaleBatch; ++j) {
+                    const int g = g0 + j * kScaleParts;
+                    v[j] = g < G ? src[g] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < kScaleBatch; ++j) {
+                    const int g = g0 + j * kScaleParts;
+                    if (g < G) dst[static_cast<size_t>(g) * d.N] = v[j];
                 }
             }
         } else {
-            uint4 *dst = reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H * 2) + tid * 2;
-            st16_nt(dst, raw0);
-            st16_nt(dst + 1, raw1);
+            // one exponent byte per group, four groups per 32-bit word, words [H/512][N]
+            uint32_t *__restrict__ dst =
+                static_cast<uint32_t *>(a.recv_scales) + static_cast<size_t>(e) * (G / 4) * d.N + slot;
+            for (int g4 = part; g4 < G / 4; g4 += kScaleParts) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    word |= ((__float_as_uint(src[g4 * 4 + j]) >> 23) & 0xffu) << (8 * j);
+                dst[static_cast<size_t>(g4) * d.N] = word;
+            }
         }
     }
 }
@@ -244,22 +334,37 @@ struct CombineArgs {
     const long long *layout_range;
     const int *mask;
     const int *num_tokens_per_rank;
+    const int *row_map; // optional [R][T][K] from dispatch; replaces the search below
     LlDims d;
+    int parts; // workgroups per token; each covers blockDim.x of the token's H/8 lanes
 };
 
-// grid = R*T workgroups; block = H/8 lanes rounded up to whole waves; each lane owns 8
-// consecutive channels (16 bytes per row).
+// grid = R*T*parts workgroups; a token's row is H/8 lanes of 8 consecutive channels (16
+// bytes); a workgroup covers blockDim.x of them (a multiple of 64).
 __global__ void __launch_bounds__(1024)
 ll_combine_kernel(CombineArgs a) {
     const LlDims d = a.d;
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize, n_waves = blockDim.x / kWaveSize;
-    const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
+    const int token = blockIdx.x / a.parts, part = blockIdx.x % a.parts;
+    const int r = token / d.T, t = token % d.T;
     const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
     if (t >= nt) return;
+    const int col = part * blockDim.x + tid; // lane of the token's row
     __shared__ long long row_of_k[kMaxTopk];
     __shared__ float weight_of_k[kMaxTopk];
 
+    if (a.row_map) {
+        // Rows recorded by dispatch: one load per selection instead of a search.
+        if (tid < d.K) {
+            const size_t sel = (static_cast<size_t>(r) * d.T + t) * d.K + tid;
+            const int e = a.topk_idx[sel];
+            long long row = a.row_map[sel];
+            if (e < 0 || e >= d.E || pair_blocked(a.mask, d.R, r, e / d.El)) row = -1;
+            row_of_k[tid] = row;
+            weight_of_k[tid] = a.topk_weights[sel];
+        }
+    } else
     // Locate the K rows: wave w searches selections w, w + n_waves, ...
     for (int k = wave; k < d.K; k += n_waves) {
         const size_t sel = (static_cast<size_t>(r) * d.T + t) * d.K + k;
@@ -282,7 +387,7 @@ ll_combine_kernel(CombineArgs a) {
         }
     }
     __syncthreads();
-    if (tid >= d.H / 8) return;
+    if (col >= d.H / 8) return;
 
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < d.K; k0 += 8) {
@@ -292,7 +397,7 @@ ll_combine_kernel(CombineArgs a) {
             const long long row = (k0 + j < d.K) ? row_of_k[k0 + j] : -1;
             v[j] = make_uint4(0, 0, 0, 0);
             if (row >= 0)
-                v[j] = ld16_nt(reinterpret_cast<const uint4 *>(a.x + static_cast<size_t>(row) * d.H) + tid);
+                v[j] = ld16_nt(reinterpret_cast<const uint4 *>(a.x + static_cast<size_t>(row) * d.H) + col);
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -311,7 +416,7 @@ ll_combine_kernel(CombineArgs a) {
     out.y = f32_to_bf16(acc[2]) | (f32_to_bf16(acc[3]) << 16);
     out.z = f32_to_bf16(acc[4]) | (f32_to_bf16(acc[5]) << 16);
     out.w = f32_to_bf16(acc[6]) | (f32_to_bf16(acc[7]) << 16);
-    st16_nt(reinterpret_cast<uint4 *>(a.combined + (static_cast<size_t>(r) * d.T + t) * d.H) + tid, out);
+    st16_nt(reinterpret_cast<uint4 *>(a.combined + (static_cast<size_t>(r) * d.T + t) * d.H) + col, out);
 }
 
 __global__ void
@@ -337,14 +442,32 @@ round_up_wave(int n) {
     return (n + kWaveSize - 1) / kWaveSize * kWaveSize;
 }
 
+// Largest workgroup (in lanes) of the dispatch and combine kernels; a token whose row needs
+// more lanes is split over several workgroups.
+int g_dispatch_lanes = 1024;
+int g_combine_lanes = 1024;
+
 } // namespace
 
 extern "C" {
 
+int
+nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes) {
+    auto ok = [](int v) { return v == 0 || (v >= 64 && v <= 1024 && v % 64 == 0); };
+    if (!ok(dispatch_lanes) || !ok(combine_lanes))
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_set_tuning: lanes must be 0 or a multiple of 64 in [64, 1024]");
+    if (dispatch_lanes) g_dispatch_lanes = dispatch_lanes;
+    if (combine_lanes) g_combine_lanes = combine_lanes;
+    return NIXL_AMD_OK;
+}
+
 size_t
-nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk) {
-    if (num_ranks <= 0 || num_experts <= 0 || num_tokens < 0 || num_topk <= 0) return 0;
-    return (static_cast<size_t>(num_ranks) * num_experts + static_cast<size_t>(num_ranks) * num_tokens * num_topk) * sizeof(int);
+nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk, int hidden) {
+    if (num_ranks <= 0 || num_experts <= 0 || num_tokens < 0 || num_topk <= 0 || hidden < 0) return 0;
+    const size_t counts = static_cast<size_t>(num_ranks) * num_experts * sizeof(int);
+    const size_t rows = static_cast<size_t>(num_ranks) * num_tokens * num_topk * sizeof(int);
+    const size_t scales = static_cast<size_t>(num_ranks) * num_tokens * (hidden / 128) * sizeof(float);
+    return counts + 2 * rows + scales; // positions and final rows are separate arrays
 }
 
 int
@@ -367,6 +490,7 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                         int use_fp8,
                         int round_scale,
                         int use_ue8m0,
+                        int *row_map,
                         void *workspace,
                         size_t workspace_bytes,
                         void *stream) {
@@ -382,42 +506,67 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
     if (use_fp8 && !packed_recv_x_scales) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: scales pointer is null");
     if (use_ue8m0 && !(use_fp8 && round_scale)) // kernels/nixl_ep_ll.cu:428-430
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: UE8M0 scales need use_fp8 and round_scale");
-    if (workspace_bytes < nixl_amd_ep_ll_workspace_bytes(num_ranks, num_experts, num_tokens, num_topk))
+    if (workspace_bytes < nixl_amd_ep_ll_workspace_bytes(num_ranks, num_experts, num_tokens, num_topk, hidden))
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: workspace too small");
+    if (reinterpret_cast<uintptr_t>(workspace) % 4 != 0)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: workspace must be 4-byte aligned");
+    if (static_cast<long long>(d.E) * d.N >= (1ll << 31))
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: num_experts * num_ranks * max tokens must be below 2^31");
+    if (static_cast<size_t>(d.E) * sizeof(int) > 48 * 1024 || static_cast<size_t>(d.R) * sizeof(int) > 48 * 1024)
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: too many experts or ranks");
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t n_sel = static_cast<size_t>(d.R) * d.T * d.K;
     int *send_count = static_cast<int *>(workspace);
-    int *pos = send_count + static_cast<size_t>(d.R) * d.E;
+    int *positions = send_count + static_cast<size_t>(d.R) * d.E;
+    int *rows_ws = positions + n_sel;
+    float *token_scales = reinterpret_cast<float *>(rows_ws + n_sel);
+    int *rows = row_map ? row_map : rows_ws;
 
     const int W = (d.T + 63) / 64 > 0 ? (d.T + 63) / 64 : 1;
     int per_pass = kLayoutLdsBytes / (W * 8);
     if (per_pass < 1) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: too many tokens per rank for the layout pass");
     if (per_pass > d.E) per_pass = d.E;
     hipLaunchKernelGGL(ll_layout_kernel, dim3(d.R), dim3(kLayoutThreads), static_cast<size_t>(per_pass) * W * 8, s, topk_idx,
-                       num_tokens_per_rank, mask_buffer, send_count, pos, d, per_pass);
+                       num_tokens_per_rank, mask_buffer, send_count, positions, d, per_pass);
     HIP_TRY(hipGetLastError());
 
-    DispatchArgs a{};
-    a.recv_x = static_cast<uint8_t *>(packed_recv_x);
-    a.recv_scales = packed_recv_x_scales;
-    a.src_info = packed_recv_src_info;
-    a.layout_range = reinterpret_cast<long long *>(packed_recv_layout_range);
-    a.recv_count = packed_recv_count;
-    a.stats = cumulative_local_expert_recv_stats;
-    a.x = static_cast<const uint16_t *>(x);
-    a.topk_idx = topk_idx;
-    a.num_tokens_per_rank = num_tokens_per_rank;
-    a.send_count = send_count;
-    a.pos = pos;
-    a.d = d;
-    a.round_scale = round_scale;
-    a.use_ue8m0 = use_ue8m0;
-    const dim3 grid(static_cast<unsigned>(d.R) + static_cast<unsigned>(d.R) * d.T);
-    const dim3 block(round_up_wave(d.H / 16));
-    if (use_fp8)
-        hipLaunchKernelGGL(ll_dispatch_kernel<true>, grid, block, 0, s, a);
-    else
-        hipLaunchKernelGGL(ll_dispatch_kernel<false>, grid, block, 0, s, a);
+    if (d.T > 0) {
+        DispatchArgs a{};
+        a.recv_x = static_cast<uint8_t *>(packed_recv_x);
+        a.src_info = packed_recv_src_info;
+        a.token_scales = token_scales;
+        a.x = static_cast<const uint16_t *>(x);
+        a.topk_idx = topk_idx;
+        a.num_tokens_per_rank = num_tokens_per_rank;
+        a.send_count = send_count;
+        a.rows = positions;
+        a.rows_out = rows;
+        a.d = d;
+        a.round_scale = round_scale;
+        const int wg = std::min(round_up_wave(d.H / 16), g_dispatch_lanes);
+        a.parts = (d.H / 16 + wg - 1) / wg;
+        const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
+        const dim3 block(wg);
+        if (use_fp8)
+            hipLaunchKernelGGL(ll_dispatch_kernel<true>, grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL(ll_dispatch_kernel<false>, grid, block, 0, s, a);
+        HIP_TRY(hipGetLastError());
+    }
+
+    ScalesArgs sa{};
+    sa.recv_scales = use_fp8 ? packed_recv_x_scales : nullptr;
+    sa.token_scales = token_scales;
+    sa.src_info = packed_recv_src_info;
+    sa.send_count = send_count;
+    sa.layout_range = reinterpret_cast<long long *>(packed_recv_layout_range);
+    sa.recv_count = packed_recv_count;
+    sa.stats = cumulative_local_expert_recv_stats;
+    sa.d = d;
+    sa.use_ue8m0 = use_ue8m0;
+    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * kScaleParts), dim3(kLayoutThreads),
+                       static_cast<size_t>(d.R) * sizeof(int), s, sa);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }
@@ -431,6 +580,7 @@ nixl_amd_ep_ll_combine(void *combined_x,
                        const int64_t *layout_range,
                        const int *mask_buffer,
                        const int *num_tokens_per_rank,
+                       const int *row_map,
                        int num_tokens,
                        int hidden,
                        int num_max_dispatch_tokens_per_rank,
@@ -456,8 +606,11 @@ nixl_amd_ep_ll_combine(void *combined_x,
     a.layout_range = reinterpret_cast<const long long *>(layout_range);
     a.mask = mask_buffer;
     a.num_tokens_per_rank = num_tokens_per_rank;
+    a.row_map = row_map;
     a.d = d;
-    hipLaunchKernelGGL(ll_combine_kernel, dim3(static_cast<unsigned>(d.R) * d.T), dim3(round_up_wave(d.H / 8)), 0,
+    const int wg = std::min(round_up_wave(d.H / 8), g_combine_lanes);
+    a.parts = (d.H / 8 + wg - 1) / wg;
+    hipLaunchKernelGGL(ll_combine_kernel, dim3(static_cast<unsigned>(d.R) * d.T * a.parts), dim3(wg), 0,
                        static_cast<hipStream_t>(stream), a);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;

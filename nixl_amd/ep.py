@@ -51,6 +51,14 @@ def _check(rc, what):
         raise EPError(f"{what}: {_lib.kernels_error()} (status {rc})")
 
 
+class DispatchHandle(tuple):
+    """The reference's dispatch handle (src_info, layout_range, num_max_dispatch_tokens_per_rank,
+    hidden) (nixl_ep/buffer.py:415-420), plus the row map the dispatch kernel recorded, which
+    lets combine skip its search.  A plain 4-tuple built by the caller works as well."""
+
+    row_map = None
+
+
 class Buffer:
     """All virtual ranks of one expert-parallel job on one GPU.
 
@@ -140,19 +148,21 @@ class Buffer:
                 scales = torch.empty((R, El, H // 512, N), dtype=torch.int32, device=dev)
             else:
                 scales = torch.empty((R, El, H // 128, N), dtype=torch.float32, device=dev)
-        ws_bytes = self._k.nixl_amd_ep_ll_workspace_bytes(R, num_experts, T, K)
+        row_map = torch.empty((R, T, K), dtype=torch.int32, device=dev)
+        ws_bytes = self._k.nixl_amd_ep_ll_workspace_bytes(R, num_experts, T, K, H)
         ws = self._get_workspace(ws_bytes)
         rc = self._k.nixl_amd_ep_ll_dispatch(
             _ptr(packed_recv_x), _ptr(scales), _ptr(packed_recv_src_info), _ptr(packed_recv_layout_range),
             _ptr(packed_recv_count), self._mask_ptr(), _ptr(cumulative_local_expert_recv_stats), _ptr(x),
             _ptr(topk_idx), _ptr(num_tokens_per_rank), T, H, num_max_dispatch_tokens_per_rank, K, R, num_experts,
-            int(use_fp8), int(round_scale), int(use_ue8m0), _ptr(ws), ws.numel(), _stream())
+            int(use_fp8), int(round_scale), int(use_ue8m0), _ptr(row_map), _ptr(ws), ws.numel(), _stream())
         _check(rc, "low_latency_dispatch")
         event = None
         if async_finish:
             event = torch.cuda.Event()
             event.record()
-        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H)
+        handle = DispatchHandle((packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H))
+        handle.row_map = row_map
         recv = (packed_recv_x, scales.transpose(2, 3)) if use_fp8 else packed_recv_x
         hook = (lambda: None) if return_recv_hook else None
         return recv, packed_recv_count, handle, EventOverlap(event), hook
@@ -181,8 +191,8 @@ class Buffer:
         combined = out if out is not None else torch.empty((R, T, hidden), dtype=torch.bfloat16, device=x.device)
         rc = self._k.nixl_amd_ep_ll_combine(
             _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
-            self._mask_ptr(), _ptr(num_tokens_per_rank), T, hidden, max_tok, K, R, num_experts, int(use_logfmt),
-            _stream())
+            self._mask_ptr(), _ptr(num_tokens_per_rank), _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K,
+            R, num_experts, int(use_logfmt), _stream())
         _check(rc, "low_latency_combine")
         event = None
         if async_finish:

@@ -1,0 +1,178 @@
+"""Timing of the expert-parallel kernels on the BASELINE shapes, used by bench.py.
+
+Method follows the reference's EP benchmark helper (examples/device/ep/tests/utils.py:
+116-143): device events around each call, a cache-flushing write of 512 MB before every
+timed call (the reference flushes 256 MB for a 50 MB L2; MI355X has a 256 MB last-level
+cache), warm-ups first, first sample dropped, average / min / max reported.  Byte counts
+are the algorithmic ones: each input row read once, each output row written once
+(reference formula for the low-latency mode: tests/elastic/elastic.py:424-432).
+"""
+import os
+import time
+
+import numpy as np
+import torch
+
+from .ep import Buffer
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def _timed(fn, flush, warmup, iters):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters + 1):
+        flush.fill_(1)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3)
+    times = np.array(times[1:])
+    return {"avg_us": round(float(times.mean()), 2), "min_us": round(float(times.min()), 2),
+            "max_us": round(float(times.max()), 2)}
+
+
+def _rate(nbytes, us):
+    gbps = nbytes / (us * 1e-6) / 1e9
+    return {"bytes": int(nbytes), "GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+
+
+def run_low_latency(dev, warmup=20, iters=50):
+    """BASELINE config 4: 32 virtual ranks x 128 tokens x 7168, 256 experts, top-8, fp8."""
+    R, T, H, K, E, M = 32, 128, 7168, 8, 256, 128
+    El, N = E // R, R * M
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn((R, T, H), generator=g, device=dev).to(torch.bfloat16)
+    logits = torch.randn((R, T, E), generator=g, device=dev)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    buf = Buffer(R, device=dev)
+    topk, w = buf.route(logits, K)
+    state = {}
+
+    def dispatch():
+        state["out"] = buf.dispatch(x, topk, M, E, use_fp8=True)
+
+    t_router = _timed(lambda: buf.route(logits, K), flush, warmup, iters)
+    t_dispatch = _timed(dispatch, flush, warmup, iters)
+    (q, sc_t), cnt, handle, _, _ = state["out"]
+    # expert step (not timed): dequantise, scale by (1 + 0.001 e), back to bf16
+    sc = sc_t.contiguous()
+    y = torch.zeros((R, El, N, H), dtype=torch.bfloat16, device=dev)
+    valid = torch.arange(N, device=dev).view(1, 1, -1) < cnt.unsqueeze(-1)
+    for d in range(R):
+        deq = (q[d].float().view(El, N, H // 128, 128) * sc[d].unsqueeze(-1)).view(El, N, H)
+        f = (1 + 0.001 * (d * El + torch.arange(El, device=dev, dtype=torch.float32))).view(El, 1, 1)
+        y[d] = torch.where(valid[d].unsqueeze(-1), (deq.to(torch.bfloat16).float() * f).to(torch.bfloat16), y[d])
+    del deq, sc
+    t_combine = _timed(lambda: buf.combine(y, topk, w, handle), flush, warmup, iters)
+
+    tokens, pairs = R * T, int((topk >= 0).sum())
+    meta = R * El * R * 8 + R * El * 4
+    dispatch_bytes = tokens * H * 2 + tokens * K * 4 + pairs * (H + H // 128 * 4 + 4) + meta
+    combine_bytes = pairs * H * 2 + tokens * K * 8 + tokens * H * 2
+    both_us = t_dispatch["avg_us"] + t_combine["avg_us"]
+    return {
+        "workload": f"{R} virtual ranks x {T} tokens x hidden {H}, {E} experts, top-{K}, fp8 e4m3 dispatch, bf16 combine",
+        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"])},
+        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
+        "dispatch_plus_combine_us": round(both_us, 2),
+        "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
+        "router": {**t_router, "bytes": tokens * E * 4},
+    }
+
+
+def zipf_topk(rng, R, T, K, E, s=1.2):
+    """K distinct experts per token from a Zipf(s) law over a seeded expert permutation
+    (Gumbel top-k), softmax weights over the drawn scores."""
+    perm = rng.permutation(E)
+    p = 1.0 / np.arange(1, E + 1) ** s
+    logp = np.log(p / p.sum())[np.argsort(perm)]
+    keys = logp[None, None, :] + rng.gumbel(size=(R, T, E))
+    topk = np.argsort(-keys, axis=2)[:, :, :K].astype(np.int32)
+    sel = np.take_along_axis(keys, topk, 2)
+    w = np.exp(sel - sel.max(2, keepdims=True))
+    return topk, (w / w.sum(2, keepdims=True)).astype(np.float32)
+
+
+def run_normal(dev, warmup=5, iters=20):
+    """BASELINE config 5: 8 virtual ranks x 4096 tokens x 7168, 256 experts, top-8, Zipf."""
+    R, T, H, K, E, C = 8, 4096, 7168, 8, 256, 10
+    rng = np.random.default_rng(5)
+    topk_h, w_h = zipf_topk(rng, R, T, K, E)
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn((R, T, H), generator=g, device=dev).to(torch.bfloat16)
+    topk, w = torch.from_numpy(topk_h).to(dev), torch.from_numpy(w_h).to(dev)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    buf = Buffer(R, low_latency_mode=False, device=dev)
+    state = {}
+
+    def layout():
+        state["layout"] = buf.get_dispatch_layout(topk, E)
+
+    def dispatch():
+        per_rank, _, per_expert, in_rank, _ = state["layout"]
+        state["out"] = buf.ht_dispatch(x, num_tokens_per_rank=per_rank, is_token_in_rank=in_rank,
+                                       num_tokens_per_expert=per_expert, topk_idx=topk, topk_weights=w, num_channels=C)
+
+    t_layout = _timed(layout, flush, warmup, iters)
+    t_dispatch = _timed(dispatch, flush, warmup, iters)
+    recv_x, recv_idx, recv_w, per_expert_list, handle, _ = state["out"]
+    rows = recv_x.shape[0]
+    coef = (recv_w * (recv_idx >= 0)).sum(1, keepdim=True)
+    y = (recv_x.float() * coef).to(torch.bfloat16)
+    t_combine = _timed(lambda: buf.ht_combine(y, handle, topk_weights=recv_w), flush, warmup, iters)
+    tokens = R * T
+    dispatch_bytes = tokens * H * 2 + rows * H * 2 + tokens * K * 8 + rows * (K * 8 + 8) + tokens * K * 4 + tokens * R
+    combine_bytes = rows * H * 2 + rows * K * 4 + tokens * H * 2 + tokens * K * 4
+    counts = np.array(per_expert_list).reshape(-1)
+    return {
+        "workload": f"{R} virtual ranks x {T} tokens x hidden {H}, {E} experts, top-{K}, Zipf(1.2) expert popularity, bf16",
+        "rows_received": int(rows),
+        "expert_load": {"max": int(counts.max()), "mean": round(float(counts.mean()), 1), "min": int(counts.min())},
+        "layout": t_layout,
+        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]),
+                     "note": "includes the host read-back of the receive counts that sizes recv_x"},
+        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
+    }
+
+
+def run_cpu_baseline(seconds=10.0):
+    """Scalar CPU restatement of the low-latency kernels (the oracle), one thread, on a
+    bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8, fp8."""
+    from oracle import ep_oracle as eo
+    R, T, H, K, E, M = 4, 128, 7168, 8, 32, 128
+    rng = np.random.default_rng(4)
+    x = eo.f32_to_bf16(rng.standard_normal((R, T, H)).astype(np.float32))
+    logits = rng.standard_normal((R * T, E)).astype(np.float32)
+    topk, w = eo.router(logits, K)
+    topk, w = topk.reshape(R, T, K), w.reshape(R, T, K)
+    t0 = time.perf_counter()
+    n = 0
+    d_us, c_us = [], []
+    while time.perf_counter() - t0 < seconds or n < 2:
+        a = time.perf_counter()
+        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True)
+        b = time.perf_counter()
+        y = np.zeros((R, E // R, R * M, H), np.uint16)
+        c = time.perf_counter()
+        eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M)
+        d = time.perf_counter()
+        d_us.append((b - a) * 1e6)
+        c_us.append((d - c) * 1e6)
+        n += 1
+    return {"dispatch_us": round(float(np.mean(d_us)), 1), "combine_us": round(float(np.mean(c_us)), 1),
+            "cores": 1, "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
+                      "(1/8 of the GPU workload's tokens)"}
+
+
+def run(args):
+    dev = torch.device("cuda:0")
+    out = {"low_latency": run_low_latency(dev), "normal": run_normal(dev)}
+    if not getattr(args, "no_cpu_baseline", False):
+        out["cpu_baseline"] = run_cpu_baseline()
+    return out

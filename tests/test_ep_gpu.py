@@ -53,10 +53,10 @@ def raw_ll_dispatch(cuda, x, topk, E, M, use_fp8, round_scale=False, use_ue8m0=F
     src_info = torch.full((R, El, N, 4), fill, dtype=torch.uint8, device=cuda)
     layout = torch.zeros((R, El, R), dtype=torch.int64, device=cuda)
     count = torch.zeros((R, El), dtype=torch.int32, device=cuda)
-    ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K) + 16, dtype=torch.uint8, device=cuda)
+    ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K, H) + 16, dtype=torch.uint8, device=cuda)
     p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
     rc = k.nixl_amd_ep_ll_dispatch(p(recv_x), p(scales), p(src_info), p(layout), p(count), p(md), p(stats), p(xd), p(td),
-                                   p(ntd), T, H, M, K, R, E, int(use_fp8), int(round_scale), int(use_ue8m0), p(ws),
+                                   p(ntd), T, H, M, K, R, E, int(use_fp8), int(round_scale), int(use_ue8m0), None, p(ws),
                                    ws.numel(), None)
     torch.cuda.synchronize()
     return rc, dict(recv_x=recv_x.cpu().numpy(), scales=None if scales is None else scales.cpu().numpy(),
@@ -180,8 +180,11 @@ def test_ll_combine_matches_oracle(cuda, shape):
     y = torch.where(valid, (rx.float() * factor).to(torch.bfloat16), torch.zeros_like(rx))
     comb = torch.full((R, T, H), 7.0, dtype=torch.bfloat16, device=cuda)
     out, _, _ = buf.combine(y, td, wd, handle, out=comb, num_tokens_per_rank=ntd)
+    # the same through a plain tuple handle: rows are then found by searching src_info
+    searched, _, _ = buf.combine(y, td, wd, tuple(handle), out=comb.clone(), num_tokens_per_rank=ntd)
     torch.cuda.synchronize()
-    assert out is comb
+    assert out is comb and handle.row_map is not None
+    assert torch.equal(searched.view(torch.int16), comb.view(torch.int16))
     si, lr = handle[0].cpu().numpy(), handle[1].cpu().numpy()
     want = eo.ll_combine(bits16(y).reshape(R, El, R * M, H), topk, w, si, lr, E, M, num_tokens=nt, use_fma=True)
     got = bits16(comb).reshape(R, T, H)
