@@ -512,3 +512,89 @@ def test_router_matches_oracle(cuda):
         assert np.allclose(w.cpu().numpy(), ow, rtol=2e-6, atol=0)
     with pytest.raises(EPError):
         buf.route(torch.zeros((4, 2000), device=cuda), 2)
+
+
+# ---- committed golden vectors (tests/golden, independent of the oracle) ---------------------------
+
+def _golden(name):
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name), allow_pickle=False)
+
+
+def test_golden_encoder_and_router(cuda):
+    g = _golden("e4m3_encode.npz")
+    v = np.concatenate([g["values"], g["sat_values"]])
+    vin = torch.from_numpy(v).to(cuda)
+    out = torch.empty(v.size, dtype=torch.uint8, device=cuda)
+    rc = _lib.ep_kernels().nixl_amd_ep_f32_to_e4m3(ctypes.c_void_p(vin.data_ptr()), ctypes.c_void_p(out.data_ptr()), v.size, None)
+    assert rc == 0, _lib.kernels_error()
+    assert np.array_equal(out.cpu().numpy(), np.concatenate([g["codes"], g["sat_codes"]]))
+    r = _golden("router.npz")
+    idx, w = Buffer(2, device=cuda).route(torch.from_numpy(r["logits"]).to(cuda), r["topk_idx"].shape[1])
+    assert np.array_equal(idx.cpu().numpy(), r["topk_idx"])
+    assert np.allclose(w.cpu().numpy(), r["topk_weights"], rtol=2e-6, atol=0)
+
+
+def test_golden_low_latency_world(cuda):
+    g = _golden("ll_world.npz")
+    E, M = int(g["num_experts"]), int(g["max_tok"])
+    R, T, H = g["x"].shape
+    El, N = E // R, R * M
+    x = torch.from_numpy(g["x"].view(np.int16)).view(torch.bfloat16)
+    for use_fp8 in (True, False):
+        rc, got = raw_ll_dispatch(cuda, x, g["topk_idx"], E, M, use_fp8, num_tokens=g["num_tokens"])
+        assert rc == 0, _lib.kernels_error()
+        assert np.array_equal(got["recv_count"], g["recv_count"])
+        assert np.array_equal(got["layout_range"], g["layout_range"])
+        rx = got["recv_x"].reshape(R, El, N, -1)
+        want = g["recv_fp8"] if use_fp8 else g["recv_bf16"].view(np.uint8).reshape(R, El, N, -1)
+        si = got["src_info"].view(np.int32).reshape(R, El, N)
+        for d in range(R):
+            for le in range(El):
+                n = int(g["recv_count"][d, le])
+                assert np.array_equal(rx[d, le, :n], want[d, le, :n])
+                assert np.array_equal(si[d, le, :n], g["src_info"][d, le, :n])
+                if use_fp8:
+                    sc = got["scales"].view(np.uint32).reshape(R, El, H // 128, N)
+                    assert np.array_equal(sc[d, le, :, :n], g["scales"][d, le, :, :n].view(np.uint32))
+    # combine from the fixture's own handle (rows located through src_info / layout_range)
+    buf = Buffer(R, device=cuda)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+    y = dev(g["expert_out"].view(np.int16)).view(torch.bfloat16)
+    handle = (dev(g["src_info"]), dev(g["layout_range"]), M, H)
+    out, _, _ = buf.combine(y, dev(g["topk_idx"]), dev(g["topk_weights"]), handle, num_tokens_per_rank=dev(g["num_tokens"]))
+    torch.cuda.synchronize()
+    got = bits16(out).reshape(R, T, H)
+    for r, n in enumerate(g["num_tokens"]):
+        assert np.array_equal(got[r, :n], g["combined"][r, :n])
+
+
+def test_golden_normal_mode_world(cuda):
+    g = _golden("ht_world.npz")
+    R, T, K = g["topk_idx"].shape
+    E, C = int(g["num_experts"]), int(g["num_channels"])
+    H = g["x"].shape[2]
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+    bf = lambda a: dev(a.view(np.int16)).view(torch.bfloat16)
+    buf = Buffer(R, low_latency_mode=False, device=cuda)
+    td, wd = dev(g["topk_idx"]), dev(g["topk_weights"])
+    per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(td, E)
+    assert np.array_equal(per_rank.cpu().numpy(), g["per_rank"])
+    assert np.array_equal(per_expert.cpu().numpy(), g["per_expert"])
+    assert np.array_equal(in_rank.cpu().numpy().astype(np.uint8), g["in_rank"])
+    recv_x, recv_idx, recv_w, per_expert_list, handle, _ = buf.ht_dispatch(
+        bf(g["x"]), num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert,
+        topk_idx=td, topk_weights=wd, num_channels=C)
+    _, prefix, chan, meta, send_head, row_offset = handle
+    assert np.array_equal(prefix.cpu().numpy(), g["prefix"])
+    assert np.array_equal(chan.cpu().numpy(), g["channel_prefix"])
+    assert per_expert_list == g["expert_count"].tolist()
+    assert np.array_equal(row_offset.cpu().numpy(), g["row_offset"])
+    assert np.array_equal(send_head.cpu().numpy(), g["send_head"])
+    assert np.array_equal(bits16(recv_x).reshape(-1, H), g["recv_x"])
+    assert np.array_equal(recv_idx.cpu().numpy(), g["recv_topk_idx"])
+    assert np.array_equal(recv_w.cpu().numpy(), g["recv_topk_weights"])
+    assert np.array_equal(meta.cpu().numpy(), g["recv_src_meta"])
+    comb, comb_w, _ = buf.ht_combine(recv_x, handle, topk_weights=recv_w, bias=(bf(g["bias0"]), bf(g["bias1"])))
+    assert np.array_equal(bits16(comb).reshape(R, T, H), g["combined"])
+    assert np.array_equal(comb_w.cpu().numpy(), g["combined_topk_weights"])

@@ -354,3 +354,19 @@ def test_config3_small_descriptor_stress_full_size(hip_agent, cuda):
     assert diff == 0, f"{diff} of {buf_bytes // 8} 8-byte words differ"
     for h in (req, hl, hr):
         h.release()
+
+
+def test_golden_descriptor_list(cuda):
+    """Committed vector (tests/golden/kv_descs.npz): mixed aligned / unaligned / empty
+    descriptors, destination pre-filled with a canary byte."""
+    import os
+    import torch
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kv_descs.npz"), allow_pickle=False)
+    src = torch.from_numpy(g["src"]).to(cuda)
+    dst = torch.full((g["src"].size,), int(g["canary"]), dtype=torch.uint8, device=cuda)
+    plan = _plan([(src.data_ptr() + int(s), dst.data_ptr() + int(d), int(n))
+                  for s, d, n in zip(g["src_off"], g["dst_off"], g["lens"])])
+    _run_plan(torch, plan)
+    assert _lib.kernels().nixl_amd_copy_plan_destroy(plan) == 0
+    assert np.array_equal(dst.cpu().numpy(), g["dst"])
+    assert np.array_equal(src.cpu().numpy(), g["src"])
