@@ -140,6 +140,18 @@ def run_kv(args):
     return out
 
 
+def run_calibration_copy():
+    """One launch of torch's element-wise add over 2^28 int32: reads exactly 1 GiB, writes 1 GiB."""
+    import torch
+    a = torch.ones(1 << 28, dtype=torch.int32, device="cuda:0")
+    b = torch.empty_like(a)
+    torch.cuda.synchronize()
+    torch.add(a, 1, out=b)
+    torch.cuda.synchronize()
+    del a, b
+    torch.cuda.empty_cache()
+
+
 def run_cpu_baseline(seconds=12.0):
     """Reference-shaped CPU path: one agent, loopback, DRAM->DRAM, one memcpy per descriptor
     (the semantics of the reference's UCX loopback puts, src/plugins/ucx/ucx_backend.cpp:
@@ -203,6 +215,11 @@ def main():
     ap.add_argument("--block-bytes", type=int, default=32768, help="bytes per (layer, K|V) sub-block")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ep", action="store_true")
+    ap.add_argument("--ep-iters", type=int, default=50, help="timed calls per expert-parallel kernel")
+    ap.add_argument("--ep-warmup", type=int, default=20)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain element-wise kernel that reads 1 GiB and writes 1 GiB, as the "
+                         "known-size yardstick for hardware counter runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (virtual ranks are regions of one "
@@ -211,6 +228,8 @@ def main():
     import __graft_entry__ as entry
     entry._ensure_built()
 
+    if args.calibrate_copy:
+        run_calibration_copy()
     kv = run_kv(args)
     line = {
         "metric": "KV xfer GB/s (% HBM peak) @16KB blocks; EP dispatch+combine µs @7168 top-8",

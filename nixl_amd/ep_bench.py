@@ -172,7 +172,9 @@ def run_cpu_baseline(seconds=10.0):
 
 def run(args):
     dev = torch.device("cuda:0")
-    out = {"low_latency": run_low_latency(dev), "normal": run_normal(dev)}
+    warmup, iters = getattr(args, "ep_warmup", 20), getattr(args, "ep_iters", 50)
+    out = {"low_latency": run_low_latency(dev, warmup, iters),
+           "normal": run_normal(dev, max(warmup // 4, 1), max(iters // 2, 1))}
     if not getattr(args, "no_cpu_baseline", False):
         out["cpu_baseline"] = run_cpu_baseline()
     return out
