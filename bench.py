@@ -29,6 +29,12 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 
+# HBM bytes per launch of the copy kernel from hardware counters (FETCH_SIZE and WRITE_SIZE,
+# one rocprofv3 --pmc run each, scaled by a plain 1 GiB element-wise kernel in the same run;
+# profiles/copy_uniform_kernel_kv_llama3_32KiB.txt).  Keyed by (blocks, pool blocks, block
+# bytes); counters cannot be read from inside this process, so other shapes report null.
+MEASURED_TRAFFIC_BYTES = {(1024, 8192, 32768): 4563374659}
+
 
 def _kv_descs(base, layers, pool_blocks, blk, block_ids):
     """One descriptor per (block, layer, K|V) in a pool laid out [layer][K|V][block][blk]."""
@@ -124,7 +130,8 @@ def run_kv(args):
         "value": payload_per_step * args.steps / wall / 1e9,
         "ms_per_step": wall / args.steps * 1e3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((n_sel, pool_blocks, blk)),
                      "kernel": "copy_uniform_kernel<1,true,1>",
                      "avg_launch_ms": round(avg_launch_ms, 4),
                      "gather_ms": round(float(np.mean(kernel_ms[0::2])), 4),

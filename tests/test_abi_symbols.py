@@ -3,7 +3,7 @@
 No compute call is made here.  The C headers are parsed for their function declarations;
 the C++ agent header for its nixlAgent member functions; the plugin library is checked
 for the two discovery symbols the reference's plugin manager resolves
-(src/core/nixl_plugin_manager.cpp:164-193).
+(src/core/nixl_plugin_manager.cpp:46-51,94-122).
 """
 import ctypes
 import os
