@@ -91,17 +91,22 @@ logical_workgroup(uint32_t n_wgs, bool swizzle) {
     return (b % kNumXcd) * per + b / kNumXcd; // may be >= n_wgs; caller checks
 }
 
-// One wavefront per full, single-descriptor chunk.
+// One wavefront per full, single-descriptor chunk.  A record covers `chunks_per_rec`
+// consecutive chunks of one descriptor (1 when the runs of such chunks differ in length;
+// with equal-length descriptors, e.g. KV blocks, one record per descriptor), so that the
+// record array stays small next to the payload.
 template<int UPL, bool NT, int WAVES>
 __global__ void __launch_bounds__(kWaveSize *WAVES)
-copy_uniform_kernel(const UniformRec *recs, uint32_t n_recs, uint32_t n_wgs, int swizzle) {
+copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, int swizzle, uint32_t chunks_per_rec) {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = threadIdx.x / kWaveSize;
     const uint32_t wg = logical_workgroup(n_wgs, swizzle != 0);
-    const uint32_t r = uniform(wg * WAVES + wave);
-    if (wg >= n_wgs || r >= n_recs) return;
-    const uint64_t s = uniform64(recs[r].src) + lane * 16u;
-    const uint64_t d = uniform64(recs[r].dst) + lane * 16u;
+    const uint32_t c = uniform(wg * WAVES + wave);
+    if (wg >= n_wgs || c >= n_chunks) return;
+    const uint32_t r = c / chunks_per_rec;
+    const uint64_t off = static_cast<uint64_t>(c % chunks_per_rec) * (kWaveSize * UPL * 16u) + lane * 16u;
+    const uint64_t s = uniform64(recs[r].src) + off;
+    const uint64_t d = uniform64(recs[r].dst) + off;
     v4u v[UPL];
 #pragma unroll
     for (int k = 0; k < UPL; ++k)
@@ -235,25 +240,25 @@ copy_generic_kernel(const GenericItem *items, uint32_t n_items) {
 
 template<int UPL, bool NT>
 void
-launch_uniform(int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz) {
+launch_uniform(int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz, uint32_t cpr) {
     switch (waves) {
-    case 1: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 1>), grid, dim3(64), 0, s, recs, n, n_wgs, swz); break;
-    case 2: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 2>), grid, dim3(128), 0, s, recs, n, n_wgs, swz); break;
-    case 4: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 4>), grid, dim3(256), 0, s, recs, n, n_wgs, swz); break;
-    case 8: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 8>), grid, dim3(512), 0, s, recs, n, n_wgs, swz); break;
-    default: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 16>), grid, dim3(1024), 0, s, recs, n, n_wgs, swz); break;
+    case 1: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 1>), grid, dim3(64), 0, s, recs, n, n_wgs, swz, cpr); break;
+    case 2: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 2>), grid, dim3(128), 0, s, recs, n, n_wgs, swz, cpr); break;
+    case 4: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 4>), grid, dim3(256), 0, s, recs, n, n_wgs, swz, cpr); break;
+    case 8: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 8>), grid, dim3(512), 0, s, recs, n, n_wgs, swz, cpr); break;
+    default: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 16>), grid, dim3(1024), 0, s, recs, n, n_wgs, swz, cpr); break;
     }
 }
 
 template<bool NT>
 void
-launch_uniform_upl(int upl, int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz) {
+launch_uniform_upl(int upl, int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz, uint32_t cpr) {
     switch (upl) {
-    case 1: launch_uniform<1, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
-    case 2: launch_uniform<2, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
-    case 4: launch_uniform<4, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
-    case 8: launch_uniform<8, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
-    default: launch_uniform<16, NT>(waves, grid, s, recs, n, n_wgs, swz); break;
+    case 1: launch_uniform<1, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
+    case 2: launch_uniform<2, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
+    case 4: launch_uniform<4, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
+    case 8: launch_uniform<8, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
+    default: launch_uniform<16, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
     }
 }
 
@@ -283,7 +288,8 @@ struct nixl_amd_copy_plan {
     void *arena = nullptr;
     size_t arena_bytes = 0;
     const UniformRec *uniform_recs = nullptr;
-    uint32_t n_uniform = 0;
+    uint32_t n_uniform = 0; // uniform chunks
+    uint32_t chunks_per_rec = 1;
     uint32_t uniform_wgs = 0;
     MixedArgs mixed_args{};
     uint32_t mixed_wgs = 0;
@@ -373,6 +379,19 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     std::vector<UniformRec> uni;
     std::vector<uint32_t> mixed;
     uni.reserve(n_chunks);
+    // Runs of consecutive uniform chunks inside one descriptor: if all runs have the same
+    // length L, one record per run is kept and the kernel derives the rest.
+    uint32_t run_len = 0, common_run = 0;
+    bool runs_equal = true;
+    size_t run_desc = ~size_t(0);
+    auto close_run = [&]() {
+        if (run_len == 0) return;
+        if (common_run == 0)
+            common_run = run_len;
+        else if (common_run != run_len)
+            runs_equal = false;
+        run_len = 0;
+    };
     {
         size_t j = 0;
         for (uint32_t c = 0; c < n_chunks; ++c) {
@@ -386,11 +405,25 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             span[c] = make_uint2(static_cast<uint32_t>(j), static_cast<uint32_t>(jl));
             if (j == jl && last - first + 1 == chunk_units) {
                 const uint64_t off = (first - vprefix[j]) * 16u;
+                if (run_len && run_desc != j) close_run();
+                run_desc = j;
+                ++run_len;
                 uni.push_back(UniformRec{vsrc[j] + off, vdst[j] + off});
             } else {
+                close_run();
                 mixed.push_back(c);
             }
         }
+        close_run();
+    }
+    const uint32_t n_uniform_chunks = static_cast<uint32_t>(uni.size());
+    uint32_t chunks_per_rec = 1;
+    if (runs_equal && common_run > 1) {
+        chunks_per_rec = common_run;
+        size_t w = 0;
+        for (size_t i = 0; i < uni.size(); i += common_run)
+            uni[w++] = uni[i];
+        uni.resize(w);
     }
 
     // ---- one device arena for all plan arrays --------------------------------------
@@ -446,7 +479,8 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         plan->mixed_args.chunks = reinterpret_cast<const uint32_t *>(base + off_mixed);
         plan->generic_items = reinterpret_cast<const GenericItem *>(base + off_items);
     }
-    plan->n_uniform = static_cast<uint32_t>(uni.size());
+    plan->n_uniform = n_uniform_chunks;
+    plan->chunks_per_rec = chunks_per_rec;
     plan->mixed_args.total_units = units;
     plan->mixed_args.n_mixed = static_cast<uint32_t>(mixed.size());
     plan->n_generic = static_cast<uint32_t>(items.size());
@@ -486,10 +520,10 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
         if (plan->swizzle) grid = ((grid + kNumXcd - 1) / kNumXcd) * kNumXcd;
         if (plan->nt)
             launch_uniform_upl<true>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
-                                     plan->uniform_wgs, plan->swizzle);
+                                     plan->uniform_wgs, plan->swizzle, plan->chunks_per_rec);
         else
             launch_uniform_upl<false>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
-                                      plan->uniform_wgs, plan->swizzle);
+                                      plan->uniform_wgs, plan->swizzle, plan->chunks_per_rec);
         HIP_TRY(hipGetLastError());
     }
     if (plan->mixed_wgs) {

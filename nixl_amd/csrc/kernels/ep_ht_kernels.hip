@@ -82,8 +82,8 @@ layout_kernel(const int32_t *__restrict__ topk_idx,
         per_rank[static_cast<size_t>(src) * R + i] = counters[E + i];
 }
 
-// ---- notify, part 1: per source rank, positions inside each (src -> dst) segment and the
-// per-channel prefix (kernels/nixl_ep_ht.cu:324-373) ----------------------------------------
+// ---- notify, part 1: per (source, destination) pair, positions inside the segment and the
+// per-channel prefix (kernels/nixl_ep_ht.cu:324-373).  grid = R * R workgroups. ----------------
 __global__ void __launch_bounds__(kScanThreads)
 ht_scan_kernel(const uint8_t *__restrict__ in_rank,
                int *__restrict__ send_head,
@@ -92,32 +92,30 @@ ht_scan_kernel(const uint8_t *__restrict__ in_rank,
                int R,
                int C) {
     __shared__ int wave_sums[kScanThreads / kWaveSize];
-    const int src = blockIdx.x;
+    const int src = blockIdx.x / R, d = blockIdx.x % R;
     const int per_thread = (T + kScanThreads - 1) / kScanThreads;
     const int t0 = min(static_cast<int>(threadIdx.x) * per_thread, T), t1 = min(t0 + per_thread, T);
     const int per_channel = (T + C - 1) / C;
-    for (int d = 0; d < R; ++d) {
-        int mine = 0;
-        for (int t = t0; t < t1; ++t)
-            mine += in_rank[(static_cast<size_t>(src) * T + t) * R + d];
-        int total;
-        int pos = block_exclusive_scan(mine, wave_sums, total);
-        for (int t = t0; t < t1; ++t) {
-            const bool hit = in_rank[(static_cast<size_t>(src) * T + t) * R + d] != 0;
-            send_head[(static_cast<size_t>(src) * T + t) * R + d] = hit ? pos : -1;
-            pos += hit;
-            // `pos` is now the number of hits in tokens [0, t]; a channel's inclusive prefix
-            // is that number at the channel's last token.
-            if ((t + 1) % per_channel == 0 || t + 1 == T) {
-                const int c = t / per_channel;
-                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = pos;
-            }
+    int mine = 0;
+    for (int t = t0; t < t1; ++t)
+        mine += in_rank[(static_cast<size_t>(src) * T + t) * R + d] != 0;
+    int total;
+    int pos = block_exclusive_scan(mine, wave_sums, total);
+    for (int t = t0; t < t1; ++t) {
+        const bool hit = in_rank[(static_cast<size_t>(src) * T + t) * R + d] != 0;
+        send_head[(static_cast<size_t>(src) * T + t) * R + d] = hit ? pos : -1;
+        pos += hit;
+        // `pos` is now the number of hits in tokens [0, t]; a channel's inclusive prefix
+        // is that number at the channel's last token.
+        if ((t + 1) % per_channel == 0 || t + 1 == T) {
+            const int c = t / per_channel;
+            channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = pos;
         }
-        // channels that start at or beyond T are empty: they repeat the grand total
-        if (threadIdx.x == 0)
-            for (int c = (T + per_channel - 1) / per_channel; c < C; ++c)
-                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = total;
     }
+    // channels that start at or beyond T are empty: they repeat the grand total
+    if (threadIdx.x == 0)
+        for (int c = (T + per_channel - 1) / per_channel; c < C; ++c)
+            channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = total;
 }
 
 // ---- notify, part 2: receive-side prefix over source ranks and aligned per-expert counts
@@ -158,6 +156,45 @@ recv_row(const int *prefix, const int *send_head, const long long *row_offset, c
     return row_offset[dst] + seg + send_head[(static_cast<size_t>(r) * d.T + t) * d.R + dst];
 }
 
+constexpr int kMaxHtRanks = 1024;
+constexpr int kHtBatch = 8; // row loads a lane keeps in flight in combine
+
+// The rows of token (r, t) at the destination ranks that hold it, in ascending rank order,
+// gathered into LDS by the first wave (64 destinations per step, compacted with a ballot).
+// Every thread of the workgroup calls this; the return value is the number of rows.
+__device__ __forceinline__ int
+collect_rows(const uint8_t *in_rank,
+             const int *prefix,
+             const int *send_head,
+             const long long *row_offset,
+             const HtDims &d,
+             int r,
+             int t,
+             long long *rows,
+             int *dsts,
+             int *n_rows) {
+    if (threadIdx.x < kWaveSize) {
+        const int lane = threadIdx.x;
+        const size_t tok = static_cast<size_t>(r) * d.T + t;
+        int n = 0;
+        for (int d0 = 0; d0 < d.R; d0 += kWaveSize) {
+            const int dst = d0 + lane;
+            const bool hit = dst < d.R && in_rank[tok * d.R + dst] != 0;
+            const long long row = hit ? recv_row(prefix, send_head, row_offset, d, r, t, dst) : 0;
+            const unsigned long long m = __ballot(hit);
+            if (hit) {
+                const int p = n + __popcll(m & ((1ull << lane) - 1ull));
+                rows[p] = row;
+                dsts[p] = dst;
+            }
+            n += __popcll(m);
+        }
+        if (lane == 0) *n_rows = n;
+    }
+    __syncthreads();
+    return *n_rows;
+}
+
 // ---- dispatch (result of kernels/nixl_ep_ht.cu:1109-1243) -------------------------------------
 // grid = R*T; block = H/8 lanes rounded up to whole waves (16 bytes of a row per lane).
 __global__ void __launch_bounds__(1024)
@@ -173,6 +210,9 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
                    const int *__restrict__ send_head,
                    const long long *__restrict__ row_offset,
                    HtDims d) {
+    __shared__ long long rows[kMaxHtRanks];
+    __shared__ int dsts[kMaxHtRanks];
+    __shared__ int n_rows;
     const int tid = threadIdx.x;
     const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
     const size_t tok = static_cast<size_t>(r) * d.T + t;
@@ -186,11 +226,12 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
         sel = topk_idx[tok * d.K + tid];
         w = topk_weights ? topk_weights[tok * d.K + tid] : 0.f;
     }
-    for (int dst = 0; dst < d.R; ++dst) {
-        if (!in_rank[tok * d.R + dst]) continue; // uniform over the workgroup
-        const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+    const int n = collect_rows(in_rank, prefix, send_head, row_offset, d, r, t, rows, dsts, &n_rows);
+    for (int i = 0; i < n; ++i) {
+        const long long row = rows[i];
         if (active) st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(row) * d.H) + tid, v);
         if (tid < d.K && recv_topk_idx) {
+            const int dst = dsts[i];
             const bool local = sel >= dst * El && sel < (dst + 1) * El;
             recv_topk_idx[row * d.K + tid] = local ? sel - dst * El : -1;
             if (recv_topk_weights) recv_topk_weights[row * d.K + tid] = local ? w : 0.f;
@@ -215,15 +256,21 @@ ht_combine_kernel(uint16_t *__restrict__ combined,
                   const int *__restrict__ send_head,
                   const long long *__restrict__ row_offset,
                   HtDims d) {
+    __shared__ long long rows[kMaxHtRanks];
+    __shared__ int dsts[kMaxHtRanks];
+    __shared__ int n_rows;
     const int tid = threadIdx.x;
     const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
     const size_t tok = static_cast<size_t>(r) * d.T + t;
     const bool active = tid < d.H / 8;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint4 b0 = make_uint4(0, 0, 0, 0), b1 = b0;
     if (active) {
-        uint4 b0 = make_uint4(0, 0, 0, 0), b1 = b0;
         if (bias0) b0 = ld16_nt(reinterpret_cast<const uint4 *>(bias0 + tok * d.H) + tid);
         if (bias1) b1 = ld16_nt(reinterpret_cast<const uint4 *>(bias1 + tok * d.H) + tid);
+    }
+    const int n = collect_rows(in_rank, prefix, send_head, row_offset, d, r, t, rows, dsts, &n_rows);
+    float acc[8];
+    {
         const uint32_t u0[4] = {b0.x, b0.y, b0.z, b0.w}, u1[4] = {b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -232,19 +279,31 @@ ht_combine_kernel(uint16_t *__restrict__ combined,
         }
     }
     float wsum = 0.f;
-    for (int dst = 0; dst < d.R; ++dst) {
-        if (!in_rank[tok * d.R + dst]) continue;
-        const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
-        if (active) {
-            const uint4 v = ld16_nt(reinterpret_cast<const uint4 *>(x + static_cast<size_t>(row) * d.H) + tid);
-            const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    for (int i0 = 0; i0 < n; i0 += kHtBatch) {
+        // all loads of the batch first, then the additions in ascending rank order
+        uint4 v[kHtBatch];
+        float wv[kHtBatch];
+#pragma unroll
+        for (int j = 0; j < kHtBatch; ++j) {
+            v[j] = make_uint4(0, 0, 0, 0);
+            wv[j] = 0.f;
+            if (i0 + j < n) {
+                const long long row = rows[i0 + j];
+                if (active) v[j] = ld16_nt(reinterpret_cast<const uint4 *>(x + static_cast<size_t>(row) * d.H) + tid);
+                if (topk_weights && tid < d.K) wv[j] = topk_weights[row * d.K + tid];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kHtBatch; ++j) {
+            if (i0 + j >= n) continue;
+            const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 acc[2 * c] += bf16_lo_to_f32(u[c]);
                 acc[2 * c + 1] += bf16_hi_to_f32(u[c]);
             }
+            wsum += wv[j];
         }
-        if (topk_weights && tid < d.K) wsum += topk_weights[row * d.K + tid];
     }
     if (active) {
         uint4 out;
@@ -381,7 +440,7 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
         !gbl_channel_prefix_matrix || !send_head)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_notify_dispatch: null pointer argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(ht_scan_kernel, dim3(num_ranks), dim3(kScanThreads), 0, s, is_token_in_rank, send_head,
+    hipLaunchKernelGGL(ht_scan_kernel, dim3(static_cast<unsigned>(num_ranks) * num_ranks), dim3(kScanThreads), 0, s, is_token_in_rank, send_head,
                        gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
     HIP_TRY(hipGetLastError());
     const int n = num_experts > num_ranks ? num_experts : num_ranks;

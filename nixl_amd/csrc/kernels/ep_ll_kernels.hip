@@ -141,6 +141,17 @@ ll_dispatch_kernel(DispatchArgs a) {
     const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
     if (t >= nt) return;
 
+    // The row is requested first so that it travels while the rows are being located.
+    const int lane = part * blockDim.x + tid; // lane of the token's row
+    const bool active = lane < d.H / 16;
+    uint4 raw0 = make_uint4(0, 0, 0, 0), raw1 = raw0;
+    if (active) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.x + (static_cast<size_t>(r) * d.T + t) * d.H) + lane * 2;
+        raw0 = ld16_nt(src);
+        raw1 = ld16_nt(src + 1);
+    }
+
+
     // Final row of selection k: e * N + (tokens the lower source ranks send to e) + position.
     // Half a wave per selection: its 32 lanes fetch the lower ranks' counts in parallel.
     for (int k = tid >> 5; k < d.K; k += blockDim.x >> 5) {
@@ -159,15 +170,6 @@ ll_dispatch_kernel(DispatchArgs a) {
         partial += __shfl_xor(partial, 1);
         if (q0 == 0) row_of_k[k] = p >= 0 ? e * d.N + partial + p : -1;
     }
-    const int lane = part * blockDim.x + tid; // lane of the token's row
-    const bool active = lane < d.H / 16;
-    uint4 raw0 = make_uint4(0, 0, 0, 0), raw1 = raw0;
-    if (active) {
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.x + (static_cast<size_t>(r) * d.T + t) * d.H) + lane * 2;
-        raw0 = ld16_nt(src);
-        raw1 = ld16_nt(src + 1);
-    }
-
     uint4 q = make_uint4(0, 0, 0, 0);
     if constexpr (FP8) {
         const uint32_t w[8] = {raw0.x, raw0.y, raw0.z, raw0.w, raw1.x, raw1.y, raw1.z, raw1.w};
@@ -227,6 +229,7 @@ struct ScalesArgs {
     int *stats;
     LlDims d;
     int use_ue8m0;
+    int parts; // workgroups per expert
 };
 
 // grid = E * kScaleParts workgroups.  Every workgroup of expert e scans the R per-rank
@@ -237,14 +240,15 @@ struct ScalesArgs {
 // gathers that token's scales (contiguous per token) and writes them at stride N, so that
 // for each scale group the threads of a wave write consecutive addresses (the column-major
 // layout of csrc/nixl_ep.cpp:1093-1100, kernels/nixl_ep_ll.cu:372-391).
-constexpr int kScaleParts = 4;
+constexpr int kScaleParts = 4; // workgroups per expert; 8 and 14 measured slower
 constexpr int kScaleBatch = 8;
 
 __global__ void __launch_bounds__(kLayoutThreads)
 ll_scales_kernel(ScalesArgs a) {
     extern __shared__ int seg_end[]; // [R] end of each source rank's segment of expert e
     const LlDims d = a.d;
-    const int e = blockIdx.x / kScaleParts, part = blockIdx.x % kScaleParts, tid = threadIdx.x;
+    const int parts = a.parts;
+    const int e = blockIdx.x / parts, part = blockIdx.x % parts, tid = threadIdx.x;
     const int G = d.H / 128;
     if (!a.recv_scales && part != 0) return; // metadata only: one workgroup per expert is enough
     // the first row's source token is fetched before its validity is known (always in bounds)
@@ -295,16 +299,16 @@ ll_scales_kernel(ScalesArgs a) {
         const float *__restrict__ src = a.token_scales + (static_cast<size_t>(lo) * d.T + t) * G;
         if (!a.use_ue8m0) {
             float *__restrict__ dst = static_cast<float *>(a.recv_scales) + static_cast<size_t>(e) * G * d.N + slot;
-            for (int g0 = part; g0 < G; g0 += kScaleParts * kScaleBatch) {
+            for (int g0 = part; g0 < G; g0 += parts * kScaleBatch) {
                 float v[kScaleBatch];
 #pragma unroll
                 for (int j = 0; j < kScaleBatch; ++j) {
-                    const int g = g0 + j * kScaleParts;
+                    const int g = g0 + j * parts;
                     v[j] = g < G ? src[g] : 0.f;
                 }
 #pragma unroll
                 for (int j = 0; j < kScaleBatch; ++j) {
-                    const int g = g0 + j * kScaleParts;
+                    const int g = g0 + j * parts;
                     if (g < G) dst[static_cast<size_t>(g) * d.N] = v[j];
                 }
             }
@@ -312,7 +316,7 @@ ll_scales_kernel(ScalesArgs a) {
             // one exponent byte per group, four groups per 32-bit word, words [H/512][N]
             uint32_t *__restrict__ dst =
                 static_cast<uint32_t *>(a.recv_scales) + static_cast<size_t>(e) * (G / 4) * d.N + slot;
-            for (int g4 = part; g4 < G / 4; g4 += kScaleParts) {
+            for (int g4 = part; g4 < G / 4; g4 += parts) {
                 uint32_t word = 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -565,7 +569,8 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
     sa.stats = cumulative_local_expert_recv_stats;
     sa.d = d;
     sa.use_ue8m0 = use_ue8m0;
-    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * kScaleParts), dim3(kLayoutThreads),
+    sa.parts = kScaleParts;
+    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * sa.parts), dim3(kLayoutThreads),
                        static_cast<size_t>(d.R) * sizeof(int), s, sa);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
