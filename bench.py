@@ -259,6 +259,15 @@ def main():
         "roofline": kv["roofline"],
         "kv": kv["kv"],
     }
+    if args.block_bytes != 16384:
+        # the "@16KB" point the metric's name mentions: same shape with 16 KiB sub-blocks
+        half = argparse.Namespace(**vars(args))
+        half.block_bytes, half.steps, half.warmup = 16384, max(args.steps // 2, 1), max(args.warmup // 2, 1)
+        kv16 = run_kv(half)
+        line["kv"]["at_16KiB_descriptors"] = {
+            "value_GBps": round(kv16["value"], 1), "avg_launch_ms": kv16["roofline"]["avg_launch_ms"],
+            "achieved_GBps": kv16["roofline"]["achieved"], "frac": kv16["roofline"]["frac"],
+            "descriptors_per_request": kv16["kv"]["descriptors_per_request"]}
     if not args.no_ep:
         try:
             from nixl_amd import ep_bench

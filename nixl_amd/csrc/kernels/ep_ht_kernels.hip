@@ -196,7 +196,11 @@ collect_rows(const uint8_t *in_rank,
 }
 
 // ---- dispatch (result of kernels/nixl_ep_ht.cu:1109-1243) -------------------------------------
-// grid = R*T; block = H/8 lanes rounded up to whole waves (16 bytes of a row per lane).
+// grid = R*T*parts; a row is H/8 lanes of 16 bytes and a workgroup covers blockDim.x of them.
+// Narrow workgroups (one wave) measured fastest for this write-dominated scatter.
+// Dynamic LDS: R * 12 bytes (rows, then destination ranks).
+constexpr int kHtDispatchLanes = 64;
+
 __global__ void __launch_bounds__(1024)
 ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
                    int32_t *__restrict__ recv_topk_idx,
@@ -209,34 +213,38 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
                    const int *__restrict__ prefix,
                    const int *__restrict__ send_head,
                    const long long *__restrict__ row_offset,
-                   HtDims d) {
-    __shared__ long long rows[kMaxHtRanks];
-    __shared__ int dsts[kMaxHtRanks];
+                   HtDims d,
+                   int parts) {
+    extern __shared__ long long rows[]; // [R] rows, then [R] int destination ranks
+    int *dsts = reinterpret_cast<int *>(rows + d.R);
     __shared__ int n_rows;
     const int tid = threadIdx.x;
-    const int r = blockIdx.x / d.T, t = blockIdx.x % d.T;
+    const int token = blockIdx.x / parts, part = blockIdx.x % parts;
+    const int r = token / d.T, t = token % d.T;
     const size_t tok = static_cast<size_t>(r) * d.T + t;
     const int El = d.E / d.R;
-    const bool active = tid < d.H / 8;
+    const int col = part * blockDim.x + tid;
+    const bool active = col < d.H / 8;
     uint4 v = make_uint4(0, 0, 0, 0);
-    if (active) v = ld16_nt(reinterpret_cast<const uint4 *>(x + tok * d.H) + tid);
+    if (active) v = ld16_nt(reinterpret_cast<const uint4 *>(x + tok * d.H) + col);
     int sel = -1;
     float w = 0.f;
-    if (tid < d.K && topk_idx) {
+    const bool meta = part == 0;
+    if (meta && tid < d.K && topk_idx) {
         sel = topk_idx[tok * d.K + tid];
         w = topk_weights ? topk_weights[tok * d.K + tid] : 0.f;
     }
     const int n = collect_rows(in_rank, prefix, send_head, row_offset, d, r, t, rows, dsts, &n_rows);
     for (int i = 0; i < n; ++i) {
         const long long row = rows[i];
-        if (active) st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(row) * d.H) + tid, v);
-        if (tid < d.K && recv_topk_idx) {
+        if (active) st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(row) * d.H) + col, v);
+        if (meta && tid < d.K && recv_topk_idx) {
             const int dst = dsts[i];
             const bool local = sel >= dst * El && sel < (dst + 1) * El;
             recv_topk_idx[row * d.K + tid] = local ? sel - dst * El : -1;
             if (recv_topk_weights) recv_topk_weights[row * d.K + tid] = local ? w : 0.f;
         }
-        if (tid == 0 && recv_src_meta) {
+        if (meta && tid == 0 && recv_src_meta) {
             recv_src_meta[row * 2] = r;
             recv_src_meta[row * 2 + 1] = t;
         }
@@ -476,10 +484,15 @@ nixl_amd_ep_ht_dispatch(void *recv_x,
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: null pointer argument");
     if (recv_topk_idx && !topk_idx) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: recv_topk_idx without topk_idx");
     const HtDims d{num_ranks, num_tokens, hidden, num_topk, num_experts};
-    hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens), dim3(round_up_wave(hidden / 8)),
-                       0, static_cast<hipStream_t>(stream), static_cast<uint16_t *>(recv_x), recv_topk_idx, recv_topk_weights,
-                       recv_src_meta, static_cast<const uint16_t *>(x), topk_idx, topk_weights, is_token_in_rank,
-                       recv_gbl_rank_prefix_sum, send_head, reinterpret_cast<const long long *>(recv_row_offset), d);
+    const int lanes = round_up_wave(hidden / 8);
+    const int parts = (lanes + kHtDispatchLanes - 1) / kHtDispatchLanes;
+    if (static_cast<long long>(num_ranks) * num_tokens * parts >= (1ll << 31))
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many tokens");
+    hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens * parts), dim3(kHtDispatchLanes),
+                       static_cast<size_t>(num_ranks) * 12, static_cast<hipStream_t>(stream), static_cast<uint16_t *>(recv_x),
+                       recv_topk_idx, recv_topk_weights, recv_src_meta, static_cast<const uint16_t *>(x), topk_idx, topk_weights,
+                       is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                       reinterpret_cast<const long long *>(recv_row_offset), d, parts);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }
