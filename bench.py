@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 # one rocprofv3 --pmc run each, scaled by a plain 1 GiB element-wise kernel in the same run;
 # profiles/copy_uniform_kernel_kv_llama3_32KiB.txt).  Keyed by (blocks, pool blocks, block
 # bytes); counters cannot be read from inside this process, so other shapes report null.
-MEASURED_TRAFFIC_BYTES = {(1024, 8192, 32768): 4563374659}
+MEASURED_TRAFFIC_BYTES = {(1024, 8192, 32768): 4311669989}
 
 
 def _kv_descs(base, layers, pool_blocks, blk, block_ids):
