@@ -147,6 +147,9 @@ nixl_amd_ep_get_dispatch_layout(const int32_t *topk_idx,
  *                            covers tokens [c * ceil(T/C), (c+1) * ceil(T/C))
  *   send_head                [R src][T][R dst] int32: position of the token inside the
  *                            (src -> dst) segment, -1 if it does not go there
+ *   recv_row_offset          [R + 1] int64 or NULL (no reference counterpart): exclusive prefix
+ *                            of the per-destination row totals, the form ht_dispatch and
+ *                            ht_combine take; its last entry is the row count of recv_x
  */
 int
 nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
@@ -155,6 +158,7 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
                                int *recv_expert_count,
                                int *gbl_channel_prefix_matrix,
                                int *send_head,
+                               int64_t *recv_row_offset,
                                int num_tokens,
                                int num_ranks,
                                int num_experts,

@@ -118,31 +118,52 @@ ht_scan_kernel(const uint8_t *__restrict__ in_rank,
             channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = total;
 }
 
-// ---- notify, part 2: receive-side prefix over source ranks and aligned per-expert counts
-// (kernels/nixl_ep_ht.cu:295-314) -------------------------------------------------------------
-__global__ void
+// ---- notify, part 2: receive-side prefix over source ranks, aligned per-expert counts
+// (kernels/nixl_ep_ht.cu:295-314) and where each destination's rows start in the
+// concatenated outputs.  One workgroup. ------------------------------------------------------
+__global__ void __launch_bounds__(kScanThreads)
 ht_prefix_kernel(const int *__restrict__ channel_prefix,
                  const int *__restrict__ per_expert,
                  int *__restrict__ recv_rank_prefix,
                  int *__restrict__ recv_expert_count,
+                 long long *__restrict__ row_offset,
                  int R,
                  int E,
                  int C,
                  int alignment) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < R) {
-        const int d = i;
-        int sum = 0;
-        for (int r = 0; r < R; ++r) {
-            sum += channel_prefix[(static_cast<size_t>(r) * R + d) * C + (C - 1)];
-            recv_rank_prefix[d * R + r] = sum;
-        }
-    }
-    if (i < E) {
+    __shared__ int wave_sums[kScanThreads / kWaveSize];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += kScanThreads) {
         int n = 0;
         for (int r = 0; r < R; ++r)
-            n += per_expert[static_cast<size_t>(r) * E + i];
-        recv_expert_count[i] = (n + alignment - 1) / alignment * alignment;
+            n += per_expert[static_cast<size_t>(r) * E + e];
+        recv_expert_count[e] = (n + alignment - 1) / alignment * alignment;
+    }
+    // R <= kScanThreads: thread d owns destination d
+    int total = 0;
+    if (tid < R) {
+        for (int r = 0; r < R; ++r) {
+            total += channel_prefix[(static_cast<size_t>(r) * R + tid) * C + (C - 1)];
+            recv_rank_prefix[tid * R + r] = total;
+        }
+    }
+    if (row_offset) {
+        // exclusive prefix of the per-destination totals in 64 bits
+        long long incl = total;
+        const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
+#pragma unroll
+        for (int off = 1; off < kWaveSize; off <<= 1) {
+            const long long up = __shfl_up(incl, off);
+            if (lane >= off) incl += up;
+        }
+        // wave totals fit in 32 bits each only if R * T does; check_ht bounds R * T by 2^30
+        if (lane == kWaveSize - 1) wave_sums[wave] = static_cast<int>(incl);
+        __syncthreads();
+        long long before = 0;
+        for (int w = 0; w < wave; ++w)
+            before += wave_sums[w];
+        if (tid < R) row_offset[tid + 1] = before + incl;
+        if (tid == 0) row_offset[0] = 0;
     }
 }
 
@@ -434,6 +455,7 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
                                int *recv_expert_count,
                                int *gbl_channel_prefix_matrix,
                                int *send_head,
+                               int64_t *recv_row_offset,
                                int num_tokens,
                                int num_ranks,
                                int num_experts,
@@ -451,10 +473,10 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
     hipLaunchKernelGGL(ht_scan_kernel, dim3(static_cast<unsigned>(num_ranks) * num_ranks), dim3(kScanThreads), 0, s, is_token_in_rank, send_head,
                        gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
     HIP_TRY(hipGetLastError());
-    const int n = num_experts > num_ranks ? num_experts : num_ranks;
-    hipLaunchKernelGGL(ht_prefix_kernel, dim3((n + 255) / 256), dim3(256), 0, s, gbl_channel_prefix_matrix,
-                       num_tokens_per_expert, recv_gbl_rank_prefix_sum, recv_expert_count, num_ranks, num_experts,
-                       num_channels, expert_alignment);
+    hipLaunchKernelGGL(ht_prefix_kernel, dim3(1), dim3(kScanThreads), 0, s, gbl_channel_prefix_matrix,
+                       num_tokens_per_expert, recv_gbl_rank_prefix_sum, recv_expert_count,
+                       reinterpret_cast<long long *>(recv_row_offset), num_ranks, num_experts, num_channels,
+                       expert_alignment);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }

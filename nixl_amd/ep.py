@@ -104,6 +104,13 @@ class Buffer:
     def _mask_ptr(self):
         return _ptr(self.mask_buffer) if self._mask_active else None
 
+    def _host_counts(self, n):
+        """Pinned host buffers for the counts normal-mode dispatch reads back."""
+        if getattr(self, "_pinned_counts", None) is None or self._pinned_counts[1].numel() != n:
+            self._pinned_counts = (torch.empty(1, dtype=torch.int64, pin_memory=True),
+                                   torch.empty(n, dtype=torch.int32, pin_memory=True))
+        return self._pinned_counts
+
     def _get_workspace(self, nbytes):
         if self._workspace is None or self._workspace.numel() < nbytes:
             self._workspace = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=self.device)
@@ -255,15 +262,20 @@ class Buffer:
         expert_count = torch.empty((R, El), dtype=torch.int32, device=dev)
         chan = torch.empty((R, R, num_channels), dtype=torch.int32, device=dev)
         send_head = torch.empty((R, T, R), dtype=torch.int32, device=dev)
+        row_offset = torch.empty(R + 1, dtype=torch.int64, device=dev)
         _check(self._k.nixl_amd_ep_ht_notify_dispatch(_ptr(is_token_in_rank), _ptr(num_tokens_per_expert), _ptr(prefix),
-                                                      _ptr(expert_count), _ptr(chan), _ptr(send_head), T, R, E,
-                                                      num_channels, expert_alignment, _stream()), "ht_notify_dispatch")
+                                                      _ptr(expert_count), _ptr(chan), _ptr(send_head), _ptr(row_offset),
+                                                      T, R, E, num_channels, expert_alignment, _stream()),
+               "ht_notify_dispatch")
         # The reference blocks here too, until the GPU has published the receive counts
-        # through host-mapped memory (csrc/nixl_ep.cpp:762-800), to size recv_x.
-        totals = prefix[:, -1].to(torch.int64)
-        row_offset = torch.zeros(R + 1, dtype=torch.int64, device=dev)
-        row_offset[1:] = torch.cumsum(totals, 0)
-        total = int(row_offset[-1].item())
+        # through host-mapped memory (csrc/nixl_ep.cpp:762-800), to size recv_x.  One
+        # synchronisation brings both the row total and the per-expert counts to the host.
+        host_total, host_counts = self._host_counts(R * El)
+        host_total.copy_(row_offset[-1:], non_blocking=True)
+        host_counts.copy_(expert_count.view(-1), non_blocking=True)
+        torch.cuda.current_stream(dev).synchronize()
+        total = int(host_total[0])
+        expert_count_list = host_counts.view(R, El).tolist()
         recv_x = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
         recv_topk_idx = torch.empty((total, K), dtype=torch.int32, device=dev)
         recv_topk_weights = torch.empty((total, K), dtype=torch.float32, device=dev)
@@ -273,7 +285,7 @@ class Buffer:
                                                _ptr(is_token_in_rank), _ptr(prefix), _ptr(send_head), _ptr(row_offset),
                                                T, H, K, R, E, _stream()), "ht_dispatch")
         out_handle = (is_token_in_rank, prefix, chan, recv_src_meta, send_head, row_offset)
-        return recv_x, recv_topk_idx, recv_topk_weights, expert_count.tolist(), out_handle, EventOverlap(None)
+        return recv_x, recv_topk_idx, recv_topk_weights, expert_count_list, out_handle, EventOverlap(None)
 
     def ht_combine(self, x, handle, topk_weights=None, bias=None, previous_event=None, async_finish=False,
                    allocate_on_comm_stream=False):
