@@ -598,3 +598,25 @@ def test_golden_normal_mode_world(cuda):
     comb, comb_w, _ = buf.ht_combine(recv_x, handle, topk_weights=recv_w, bias=(bf(g["bias0"]), bf(g["bias1"])))
     assert np.array_equal(bits16(comb).reshape(R, T, H), g["combined"])
     assert np.array_equal(comb_w.cpu().numpy(), g["combined_topk_weights"])
+
+
+@pytest.mark.parametrize("shape", [(64, 3, 512, 2, 128, 4), (2, 1, 8192, 16, 32, 1), (16, 64, 1024, 6, 48, 64), (1, 40, 512, 4, 8, 64)])
+def test_ll_wide_and_narrow_worlds(cuda, shape):
+    """Many ranks with few tokens, the largest hidden size and top-k, one rank alone:
+    dispatch (fp8 and bf16) and combine against the oracle."""
+    R, T, H, K, E, M = shape
+    x, topk, w = make_world(R * 7 + K, R, T, H, K, E, drop=0.05, scale=2.0)
+    for use_fp8 in (True, False):
+        rc, got = raw_ll_dispatch(cuda, x, topk, E, M, use_fp8)
+        assert rc == 0, _lib.kernels_error()
+        assert_dispatch_equal(got, eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, use_fp8, fill=0x55), use_fp8)
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, rx, torch.zeros_like(rx))
+    out, _, _ = buf.combine(y, td, wd, handle)
+    torch.cuda.synchronize()
+    want = eo.ll_combine(bits16(y).reshape(R, E // R, R * M, H), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(),
+                         E, M, use_fma=True)
+    assert np.array_equal(bits16(out).reshape(R, T, H), want)
