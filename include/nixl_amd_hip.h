@@ -88,10 +88,11 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream);
 int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan);
 
-/* Plan facts: total payload bytes, descriptors on the 128-bit path, descriptors on the
- * byte path, device bytes held by the plan's own arrays, and how the 128-bit stream was
- * cut: chunks lying inside one descriptor (uniform) versus chunks crossing descriptor
- * boundaries (mixed). */
+/* Plan facts: total payload bytes, descriptors on the 128-bit paths, descriptors on the
+ * byte path, device bytes held by the plan's own arrays, and how the 128-bit work was cut:
+ * chunks of the packed stream lying inside one descriptor (uniform) versus chunks crossing
+ * descriptor boundaries (mixed), and pieces (one wavefront each) of the descriptors that are
+ * short or do not start on a 128-byte line. */
 typedef struct nixl_amd_copy_plan_info {
     uint64_t payload_bytes;
     uint64_t vec_descs;
@@ -103,6 +104,7 @@ typedef struct nixl_amd_copy_plan_info {
     uint32_t generic_items;
     uint32_t units_per_lane;
     uint32_t uniform_workgroups;
+    uint32_t piece_items;
 } nixl_amd_copy_plan_info_t;
 
 int

@@ -45,7 +45,7 @@ class CopyPlanInfo(Structure):
                 ("plan_device_bytes", c_uint64), ("vec_chunks", c_uint32),
                 ("uniform_chunks", c_uint32), ("mixed_chunks", c_uint32),
                 ("generic_items", c_uint32), ("units_per_lane", c_uint32),
-                ("uniform_workgroups", c_uint32)]
+                ("uniform_workgroups", c_uint32), ("piece_items", c_uint32)]
 
 
 _kernels = None

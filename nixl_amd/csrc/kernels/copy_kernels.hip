@@ -2,8 +2,12 @@
 // them (declared in include/nixl_amd_hip.h).
 //
 // Data layout of a plan in HBM
-//   The 16-byte-aligned descriptors of a request are concatenated, in request order, into
-//   one virtual stream measured in 16-byte units.  The stream is cut into chunks of
+//   16-byte-aligned descriptors of 256 B to 8 KiB, and longer ones whose source or
+//   destination does not start on a 128-byte line, become pieces of at most 4 KiB: a
+//   24-byte record {src, dst, units} and one wavefront each (wavefront-per-descriptor for
+//   anything up to 4 KiB); pieces after the first start on a destination line.
+//   The other 16-byte-aligned descriptors (long and line-aligned, or tiny) are
+//   concatenated, in request order, into one virtual stream measured in 16-byte units.  The stream is cut into chunks of
 //   64*UPL units; one wavefront moves one chunk: lane l moves units k*64 + l of the chunk,
 //   k < UPL, so every load/store instruction of a wave touches 1 KiB of consecutive bytes
 //   unless a descriptor boundary falls inside it.  Chunks are classified on the host:
@@ -49,6 +53,14 @@ struct MixedArgs {
     const uint32_t *chunks; // [n_mixed] chunk indices
     uint64_t total_units;
     uint32_t n_mixed;
+};
+
+// A piece of a small descriptor: at most kPieceUnits 16-byte units, one wavefront's work.
+struct PieceRec {
+    uint64_t src;
+    uint64_t dst;
+    uint32_t units;
+    uint32_t pad;
 };
 
 struct GenericItem {
@@ -114,6 +126,34 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, i
 #pragma unroll
     for (int k = 0; k < UPL; ++k)
         store16<NT>(d + k * (kWaveSize * 16u), v[k]);
+}
+
+// One wavefront per piece: the descriptor's own {src, dst, units} record, up to
+// kPieceLoads 128-bit loads in flight per lane, then the stores.  No search and no LDS:
+// the shape for descriptors of a few hundred bytes to a few KiB.
+
+constexpr int kPieceLoads = 4;
+constexpr uint32_t kPieceUnits = kWaveSize * kPieceLoads; // 4 KiB
+
+template<bool NT, int LOADS>
+__global__ void __launch_bounds__(kWaveSize)
+copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) {
+    const uint32_t lane = threadIdx.x;
+    const uint32_t p = blockIdx.x;
+    const PieceRec rec = recs[p]; // same address in every lane: a scalar load
+    const uint64_t d = rec.dst + lane * 16u;
+    const uint32_t units = rec.units; // >= 1
+    // Loads are unconditional (a lane past the end re-reads the piece's last unit) so that
+    // all of them are in flight together; only the stores are predicated.
+    v4u v[LOADS];
+#pragma unroll
+    for (int k = 0; k < LOADS; ++k) {
+        const uint32_t u = min(k * kWaveSize + lane, units - 1);
+        v[k] = load16<NT>(rec.src + u * 16ull);
+    }
+#pragma unroll
+    for (int k = 0; k < LOADS; ++k)
+        if (k * kWaveSize + lane < units) store16<NT>(d + k * (kWaveSize * 16u), v[k]);
 }
 
 // One wavefront per chunk that crosses descriptor boundaries or is short.
@@ -293,6 +333,8 @@ struct nixl_amd_copy_plan {
     uint32_t uniform_wgs = 0;
     MixedArgs mixed_args{};
     uint32_t mixed_wgs = 0;
+    const PieceRec *piece_recs = nullptr;
+    uint32_t n_pieces = 0;
     const GenericItem *generic_items = nullptr;
     uint32_t n_generic = 0;
     uint32_t generic_wgs = 0;
@@ -339,10 +381,15 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     // ---- host-side lowering ------------------------------------------------------
     std::vector<uint64_t> vsrc, vdst, vprefix;
     std::vector<GenericItem> items;
+    std::vector<PieceRec> pieces;
+    // Descriptors of 256 B to 8 KiB, and longer ones whose source or destination does not
+    // start on a 128-byte line, go to the piece kernel: measured faster there (fewer lines
+    // split between wavefronts); line-aligned long descriptors stream best in 1 KiB chunks.
+    constexpr uint64_t kPieceMinUnits = 16, kPieceMaxDescUnits = 512;
     vsrc.reserve(n);
     vdst.reserve(n);
     vprefix.reserve(n + 1);
-    uint64_t units = 0, payload = 0, n_generic_descs = 0;
+    uint64_t units = 0, payload = 0, n_generic_descs = 0, n_piece_descs = 0;
     for (size_t i = 0; i < n; ++i) {
         const nixl_amd_copy_desc_t &d = descs[i];
         if (d.len == 0) continue;
@@ -351,7 +398,20 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         if (d.src + d.len < d.src || d.dst + d.len < d.dst)
             return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: address range wraps in descriptor " + std::to_string(i));
         payload += d.len;
-        if (((d.src | d.dst | d.len) & 15u) == 0) {
+        const bool aligned16 = ((d.src | d.dst | d.len) & 15u) == 0;
+        const uint64_t du = d.len / 16u;
+        if (aligned16 && du >= kPieceMinUnits && (du < kPieceMaxDescUnits || ((d.src | d.dst) & 127u) != 0)) {
+            // Pieces of at most kPieceUnits units, one wavefront each.  The first piece is
+            // cut so that every later one starts on a 128-byte line of the destination: no
+            // line is then written by two wavefronts.
+            const uint64_t head = kPieceUnits - ((d.dst >> 4) & 7u);
+            for (uint64_t first = 0; first < du;) {
+                const uint64_t n_units = std::min<uint64_t>(first == 0 ? head : kPieceUnits, du - first);
+                pieces.push_back(PieceRec{d.src + first * 16u, d.dst + first * 16u, static_cast<uint32_t>(n_units), 0u});
+                first += n_units;
+            }
+            ++n_piece_descs;
+        } else if (aligned16) {
             vsrc.push_back(d.src);
             vdst.push_back(d.dst);
             vprefix.push_back(units);
@@ -371,7 +431,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     const size_t nv = vsrc.size();
     const uint64_t chunk_units = static_cast<uint64_t>(kWaveSize) * upl;
     const uint64_t n_chunks64 = (units + chunk_units - 1) / chunk_units;
-    if (n_chunks64 >= (1ull << 32) || items.size() >= (1ull << 32))
+    if (n_chunks64 >= (1ull << 32) || items.size() >= (1ull << 32) || pieces.size() >= (1ull << 31))
         return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: request too large for 32-bit chunk index");
     const uint32_t n_chunks = static_cast<uint32_t>(n_chunks64);
 
@@ -435,7 +495,8 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     const size_t off_prefix = off_dst + (need_desc_arrays ? align256(nv * 8) : 0);
     const size_t off_span = off_prefix + (need_desc_arrays ? align256((nv + 1) * 8) : 0);
     const size_t off_mixed = off_span + (need_desc_arrays ? align256(size_t(n_chunks) * sizeof(uint2)) : 0);
-    const size_t off_items = off_mixed + align256(mixed.size() * sizeof(uint32_t));
+    const size_t off_pieces = off_mixed + align256(mixed.size() * sizeof(uint32_t));
+    const size_t off_items = off_pieces + align256(pieces.size() * sizeof(PieceRec));
     const size_t total = off_items + align256(items.size() * sizeof(GenericItem));
 
     auto *plan = new nixl_amd_copy_plan();
@@ -456,6 +517,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             std::memcpy(host.data() + off_span, span.data(), size_t(n_chunks) * sizeof(uint2));
             std::memcpy(host.data() + off_mixed, mixed.data(), mixed.size() * sizeof(uint32_t));
         }
+        if (!pieces.empty()) std::memcpy(host.data() + off_pieces, pieces.data(), pieces.size() * sizeof(PieceRec));
         if (!items.empty())
             std::memcpy(host.data() + off_items, items.data(), items.size() * sizeof(GenericItem));
         hipError_t e = hipMalloc(&plan->arena, total);
@@ -477,8 +539,10 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         plan->mixed_args.prefix = reinterpret_cast<const uint64_t *>(base + off_prefix);
         plan->mixed_args.span = reinterpret_cast<const uint2 *>(base + off_span);
         plan->mixed_args.chunks = reinterpret_cast<const uint32_t *>(base + off_mixed);
+        plan->piece_recs = reinterpret_cast<const PieceRec *>(base + off_pieces);
         plan->generic_items = reinterpret_cast<const GenericItem *>(base + off_items);
     }
+    plan->n_pieces = static_cast<uint32_t>(pieces.size());
     plan->n_uniform = n_uniform_chunks;
     plan->chunks_per_rec = chunks_per_rec;
     plan->mixed_args.total_units = units;
@@ -495,13 +559,14 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     plan->generic_wgs = wgs_for(plan->n_generic, kMixedWaves, true);
 
     plan->info.payload_bytes = payload;
-    plan->info.vec_descs = nv;
+    plan->info.vec_descs = nv + n_piece_descs;
     plan->info.generic_descs = n_generic_descs;
     plan->info.plan_device_bytes = plan->arena_bytes;
     plan->info.vec_chunks = n_chunks;
     plan->info.uniform_chunks = plan->n_uniform;
     plan->info.mixed_chunks = plan->mixed_args.n_mixed;
     plan->info.generic_items = plan->n_generic;
+    plan->info.piece_items = plan->n_pieces;
     plan->info.units_per_lane = static_cast<uint32_t>(upl);
     plan->info.uniform_workgroups = plan->uniform_wgs;
     *out = plan;
@@ -524,6 +589,16 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
         else
             launch_uniform_upl<false>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
                                       plan->uniform_wgs, plan->swizzle, plan->chunks_per_rec);
+        HIP_TRY(hipGetLastError());
+    }
+    if (plan->n_pieces) {
+        const dim3 grid(plan->n_pieces);
+        if (plan->nt)
+            hipLaunchKernelGGL((copy_piece_kernel<true, kPieceLoads>), grid, dim3(kWaveSize), 0, s, plan->piece_recs,
+                               plan->n_pieces);
+        else
+            hipLaunchKernelGGL((copy_piece_kernel<false, kPieceLoads>), grid, dim3(kWaveSize), 0, s, plan->piece_recs,
+                               plan->n_pieces);
         HIP_TRY(hipGetLastError());
     }
     if (plan->mixed_wgs) {

@@ -370,3 +370,25 @@ def test_golden_descriptor_list(cuda):
     assert _lib.kernels().nixl_amd_copy_plan_destroy(plan) == 0
     assert np.array_equal(dst.cpu().numpy(), g["dst"])
     assert np.array_equal(src.cpu().numpy(), g["src"])
+
+
+def test_piece_path_line_misaligned_and_split(cuda):
+    """Descriptors that are 16-byte but not 128-byte aligned, from 256 B to 40 KiB: the
+    piece kernel with its destination-line-aligned splits, every src/dst line offset."""
+    import torch
+    rng = np.random.default_rng(12)
+    src_off, dst_off, lens = [], [], []
+    pos_s, pos_d = 0, 8 << 20
+    for i, n in enumerate([256, 272, 1008, 1024, 4080, 4096, 4112, 8176, 8192, 8208, 12304, 40960, 40976] * 8):
+        sa, da = (i * 16) % 128, (i * 48 + 16) % 128
+        src_off.append(pos_s + sa)
+        dst_off.append(pos_d + da)
+        lens.append(n)
+        pos_s += ((n + 255) // 128 + 1) * 128
+        pos_d += ((n + 255) // 128 + 1) * 128
+    assert pos_s <= (8 << 20)
+    info = _check_against_oracle(torch, cuda, 16 << 20, src_off, dst_off, lens, seed=13)
+    assert info.piece_items > len(lens) and info.generic_descs == 0
+    # a long line-aligned descriptor still streams in uniform chunks, a short one is one piece
+    info = _check_against_oracle(torch, cuda, 1 << 20, [0, 65536], [131072, 262144], [32768, 2048], seed=14)
+    assert info.uniform_chunks == 32 and info.piece_items == 1
