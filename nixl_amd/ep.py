@@ -78,6 +78,82 @@ class Buffer:
         self._mask_active = False
         self._workspace = None
 
+    # -- life cycle and sizing helpers kept for callers written against the reference ------
+    def destroy(self):
+        """Reference: buffer.py:103-110.  Drops the device buffers this object owns."""
+        self.mask_buffer = None
+        self._workspace = None
+        self._combine_buffer = None
+
+    @staticmethod
+    def capture():
+        """Reference: buffer.py:129-136: an event on the current stream."""
+        event = torch.cuda.Event()
+        event.record()
+        return EventOverlap(event)
+
+    def get_comm_stream(self):
+        """Reference: buffer.py:174-186.  The kernels run on the caller's current stream."""
+        return torch.cuda.current_stream(self.device)
+
+    @staticmethod
+    def get_low_latency_buffer_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts):
+        """Bytes of RDMA staging per rank the reference would ask for (EPLayout,
+        csrc/config.hpp:145-208): two send buffers, two receive buffers and two signalling
+        buffers, rounded up past the next multiple of 128.  Nothing here allocates that
+        memory (rows go straight to their final place); the figure is for callers that
+        budget memory with the reference's own formula."""
+        num_scales = hidden // 128
+        if num_scales * 4 > hidden:
+            raise EPError("hidden too small for per-128-channel scales")
+        dispatch_msg = 16 + max(hidden * 2, hidden + num_scales * 4)
+        combine_msg = num_scales * 4 + hidden * 2
+        send = max(num_max_dispatch_tokens_per_rank * dispatch_msg,
+                   num_experts * num_max_dispatch_tokens_per_rank * combine_msg)
+        recv = max(num_experts * num_max_dispatch_tokens_per_rank * dispatch_msg,
+                   num_experts * num_max_dispatch_tokens_per_rank * combine_msg)
+        signalling = (num_experts * 8 + 127) // 128 * 128
+        total = send * 2 + recv * 2 + signalling * 2
+        return (total + 128) // 128 * 128
+
+    @staticmethod
+    def get_rdma_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts):
+        """Reference alias, buffer.py:163-172."""
+        return Buffer.get_low_latency_buffer_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts)
+
+    def get_next_combine_buffer(self, handle):
+        """Reference: buffer.py:743-764.  A bf16 tensor shaped like the packed_recv_x of the
+        dispatch that produced `handle`; experts may write their outputs into it and call
+        combine(..., zero_copy=True), which then reads it instead of its `x` argument."""
+        src_info, _layout_range, max_tok, hidden = handle
+        R, El, N = src_info.shape
+        shape = (R, El, N, hidden)
+        if getattr(self, "_combine_buffer", None) is None or tuple(self._combine_buffer.shape) != shape:
+            self._combine_buffer = torch.empty(shape, dtype=torch.bfloat16, device=self.device)
+        return self._combine_buffer
+
+    # Connection management of the reference (buffer.py:766-880) has nothing to do when all
+    # ranks live in one process; the calls exist so that code written for it runs unchanged.
+    def update_memory_buffers(self, num_ranks=None, num_experts_per_rank=None, num_rdma_bytes=0):
+        if num_ranks is not None and int(num_ranks) != self.num_ranks:
+            raise EPError("the number of ranks is fixed when the Buffer is created")
+
+    def connect_ranks(self, remote_ranks, activate=True):
+        for r in remote_ranks:
+            if not 0 <= int(r) < self.num_ranks:
+                raise EPError(f"rank {r} is outside this world of {self.num_ranks} ranks")
+        for r in remote_ranks:  # activate=False keeps the new ranks masked (buffer.py:848)
+            self.update_mask_buffer(int(r), not activate)
+
+    def disconnect_ranks(self, remote_ranks):
+        for r in remote_ranks:
+            if not 0 <= int(r) < self.num_ranks:
+                raise EPError(f"rank {r} is outside this world of {self.num_ranks} ranks")
+            self.update_mask_buffer(int(r), True)
+
+    def barrier(self):
+        torch.cuda.current_stream(self.device).synchronize()
+
     # -- rank masks (reference: buffer.py:716-775, csrc/nixl_ep.cpp:463-549) ---------------
     def update_mask_buffer(self, rank, mask=True):
         """Mark `rank` failed (or healthy again) in every rank's view, which is the state the
@@ -187,12 +263,14 @@ class Buffer:
         if not self.low_latency_mode:
             raise EPError("combine() requires low-latency mode (low_latency_mode=True)")
         src_info, layout_range, max_tok, hidden = handle
+        if zero_copy:
+            x = getattr(self, "_combine_buffer", None)
+            if x is None:
+                raise EPError("zero_copy=True needs get_next_combine_buffer() first")
         if x.dim() != 4 or not x.is_contiguous() or x.dtype != torch.bfloat16 or x.shape[-1] != hidden:
             raise EPError("x must be a contiguous [R, El, N, H] bfloat16 tensor")
         if topk_weights.dtype != torch.float32 or not topk_weights.is_contiguous():
             raise EPError("topk_weights must be contiguous float32")
-        if zero_copy:
-            raise EPError("zero_copy has no meaning without staging buffers")
         R, T, K = topk_idx.shape
         num_experts = x.shape[1] * R
         combined = out if out is not None else torch.empty((R, T, hidden), dtype=torch.bfloat16, device=x.device)

@@ -620,3 +620,40 @@ def test_ll_wide_and_narrow_worlds(cuda, shape):
     want = eo.ll_combine(bits16(y).reshape(R, E // R, R * M, H), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(),
                          E, M, use_fma=True)
     assert np.array_equal(bits16(out).reshape(R, T, H), want)
+
+
+def test_zero_copy_combine_and_connection_calls(cuda):
+    """get_next_combine_buffer + combine(zero_copy=True) equals combine on a caller tensor;
+    disconnect_ranks / connect_ranks drive the mask the way update_mask_buffer does."""
+    R, T, H, K, E, M = 4, 10, 512, 3, 8, 16
+    x, topk, w = make_world(77, R, T, H, K, E, drop=0.0)
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, rx, torch.zeros_like(rx))
+    want, _, _ = buf.combine(y, td, wd, handle)
+    with pytest.raises(EPError):
+        Buffer(R, device=cuda).combine(y, td, wd, handle, zero_copy=True)
+    staging = buf.get_next_combine_buffer(handle)
+    assert staging.shape == rx.shape and staging.dtype == torch.bfloat16
+    staging.copy_(y)
+    got, _, _ = buf.combine(torch.empty(0, device=cuda), td, wd, handle, zero_copy=True)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+    buf.disconnect_ranks([2])
+    status = torch.zeros(R, dtype=torch.int32, device=cuda)
+    buf.query_mask_buffer(status)
+    assert status.tolist() == [0, 0, 1, 0]
+    _, cnt_masked, _, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    assert int(cnt_masked[2].sum()) == 0
+    buf.connect_ranks([2], activate=False)
+    buf.query_mask_buffer(status)
+    assert status.tolist() == [0, 0, 1, 0]
+    buf.connect_ranks([2])
+    _, cnt_again, _, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    assert torch.equal(cnt_again, cnt)
+    with pytest.raises(EPError):
+        buf.connect_ranks([R])
+    buf.barrier()
+    buf.destroy()

@@ -412,3 +412,21 @@ def test_router_against_torch_topk_softmax():
     want = torch.softmax(tv, dim=1).numpy()
     assert np.allclose(w, want, rtol=2e-6, atol=0)
     assert np.allclose(w.sum(1), 1.0, atol=1e-6)
+
+
+def test_low_latency_buffer_size_hint_follows_the_reference_layout():
+    """EPLayout arithmetic (examples/device/ep/csrc/config.hpp:145-208) at the DeepSeek-V3
+    shape: messages of 14 352 B and 14 560 B, send = recv = 256 * 128 * 14 560 B, 2 KiB of
+    signalling, everything twice; the hint rounds up past the next multiple of 128."""
+    from nixl_amd.ep import Buffer
+    msg_d, msg_c = 16 + max(7168 * 2, 7168 + 56 * 4), 56 * 4 + 7168 * 2
+    assert (msg_d, msg_c) == (14352, 14560)
+    buf = 256 * 128 * msg_c
+    total = 2 * buf + 2 * buf + 2 * 2048
+    assert total == 1908412416
+    assert Buffer.get_low_latency_buffer_size_hint(128, 7168, 32, 256) == total + 128
+    assert Buffer.get_rdma_size_hint(128, 7168, 32, 256) == total + 128
+    # a shape where the dispatch message is the larger one on the send side
+    small = Buffer.get_low_latency_buffer_size_hint(64, 2048, 2, 1)
+    d, c = 16 + 2048 * 2, 16 * 4 + 2048 * 2
+    assert small == (2 * max(64 * d, 64 * c) + 2 * max(64 * d, 64 * c) + 2 * 128 + 128) // 128 * 128
