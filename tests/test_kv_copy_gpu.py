@@ -392,3 +392,17 @@ def test_piece_path_line_misaligned_and_split(cuda):
     # a long line-aligned descriptor still streams in uniform chunks, a short one is one piece
     info = _check_against_oracle(torch, cuda, 1 << 20, [0, 65536], [131072, 262144], [32768, 2048], seed=14)
     assert info.uniform_chunks == 32 and info.piece_items == 1
+
+
+def test_raw_south_bound_api_from_cpp(cuda):
+    """The plugin driven from C++ through nixlBackendEngine alone (no agent): plugin table,
+    registerMem / loadLocalMD, prepXfer / postXfer / checkXfer for WRITE and READ, handle
+    reuse, refusals, releaseReqH.  The program is tests/cpp/sb_api_roundtrip.cpp."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "sb_api_roundtrip")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe, os.path.join(_lib.PLUGIN_DIR, "libplugin_HIP.so")], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
