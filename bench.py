@@ -159,7 +159,7 @@ def run_calibration_copy():
     torch.cuda.empty_cache()
 
 
-def run_cpu_baseline(seconds=12.0):
+def run_cpu_baseline(seconds=12.0, threads=1):
     """Reference-shaped CPU path: one agent, loopback, DRAM->DRAM, one memcpy per descriptor
     (the semantics of the reference's UCX loopback puts, src/plugins/ucx/ucx_backend.cpp:
     1216-1262).  Same KV shape as the GPU workload with the pool cut to 512 blocks and 64
@@ -173,7 +173,7 @@ def run_cpu_baseline(seconds=12.0):
     dst_pool = np.zeros(lk * pool_blocks * blk, dtype=np.uint8)
     staging = np.zeros(n_sel * lk * blk, dtype=np.uint8)
     agent = nixl_agent("cpu", nixl_agent_config(backends=()), plugin_dirs=[plugin_dir])
-    agent.create_backend("MEMCPY", {"threads": "1"})
+    agent.create_backend("MEMCPY", {"threads": str(threads)})
     for a in (src_pool, dst_pool, staging):
         agent.register_memory(np.array([[a.ctypes.data, a.nbytes, 0]], dtype=np.uint64), "DRAM")
     sel = rng.choice(pool_blocks, n_sel, replace=False)
@@ -206,7 +206,7 @@ def run_cpu_baseline(seconds=12.0):
     for h in (gather, scatter, h_src, h_stg_r, h_stg_l, h_dst):
         h.release()
     agent.close()
-    return {"value": round(value, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+    return {"value": round(value, 3), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{steps} steps of gather+scatter, {n_desc} descriptors x {blk} B per request, "
                       f"DRAM->DRAM loopback, agent + per-descriptor memcpy backend, {wall:.1f} s",
             "host_cpus": os.cpu_count()}
@@ -276,6 +276,10 @@ def main():
             line["ep"] = None
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline()
+        # the same path with the descriptor list split over the box's CPU share, reported beside
+        many = min(16, os.cpu_count() or 1)
+        if many > 1:
+            line["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=5.0, threads=many)
     print(json.dumps(line))
 
 

@@ -140,9 +140,10 @@ def run_normal(dev, warmup=5, iters=20):
     }
 
 
-def run_cpu_baseline(seconds=10.0):
-    """Scalar CPU restatement of the low-latency kernels (the oracle), one thread, on a
-    bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8, fp8."""
+def run_cpu_baseline(seconds=10.0, threads=1):
+    """Scalar CPU restatement of the low-latency kernels (the oracle) on `threads` host
+    threads, on a bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8,
+    fp8."""
     from oracle import ep_oracle as eo
     R, T, H, K, E, M = 4, 128, 7168, 8, 32, 128
     rng = np.random.default_rng(4)
@@ -155,17 +156,17 @@ def run_cpu_baseline(seconds=10.0):
     d_us, c_us = [], []
     while time.perf_counter() - t0 < seconds or n < 2:
         a = time.perf_counter()
-        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True)
+        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True, threads=threads)
         b = time.perf_counter()
         y = np.zeros((R, E // R, R * M, H), np.uint16)
         c = time.perf_counter()
-        eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M)
+        eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M, threads=threads)
         d = time.perf_counter()
         d_us.append((b - a) * 1e6)
         c_us.append((d - c) * 1e6)
         n += 1
     return {"dispatch_us": round(float(np.mean(d_us)), 1), "combine_us": round(float(np.mean(c_us)), 1),
-            "cores": 1, "kind": "port", "host_cpus": os.cpu_count(),
+            "cores": threads, "kind": "port", "host_cpus": os.cpu_count(),
             "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
                       "(1/8 of the GPU workload's tokens)"}
 
@@ -177,4 +178,7 @@ def run(args):
            "normal": run_normal(dev, max(warmup // 4, 1), max(iters // 2, 1))}
     if not getattr(args, "no_cpu_baseline", False):
         out["cpu_baseline"] = run_cpu_baseline()
+        many = min(16, os.cpu_count() or 1)
+        if many > 1:
+            out["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=4.0, threads=many)
     return out
