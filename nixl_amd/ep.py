@@ -333,6 +333,19 @@ class Buffer:
             raise EPError("x must be a contiguous [R, T, H] bfloat16 tensor")
         R, T, H = x.shape
         dev = x.device
+        if handle is not None:
+            # Cached mode (buffer.py:560-597): the layout of an earlier dispatch is reused, so
+            # there is no count exchange and no host synchronisation; only rows travel.
+            in_rank, prefix, _chan, recv_src_meta, send_head, row_offset = handle
+            if tuple(in_rank.shape) != (R, T, R):
+                raise EPError("handle does not belong to a dispatch of this shape")
+            recv_x = torch.empty((recv_src_meta.shape[0], H), dtype=torch.bfloat16, device=dev)
+            _check(self._k.nixl_amd_ep_ht_dispatch(_ptr(recv_x), None, None, None, _ptr(x), None, None, _ptr(in_rank),
+                                                   _ptr(prefix), _ptr(send_head), _ptr(row_offset), T, H, 0, R, R,
+                                                   _stream()), "ht_dispatch")
+            return recv_x, None, None, None, None, EventOverlap(None)
+        if num_tokens_per_rank is None or is_token_in_rank is None or num_tokens_per_expert is None or topk_idx is None:
+            raise EPError("ht_dispatch needs either a handle or the tensors of get_dispatch_layout and topk_idx")
         K = topk_idx.shape[2]
         E = num_tokens_per_expert.shape[1]
         El = E // R

@@ -70,6 +70,12 @@ def run_low_latency(dev, warmup=20, iters=50):
     del deq, sc
     t_combine = _timed(lambda: buf.combine(y, topk, w, handle), flush, warmup, iters)
 
+    def both():  # one event pair around the two calls, as a layer would issue them
+        dispatch()
+        buf.combine(y, topk, w, handle)
+
+    t_both = _timed(both, flush, warmup, iters)
+
     tokens, pairs = R * T, int((topk >= 0).sum())
     meta = R * El * R * 8 + R * El * 4
     dispatch_bytes = tokens * H * 2 + tokens * K * 4 + pairs * (H + H // 128 * 4 + 4) + meta
@@ -81,6 +87,7 @@ def run_low_latency(dev, warmup=20, iters=50):
         "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
         "dispatch_plus_combine_us": round(both_us, 2),
         "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
+        "dispatch_then_combine_one_event_pair": {**t_both, **_rate(dispatch_bytes + combine_bytes, t_both["avg_us"])},
         "router": {**t_router, "bytes": tokens * E * 4},
     }
 
@@ -122,6 +129,7 @@ def run_normal(dev, warmup=5, iters=20):
     t_dispatch = _timed(dispatch, flush, warmup, iters)
     recv_x, recv_idx, recv_w, per_expert_list, handle, _ = state["out"]
     rows = recv_x.shape[0]
+    t_cached = _timed(lambda: buf.ht_dispatch(x, handle=handle), flush, warmup, iters)
     coef = (recv_w * (recv_idx >= 0)).sum(1, keepdim=True)
     y = (recv_x.float() * coef).to(torch.bfloat16)
     t_combine = _timed(lambda: buf.ht_combine(y, handle, topk_weights=recv_w), flush, warmup, iters)
@@ -136,6 +144,8 @@ def run_normal(dev, warmup=5, iters=20):
         "layout": t_layout,
         "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]),
                      "note": "includes the host read-back of the receive counts that sizes recv_x"},
+        "dispatch_cached_handle": {**t_cached, **_rate(tokens * H * 2 + rows * H * 2, t_cached["avg_us"]),
+                                   "note": "layout of an earlier dispatch reused: rows only, no count exchange"},
         "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
     }
 

@@ -421,6 +421,13 @@ def test_ht_pipeline_matches_oracle(cuda, shape):
     assert np.array_equal(recv_idx.cpu().numpy(), o["recv_topk_idx"])
     assert np.array_equal(recv_w.cpu().numpy(), o["recv_topk_weights"])
     assert np.array_equal(meta.cpu().numpy(), np.stack([o["recv_src_rank"], o["recv_src_token"]], 1))
+    # cached mode: the handle of the first dispatch moves another tensor without a count exchange
+    x2 = (xd.float() * 0.5 + 1).to(torch.bfloat16)
+    again, none_idx, none_w, none_list, none_handle, _ = buf.ht_dispatch(x2, handle=handle)
+    torch.cuda.synchronize()
+    assert none_idx is None and none_w is None and none_list is None and none_handle is None
+    o2 = eo.ht_dispatch(bits16(x2).reshape(R, T, H), topk, w, o_in_rank, o_prefix, E)
+    assert np.array_equal(bits16(again).reshape(-1, H), o2["recv_x"])
     b0 = torch.from_numpy(np.random.default_rng(1).standard_normal((R, T, H)).astype(np.float32)).to(torch.bfloat16)
     b1 = torch.from_numpy(np.random.default_rng(2).standard_normal((R, T, H)).astype(np.float32)).to(torch.bfloat16)
     for bias in (None, b0.to(cuda), (b0.to(cuda), b1.to(cuda))):
