@@ -217,19 +217,14 @@ collect_rows(const uint8_t *in_rank,
 }
 
 // ---- dispatch (result of kernels/nixl_ep_ht.cu:1109-1243) -------------------------------------
-// grid = R*T*parts; a row is H/8 lanes of 16 bytes and a workgroup covers blockDim.x of them.
-// Narrow workgroups (one wave) measured fastest for this write-dominated scatter.
+// Rows: grid = R*T*parts; a row is H/8 lanes of 16 bytes and a workgroup covers blockDim.x
+// of them.  Narrow workgroups (one wave) measured fastest for this write-dominated scatter.
 // Dynamic LDS: R * 12 bytes (rows, then destination ranks).
 constexpr int kHtDispatchLanes = 64;
 
 __global__ void __launch_bounds__(1024)
 ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
-                   int32_t *__restrict__ recv_topk_idx,
-                   float *__restrict__ recv_topk_weights,
-                   int32_t *__restrict__ recv_src_meta,
                    const uint16_t *__restrict__ x,
-                   const int32_t *__restrict__ topk_idx,
-                   const float *__restrict__ topk_weights,
                    const uint8_t *__restrict__ in_rank,
                    const int *__restrict__ prefix,
                    const int *__restrict__ send_head,
@@ -243,32 +238,53 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
     const int token = blockIdx.x / parts, part = blockIdx.x % parts;
     const int r = token / d.T, t = token % d.T;
     const size_t tok = static_cast<size_t>(r) * d.T + t;
-    const int El = d.E / d.R;
     const int col = part * blockDim.x + tid;
     const bool active = col < d.H / 8;
     uint4 v = make_uint4(0, 0, 0, 0);
     if (active) v = ld16_nt(reinterpret_cast<const uint4 *>(x + tok * d.H) + col);
-    int sel = -1;
-    float w = 0.f;
-    const bool meta = part == 0;
-    if (meta && tid < d.K && topk_idx) {
-        sel = topk_idx[tok * d.K + tid];
-        w = topk_weights ? topk_weights[tok * d.K + tid] : 0.f;
-    }
     const int n = collect_rows(in_rank, prefix, send_head, row_offset, d, r, t, rows, dsts, &n_rows);
-    for (int i = 0; i < n; ++i) {
-        const long long row = rows[i];
-        if (active) st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(row) * d.H) + col, v);
-        if (meta && tid < d.K && recv_topk_idx) {
-            const int dst = dsts[i];
+    if (!active) return;
+    for (int i = 0; i < n; ++i)
+        st16_nt(reinterpret_cast<uint4 *>(recv_x + static_cast<size_t>(rows[i]) * d.H) + col, v);
+}
+
+// Per-row metadata: rebased top-k indices, weights of the local selections, source rank and
+// token.  grid = R * R * ceil(T / 256): (source, destination) pairs major, one token per
+// thread.  Consecutive tokens that go to the destination occupy consecutive rows,
+// so a wave writes a contiguous stretch of each array; written from the row kernel above,
+// the same bytes were isolated 32-byte stores and cost five times as long.
+constexpr int kHtMetaThreads = 256;
+
+__global__ void __launch_bounds__(kHtMetaThreads)
+ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
+               float *__restrict__ recv_topk_weights,
+               int32_t *__restrict__ recv_src_meta,
+               const int32_t *__restrict__ topk_idx,
+               const float *__restrict__ topk_weights,
+               const uint8_t *__restrict__ in_rank,
+               const int *__restrict__ prefix,
+               const int *__restrict__ send_head,
+               const long long *__restrict__ row_offset,
+               HtDims d) {
+    const int blocks_per_pair = (d.T + kHtMetaThreads - 1) / kHtMetaThreads;
+    const int pair = blockIdx.x / blocks_per_pair;
+    const int r = pair / d.R, dst = pair % d.R;
+    const int t = (blockIdx.x % blocks_per_pair) * kHtMetaThreads + threadIdx.x;
+    if (t >= d.T) return;
+    const size_t tok = static_cast<size_t>(r) * d.T + t;
+    if (!in_rank[tok * d.R + dst]) return;
+    const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+    const int El = d.E / d.R;
+    if (recv_topk_idx)
+        for (int k = 0; k < d.K; ++k) {
+            const int sel = topk_idx[tok * d.K + k];
             const bool local = sel >= dst * El && sel < (dst + 1) * El;
-            recv_topk_idx[row * d.K + tid] = local ? sel - dst * El : -1;
-            if (recv_topk_weights) recv_topk_weights[row * d.K + tid] = local ? w : 0.f;
+            recv_topk_idx[row * d.K + k] = local ? sel - dst * El : -1;
+            if (recv_topk_weights) recv_topk_weights[row * d.K + k] = local && topk_weights ? topk_weights[tok * d.K + k] : 0.f;
         }
-        if (meta && tid == 0 && recv_src_meta) {
-            recv_src_meta[row * 2] = r;
-            recv_src_meta[row * 2 + 1] = t;
-        }
+    if (recv_src_meta) {
+        recv_src_meta[row * 2] = r;
+        recv_src_meta[row * 2 + 1] = t;
     }
 }
 
@@ -510,11 +526,20 @@ nixl_amd_ep_ht_dispatch(void *recv_x,
     const int parts = (lanes + kHtDispatchLanes - 1) / kHtDispatchLanes;
     if (static_cast<long long>(num_ranks) * num_tokens * parts >= (1ll << 31))
         return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many tokens");
+    hipStream_t s = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens * parts), dim3(kHtDispatchLanes),
-                       static_cast<size_t>(num_ranks) * 12, static_cast<hipStream_t>(stream), static_cast<uint16_t *>(recv_x),
-                       recv_topk_idx, recv_topk_weights, recv_src_meta, static_cast<const uint16_t *>(x), topk_idx, topk_weights,
-                       is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                       static_cast<size_t>(num_ranks) * 12, s, static_cast<uint16_t *>(recv_x),
+                       static_cast<const uint16_t *>(x), is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
                        reinterpret_cast<const long long *>(recv_row_offset), d, parts);
+    HIP_TRY(hipGetLastError());
+    if (recv_topk_idx || recv_src_meta) {
+        const long long blocks = static_cast<long long>(num_ranks) * num_ranks * ((num_tokens + kHtMetaThreads - 1) / kHtMetaThreads);
+        if (blocks >= (1ll << 31)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many ranks and tokens");
+        const dim3 grid(static_cast<unsigned>(blocks));
+        hipLaunchKernelGGL(ht_meta_kernel, grid, dim3(kHtMetaThreads), 0, s, recv_topk_idx, recv_topk_weights, recv_src_meta,
+                           topk_idx, topk_weights, is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                           reinterpret_cast<const long long *>(recv_row_offset), d);
+    }
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }
