@@ -406,3 +406,49 @@ def test_raw_south_bound_api_from_cpp(cuda):
         pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
     proc = subprocess.run([exe, os.path.join(_lib.PLUGIN_DIR, "libplugin_HIP.so")], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
+def test_requests_from_several_threads(cuda):
+    """The reference calls prepXfer / postXfer / checkXfer / releaseReqH concurrently from
+    several threads, one request each (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:
+    1847-1879).  Four threads, each creating, posting, polling and releasing its own requests
+    on a backend with four streams; every thread's bytes must arrive."""
+    import threading
+    import torch
+    a = nixl_agent("mt", nixl_agent_config(backends=()))
+    a.create_backend("HIP", {"num_streams": "4"})
+    n_threads, n_desc, blk, rounds = 4, 256, 8192, 20
+    rng = np.random.default_rng(21)
+    src = torch.from_numpy(rng.integers(0, 256, n_threads * n_desc * blk, dtype=np.uint8)).to(cuda)
+    dst = torch.zeros_like(src)
+    a.register_memory([src, dst])
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(tid):
+        try:
+            base = tid * n_desc * blk
+            perm = np.random.default_rng(tid).permutation(n_desc)
+            s_off = base + np.arange(n_desc) * blk
+            d_off = base + perm * blk
+            lens = np.full(n_desc, blk)
+            for _ in range(rounds):
+                req = a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(src, s_off, lens), "VRAM"),
+                                        a.get_xfer_descs(_descs(dst, d_off, lens), "VRAM"), "mt")
+                _wait(a, req)
+                req.release()
+        except Exception as e:  # noqa: BLE001 - reported to the main thread
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(n_threads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    got, want = dst.cpu().numpy().reshape(n_threads, n_desc, blk), src.cpu().numpy().reshape(n_threads, n_desc, blk)
+    for tid in range(n_threads):
+        perm = np.random.default_rng(tid).permutation(n_desc)
+        assert np.array_equal(got[tid][perm], want[tid])
+    a.close()
