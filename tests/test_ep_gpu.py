@@ -664,3 +664,49 @@ def test_zero_copy_combine_and_connection_calls(cuda):
         buf.connect_ranks([R])
     buf.barrier()
     buf.destroy()
+
+
+def test_ll_calls_can_be_captured_in_a_graph(cuda):
+    """Dispatch and combine allocate nothing and clear nothing with memset nodes (the caller
+    brings outputs and workspace), so both can be recorded into one HIP graph.  Every replay,
+    with eager work and synchronisation in between and outputs wiped, must equal the eager
+    result."""
+    R, T, H, K, E, M = 4, 32, 1024, 4, 16, 32
+    El, N = E // R, R * M
+    x, topk, w = make_world(91, R, T, H, K, E, drop=0.05)
+    k = _lib.ep_kernels()
+    xd, td, wd = x.to(cuda), torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    recv_x = torch.zeros((R, El, N, H), dtype=torch.uint8, device=cuda)
+    scales = torch.zeros((R, El, H // 128, N), dtype=torch.float32, device=cuda)
+    src_info = torch.zeros((R, El, N), dtype=torch.int32, device=cuda)
+    layout = torch.zeros((R, El, R), dtype=torch.int64, device=cuda)
+    count = torch.zeros((R, El), dtype=torch.int32, device=cuda)
+    row_map = torch.zeros((R, T, K), dtype=torch.int32, device=cuda)
+    ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K, H), dtype=torch.uint8, device=cuda)
+    y = torch.from_numpy(np.random.default_rng(5).standard_normal((R, El, N, H)).astype(np.float32)).to(torch.bfloat16).to(cuda)
+    out = torch.zeros((R, T, H), dtype=torch.bfloat16, device=cuda)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def both(stream):
+        s = ctypes.c_void_p(stream)
+        assert k.nixl_amd_ep_ll_dispatch(p(recv_x), p(scales), p(src_info), p(layout), p(count), None, None, p(xd), p(td), None,
+                                         T, H, M, K, R, E, 1, 0, 0, p(row_map), p(ws), ws.numel(), s) == 0, _lib.kernels_error()
+        assert k.nixl_amd_ep_ll_combine(p(out), p(y), p(td), p(wd), p(src_info), p(layout), None, None, p(row_map), T, H, M, K, R,
+                                        E, 0, s) == 0, _lib.kernels_error()
+
+    both(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (recv_x, scales, src_info, layout, count, row_map, out)]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        both(torch.cuda.current_stream().cuda_stream)
+    for i in range(3):
+        for t in (layout, count, row_map, out):
+            t.zero_()
+        (xd.float().sum() + i).item()  # eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        valid = torch.arange(N, device=cuda).view(1, 1, -1) < count.unsqueeze(-1)
+        assert torch.equal(layout, want[3]) and torch.equal(count, want[4]) and torch.equal(row_map, want[5])
+        assert torch.equal(out.view(torch.int16), want[6].view(torch.int16))
+        assert torch.equal(recv_x[valid], want[0][valid]) and torch.equal(src_info[valid], want[2][valid])
