@@ -98,7 +98,10 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
  *   combined_x    [R][T][H] bf16
  *   row_map       [R][T][K] int32 as written by the dispatch call that produced this
  *                 handle, or NULL to locate rows through src_info / layout_range
- * The LogFMT payload codec of the reference is not implemented: use_logfmt must be 0.
+ * use_logfmt: every row goes through the reference's LogFMT-10 codec (encode as the sender
+ * does, decode as the receiver does; kernels/nixl_ep_ll.cu:459-616) before it is accumulated.
+ * The codec is lossy and built on log2 / exp2, whose last bits differ between GPUs and libm:
+ * results are reproducible on one GPU and agree with the CPU restatement to a tolerance.
  */
 int
 nixl_amd_ep_ll_combine(void *combined_x,

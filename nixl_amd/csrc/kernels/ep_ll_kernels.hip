@@ -343,8 +343,43 @@ struct CombineArgs {
     int parts; // workgroups per token; each covers blockDim.x of the token's H/8 lanes
 };
 
+// LogFMT-10 as the reference's combine sender encodes a row and its receiver decodes it
+// (kernels/nixl_ep_ll.cu:459-616), applied in registers: v holds a lane's 8 magnitudes of one
+// row, 16 neighbouring lanes hold one 128-channel group.  A group is cast when
+// log2(amax) < 0 and the floored log2(amin) is below it; a magnitude then becomes
+// floor(max(log2(x) * step_inv + rounding - log_amin * step_inv, 0)) and comes back as
+// exp2((code - 1) * step + log_amin), or 0 for code 0.  Signs are kept by the caller.
+__device__ __forceinline__ void
+logfmt_roundtrip(float (&v)[8]) {
+    float amax = 0.f, amin = INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        amax = fmaxf(amax, v[j]);
+        amin = fminf(amin, v[j]);
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off));
+        amin = fminf(amin, __shfl_xor(amin, off));
+    }
+    const float log_amax = log2f(amax);
+    const float log_amin = fmaxf(log2f(amin), log_amax - 32.0f);
+    if (!(log_amax < 0.0f && log_amin < log_amax)) return; // uniform over the 16 lanes
+    const float step = (log_amax - log_amin) / 510.0f;
+    const float step_inv = 1.0f / step;
+    const float rounding = 2.0f - log2f((1.0f + exp2f(step)) * 0.5f) * step_inv;
+    const float fused_rounding = rounding - log_amin * step_inv;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float pos = fmaxf(fmaf(log2f(v[j]), step_inv, fused_rounding), 0.0f);
+        const uint32_t code = static_cast<uint32_t>(floorf(pos));
+        v[j] = code == 0 ? 0.0f : exp2f(fmaf(static_cast<float>(code - 1), step, log_amin));
+    }
+}
+
 // grid = R*T*parts workgroups; a token's row is H/8 lanes of 8 consecutive channels (16
 // bytes); a workgroup covers blockDim.x of them (a multiple of 64).
+template<bool LOGFMT>
 __global__ void __launch_bounds__(1024)
 ll_combine_kernel(CombineArgs a) {
     const LlDims d = a.d;
@@ -408,10 +443,25 @@ ll_combine_kernel(CombineArgs a) {
             if (k0 + j >= d.K || row_of_k[k0 + j] < 0) continue;
             const float w = weight_of_k[k0 + j];
             const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            if constexpr (LOGFMT) {
+                float mag[8];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                acc[2 * c] = fmaf(bf16_lo_to_f32(u[c]), w, acc[2 * c]);
-                acc[2 * c + 1] = fmaf(bf16_hi_to_f32(u[c]), w, acc[2 * c + 1]);
+                for (int c = 0; c < 4; ++c) {
+                    mag[2 * c] = bf16_lo_to_f32(u[c] & 0x7fff7fffu);
+                    mag[2 * c + 1] = bf16_hi_to_f32(u[c] & 0x7fff7fffu);
+                }
+                logfmt_roundtrip(mag);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    acc[2 * c] = fmaf((u[c] & 0x8000u) ? -mag[2 * c] : mag[2 * c], w, acc[2 * c]);
+                    acc[2 * c + 1] = fmaf((u[c] & 0x80000000u) ? -mag[2 * c + 1] : mag[2 * c + 1], w, acc[2 * c + 1]);
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    acc[2 * c] = fmaf(bf16_lo_to_f32(u[c]), w, acc[2 * c]);
+                    acc[2 * c + 1] = fmaf(bf16_hi_to_f32(u[c]), w, acc[2 * c + 1]);
+                }
             }
         }
     }
@@ -598,7 +648,6 @@ nixl_amd_ep_ll_combine(void *combined_x,
     const int rc = check_dims("ll_combine", num_tokens, hidden, num_max_dispatch_tokens_per_rank, num_topk, num_ranks,
                               num_experts, d);
     if (rc) return rc;
-    if (use_logfmt) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_combine: the LogFMT payload codec is not implemented");
     if (!combined_x || !x || !topk_idx || !topk_weights || !src_info || !layout_range)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_combine: null pointer argument");
     if (d.T == 0) return NIXL_AMD_OK;
@@ -615,8 +664,11 @@ nixl_amd_ep_ll_combine(void *combined_x,
     a.d = d;
     const int wg = std::min(round_up_wave(d.H / 8), g_combine_lanes);
     a.parts = (d.H / 8 + wg - 1) / wg;
-    hipLaunchKernelGGL(ll_combine_kernel, dim3(static_cast<unsigned>(d.R) * d.T * a.parts), dim3(wg), 0,
-                       static_cast<hipStream_t>(stream), a);
+    const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
+    if (use_logfmt)
+        hipLaunchKernelGGL(ll_combine_kernel<true>, grid, dim3(wg), 0, static_cast<hipStream_t>(stream), a);
+    else
+        hipLaunchKernelGGL(ll_combine_kernel<false>, grid, dim3(wg), 0, static_cast<hipStream_t>(stream), a);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }

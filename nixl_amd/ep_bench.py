@@ -70,6 +70,8 @@ def run_low_latency(dev, warmup=20, iters=50):
     del deq, sc
     t_combine = _timed(lambda: buf.combine(y, topk, w, handle), flush, warmup, iters)
 
+    t_logfmt = _timed(lambda: buf.combine(y, topk, w, handle, use_logfmt=True), flush, warmup, iters)
+
     def both():  # one event pair around the two calls, as a layer would issue them
         dispatch()
         buf.combine(y, topk, w, handle)
@@ -88,6 +90,7 @@ def run_low_latency(dev, warmup=20, iters=50):
         "dispatch_plus_combine_us": round(both_us, 2),
         "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
         "dispatch_then_combine_one_event_pair": {**t_both, **_rate(dispatch_bytes + combine_bytes, t_both["avg_us"])},
+        "combine_logfmt": {**t_logfmt, "note": "rows passed through the LogFMT-10 codec before accumulation"},
         "router": {**t_router, "bytes": tokens * E * 4},
     }
 

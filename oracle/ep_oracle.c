@@ -249,6 +249,50 @@ oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t *nu
 }
 
 /*
+ * LogFMT-10 as the combine sender applies it to one row and the receiver undoes it
+ * (kernels/nixl_ep_ll.cu:459-528 encode, :530-562 amax/amin check, :564-616 decode): per 128
+ * channels, with amax / amin the largest / smallest magnitude, the group is cast when
+ * log2(amax) < 0 and log2(amin) (floored at log2(amax) - 32) < log2(amax); a magnitude x
+ * becomes code = floor(max(log2(x) * step_inv + rounding - log_amin * step_inv, 0)) with
+ * step = (log_amax - log_amin) / 510, and comes back as 0 for code 0, else
+ * exp2((code - 1) * step + log_amin), with the sign restored.  Groups that are not cast pass
+ * unchanged.  The reference evaluates log2 / exp2 with approximate hardware instructions
+ * (lg2.approx, ex2.approx); libm stands in here, so results agree with any GPU only to the
+ * accuracy of those instructions: PARITY UNPINNED at bit level, checked by tolerance.
+ */
+void
+oracle_logfmt_roundtrip(const uint16_t *row, int hidden, float *out) {
+    for (int g0 = 0; g0 < hidden; g0 += 128) {
+        float amax = 0.0f, amin = INFINITY;
+        for (int j = 0; j < 128; ++j) {
+            const float a = fabsf(oracle_bf16_to_f32(row[g0 + j]));
+            amax = fmaxf(amax, a);
+            amin = fminf(amin, a);
+        }
+        const float log_amax = log2f(amax);
+        const float log_amin = fmaxf(log2f(amin), log_amax - 32.0f);
+        const int cast = log_amax < 0.0f && log_amin < log_amax;
+        if (!cast) {
+            for (int j = 0; j < 128; ++j)
+                out[g0 + j] = oracle_bf16_to_f32(row[g0 + j]);
+            continue;
+        }
+        const float step = (log_amax - log_amin) / 510.0f;
+        const float step_inv = 1.0f / step;
+        const float rounding = 2.0f - log2f((1.0f + exp2f(step)) * 0.5f) * step_inv;
+        const float fused_rounding = rounding - log_amin * step_inv;
+        for (int j = 0; j < 128; ++j) {
+            const uint16_t bits = row[g0 + j];
+            const float a = oracle_bf16_to_f32((uint16_t)(bits & 0x7fffu));
+            const float pos = fmaxf(fmaf(log2f(a), step_inv, fused_rounding), 0.0f);
+            const uint32_t code = (uint32_t)floorf(pos);
+            const float dec = code == 0 ? 0.0f : exp2f(fmaf((float)(code - 1), step, log_amin));
+            out[g0 + j] = (bits & 0x8000u) ? -dec : dec;
+        }
+    }
+}
+
+/*
  * kernels/nixl_ep_ll.cu:618-1017.  Send (:683-837): expert rank d copies row `i` of local
  * expert le, for i in the segment of source rank r, into r's slot (global expert * M +
  * src_info[i]).  Receive (:875-1016): token t accumulates, in top-k order,
@@ -259,9 +303,11 @@ oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t *nu
 int
 oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const float *topk_weights,
                   const int32_t *src_info, const int64_t *layout_range, const int32_t *num_tokens,
-                  const int32_t *mask, int R, int T, int H, int K, int E, int M, int use_fma,
+                  const int32_t *mask, int R, int T, int H, int K, int E, int M, int flags,
                   uint16_t *combined, int threads) {
     if (R <= 0 || E % R != 0) return -1;
+    const int use_fma = flags & 1, use_logfmt = (flags >> 1) & 1; /* the cast always accumulates fused */
+    if (use_logfmt && H % 128 != 0) return -1;
     const int El = E / R, N = R * M;
     /* slot area of every rank: [R][E][M] -> row index into expert_out, or -1 */
     int64_t *slot_row = (int64_t *)malloc((size_t)R * E * M * sizeof(int64_t));
@@ -283,6 +329,7 @@ oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const flo
     for (int r = 0; r < R; ++r) {
         const int nt = num_tokens ? num_tokens[r] : T;
         float *acc = (float *)malloc((size_t)H * sizeof(float));
+        float *dec = (float *)malloc((size_t)H * sizeof(float));
         for (int t = 0; t < nt; ++t) {
             for (int h = 0; h < H; ++h)
                 acc[h] = 0.0f;
@@ -293,7 +340,11 @@ oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const flo
                 if (row < 0) continue; /* never sent: the receiver times out and masks the rank */
                 const float w = topk_weights[((size_t)r * T + t) * K + k];
                 const uint16_t *src = expert_out + (size_t)row * H;
-                if (use_fma)
+                if (use_logfmt) {
+                    oracle_logfmt_roundtrip(src, H, dec);
+                    for (int h = 0; h < H; ++h)
+                        acc[h] = fmaf(dec[h], w, acc[h]);
+                } else if (use_fma)
                     for (int h = 0; h < H; ++h)
                         acc[h] = fmaf(oracle_bf16_to_f32(src[h]), w, acc[h]);
                 else
@@ -305,6 +356,7 @@ oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const flo
                 out[h] = oracle_f32_to_bf16(acc[h]);
         }
         free(acc);
+        free(dec);
     }
     free(slot_row);
     return 0;

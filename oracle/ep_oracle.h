@@ -46,8 +46,10 @@ int oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t
                        int32_t *recv_count, int threads);
 int oracle_ll_combine(const uint16_t *expert_out, const int32_t *topk_idx, const float *topk_weights,
                       const int32_t *src_info, const int64_t *layout_range, const int32_t *num_tokens,
-                      const int32_t *mask, int R, int T, int H, int K, int E, int M, int use_fma,
-                      uint16_t *combined, int threads);
+                      const int32_t *mask, int R, int T, int H, int K, int E, int M, int flags,
+                      uint16_t *combined, int threads); /* flags: 1 = fused multiply-add, 2 = LogFMT-10 rows */
+/* LogFMT-10 encode + decode of one row (hidden % 128 == 0) into fp32 values */
+void oracle_logfmt_roundtrip(const uint16_t *row, int hidden, float *out);
 
 void oracle_weighted_sum_rows(const uint16_t *rows, const float *w, int K, int H, int use_fma, uint16_t *out);
 

@@ -42,6 +42,7 @@ def lib():
         L.oracle_ht_dispatch.argtypes = [_P] * 5 + [_I] * 5 + [_P] * 7
         L.oracle_ht_combine.argtypes = [_P] * 8 + [_I] * 4 + [_P, _P]
         L.oracle_router.argtypes = [_P, _I, _I, _I, _P, _P]
+        L.oracle_logfmt_roundtrip.argtypes = [_P, _I, _P]
         _LIB = L
     return _LIB
 
@@ -123,8 +124,16 @@ def ll_dispatch(x, topk_idx, num_experts, max_tok, use_fp8=True, round_scale=Fal
     return dict(recv_x=recv_x, scales=scales, src_info=src_info, layout_range=layout_range, recv_count=recv_count)
 
 
+def logfmt_roundtrip(row):
+    """row [H] bf16 bits -> fp32 [H]: what a LogFMT-10 encoded row decodes to."""
+    row = _c(row, np.uint16)
+    out = np.zeros(row.shape[-1], np.float32)
+    lib().oracle_logfmt_roundtrip(_p(row), row.shape[-1], _p(out))
+    return out
+
+
 def ll_combine(expert_out, topk_idx, topk_weights, src_info, layout_range, num_experts, max_tok,
-               num_tokens=None, mask=None, use_fma=True, threads=1):
+               num_tokens=None, mask=None, use_fma=True, threads=1, use_logfmt=False):
     expert_out = _c(expert_out, np.uint16)
     topk_idx = _c(topk_idx, np.int32)
     topk_weights = _c(topk_weights, np.float32)
@@ -135,7 +144,7 @@ def ll_combine(expert_out, topk_idx, topk_weights, src_info, layout_range, num_e
     out = np.zeros((R, T, H), np.uint16)
     nt, mk = _c(num_tokens, np.int32), _c(mask, np.int32)
     rc = lib().oracle_ll_combine(_p(expert_out), _p(topk_idx), _p(topk_weights), _p(src_info), _p(layout_range),
-                                 _p(nt), _p(mk), R, T, H, K, num_experts, max_tok, int(use_fma), _p(out), threads)
+                                 _p(nt), _p(mk), R, T, H, K, num_experts, max_tok, int(use_fma) | (int(use_logfmt) << 1), _p(out), threads)
     if rc != 0:
         raise ValueError(f"oracle_ll_combine rejected the arguments ({rc})")
     return out

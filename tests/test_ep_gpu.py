@@ -710,3 +710,43 @@ def test_ll_calls_can_be_captured_in_a_graph(cuda):
         assert torch.equal(layout, want[3]) and torch.equal(count, want[4]) and torch.equal(row_map, want[5])
         assert torch.equal(out.view(torch.int16), want[6].view(torch.int16))
         assert torch.equal(recv_x[valid], want[0][valid]) and torch.equal(src_info[valid], want[2][valid])
+
+
+def test_ll_combine_logfmt(cuda):
+    """LogFMT-10 rows: against the CPU restatement (same formulas, libm instead of the GPU's
+    log2 / exp2, so a magnitude may land on the neighbouring code: at most one step of
+    2^(32/510) per term), and the reference test's own criterion for identity experts
+    (calc_diff < 1e-5, examples/device/ep/tests/elastic/elastic.py:377-387) on its own kind of
+    input (small random values, which are cast, mixed with values >= 1, which are not)."""
+    R, T, H, K, E, M = 4, 24, 1024, 4, 16, 32
+    El = E // R
+    rng = np.random.default_rng(61)
+    xs = rng.standard_normal((R, T, H)).astype(np.float32) * 0.5 * rng.random((R, T, 1)).astype(np.float32)
+    xs[:, ::5, :256] *= 8.0  # some groups at or above 1: left as bf16
+    xs[:, 1::7, 300:340] = 0.0
+    x = torch.from_numpy(xs).to(torch.bfloat16)
+    topk = np.stack([np.stack([rng.permutation(E)[:K] for _ in range(T)]) for _ in range(R)]).astype(np.int32)
+    topk[rng.random((R, T, K)) < 0.1] = -1
+    w = rng.random((R, T, K)).astype(np.float32)
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, rx, torch.zeros_like(rx))
+    out, _, _ = buf.combine(y, td, wd, handle, use_logfmt=True)
+    plain, _, _ = buf.combine(y, td, wd, handle)
+    torch.cuda.synchronize()
+    again, _, _ = buf.combine(y, td, wd, handle, use_logfmt=True)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))  # deterministic on one GPU
+    want = eo.ll_combine(bits16(y).reshape(R, El, R * M, H), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(), E, M,
+                         use_logfmt=True)
+    g, o = eo.bf16_to_f32(bits16(out).reshape(R, T, H)), eo.bf16_to_f32(want)
+    assert np.mean(g == o) > 0.98
+    scale = np.abs(xs).max(axis=2, keepdims=True) * np.abs(w).sum(axis=2, keepdims=True)
+    assert np.all(np.abs(g - o) <= (2.0 ** (32 / 510) - 1) * scale + 1e-6)
+    # lossy but close to the uncompressed sum, and not identical to it
+    p = eo.bf16_to_f32(bits16(plain).reshape(R, T, H))
+    assert not np.array_equal(g, p)
+    assert calc_diff(torch.from_numpy(g), torch.from_numpy(p)) < 1e-5
+    ideal = x.float().numpy() * np.where(topk >= 0, w, 0).sum(axis=2, keepdims=True)
+    assert calc_diff(torch.from_numpy(g), torch.from_numpy(ideal)) < 1e-5

@@ -430,3 +430,79 @@ def test_low_latency_buffer_size_hint_follows_the_reference_layout():
     small = Buffer.get_low_latency_buffer_size_hint(64, 2048, 2, 1)
     d, c = 16 + 2048 * 2, 16 * 4 + 2048 * 2
     assert small == (2 * max(64 * d, 64 * c) + 2 * max(64 * d, 64 * c) + 2 * 128 + 128) // 128 * 128
+
+
+def _logfmt_reference_f64(vals):
+    """LogFMT-10 round trip of one 128-channel group in float64 from its definition
+    (examples/device/ep/csrc/kernels/nixl_ep_ll.cu:459-616): returns (decoded, step) or
+    (vals, None) when the group is not cast."""
+    a = np.abs(vals.astype(np.float64))
+    amax, amin = a.max(), a.min()
+    with np.errstate(divide="ignore"):
+        log_amax = np.log2(amax) if amax > 0 else -np.inf
+        log_amin = max(np.log2(amin) if amin > 0 else -np.inf, log_amax - 32)
+    if not (log_amax < 0 and log_amin < log_amax):
+        return vals.astype(np.float64), None
+    step = (log_amax - log_amin) / 510
+    rounding = 2 - np.log2((1 + 2.0 ** step) * 0.5) / step
+    with np.errstate(divide="ignore"):
+        pos = np.maximum(np.where(a > 0, np.log2(np.where(a > 0, a, 1)), -np.inf) / step + rounding - log_amin / step, 0)
+    code = np.floor(pos)
+    dec = np.where(code == 0, 0.0, 2.0 ** ((code - 1) * step + log_amin))
+    return np.where(np.signbit(vals), -dec, dec), step
+
+
+def test_logfmt_roundtrip_against_float64_definition_and_properties():
+    rng = np.random.default_rng(77)
+    groups = [rng.standard_normal(128) * s for s in (0.5, 0.1, 0.01, 1e-3, 1e-6)]
+    groups.append(rng.standard_normal(128) * 3.0)          # amax >= 1: not cast
+    groups.append(np.full(128, 0.25))                       # constant: not cast
+    z = rng.standard_normal(128) * 0.2
+    z[::7] = 0.0
+    z[5] = -0.0
+    groups.append(z)                                        # zeros inside a cast group
+    groups.append(np.concatenate([[0.9], np.full(127, 1e-30)]))  # range wider than 2^32: amin floored
+    row = eo.f32_to_bf16(np.concatenate(groups).astype(np.float32))
+    vals = eo.bf16_to_f32(row)
+    got = eo.logfmt_roundtrip(row)
+    for i in range(len(groups)):
+        v, g = vals[i * 128:(i + 1) * 128], got[i * 128:(i + 1) * 128]
+        want, step = _logfmt_reference_f64(v)
+        if step is None:
+            assert np.array_equal(g, v), i  # untouched
+            continue
+        assert np.array_equal(np.signbit(g), np.signbit(v)), i
+        assert np.array_equal(g == 0, (want == 0)), i
+        nz = want != 0
+        # fp32 evaluation may land one code off the float64 one at a floor boundary
+        ratio = np.abs(g[nz] / want[nz])
+        assert np.all((ratio < 2.0 ** (1.01 * step)) & (ratio > 2.0 ** (-1.01 * step))), i
+        assert np.mean(np.abs(np.log2(ratio)) < 1e-3) > 0.9, i  # almost all on the same code
+        # the codec's own promise: what comes back is within half a step (in log2) of what went in,
+        # except below the smallest representable level
+        a = np.abs(v[nz].astype(np.float64))
+        floor_level = 2.0 ** (np.log2(np.abs(v).max()) - 32) if i == len(groups) - 1 else 0
+        big = a > floor_level * 2
+        err = np.abs(np.log2(np.abs(g[nz][big]) / a[big]))
+        assert np.all(err <= 0.51 * step + 1e-6), (i, err.max(), step)
+    # monotone: a larger magnitude never decodes to a smaller one
+    cast_group = eo.f32_to_bf16(np.sort(np.abs(rng.standard_normal(128)) * 0.3).astype(np.float32))
+    dec = eo.logfmt_roundtrip(cast_group)
+    assert np.all(np.diff(dec) >= 0)
+
+
+def test_ll_combine_logfmt_is_the_sum_of_decoded_rows():
+    R, T, H, K, E, M = 2, 5, 256, 2, 4, 8
+    rng = np.random.default_rng(78)
+    x = eo.f32_to_bf16((rng.standard_normal((R, T, H)) * 0.3).astype(np.float32))
+    topk = np.stack([np.stack([rng.permutation(E)[:K] for _ in range(T)]) for _ in range(R)]).astype(np.int32)
+    w = rng.random((R, T, K)).astype(np.float32)
+    o = eo.ll_dispatch(x, topk, E, M, use_fp8=False)
+    out = eo.ll_combine(o["recv_x"], topk, w, o["src_info"], o["layout_range"], E, M, use_logfmt=True)
+    for r in range(R):
+        for t in range(T):
+            dec = eo.logfmt_roundtrip(x[r, t])  # every destination holds the token's own row
+            acc = np.zeros(H, np.float32)
+            for k in range(K):
+                acc = (dec.astype(np.float64) * np.float64(w[r, t, k]) + acc).astype(np.float32)
+            assert np.array_equal(out[r, t], eo.f32_to_bf16(acc)) or np.max(np.abs(eo.bf16_to_f32(out[r, t]) - acc)) < 1e-2
