@@ -16,6 +16,12 @@
  *   layout_range      [R][El][R]       int64: low 32 bits = count, high 32 bits = begin
  *   recv_count        [R][El]          int32
  * Rows of packed_recv_x / scales / src_info at or beyond recv_count are left untouched.
+ *
+ * Parity unpinned: oracle_router (the reference has no router; pinned against torch CPU only)
+ * and oracle_logfmt_roundtrip at bit level (the reference evaluates log2 / exp2 with
+ * approximate GPU instructions; pinned against a float64 evaluation of the definition and the
+ * codec's error bound).  Everything else is pinned by library routines, format definitions,
+ * brute force and the reference tests' invariants (tests/test_ep_oracle.py, tests/test_golden.py).
  */
 #ifndef NIXL_AMD_EP_ORACLE_H
 #define NIXL_AMD_EP_ORACLE_H
