@@ -200,8 +200,10 @@ collect_rows(const uint8_t *in_rank,
         int n = 0;
         for (int d0 = 0; d0 < d.R; d0 += kWaveSize) {
             const int dst = d0 + lane;
-            const bool hit = dst < d.R && in_rank[tok * d.R + dst] != 0;
-            const long long row = hit ? recv_row(prefix, send_head, row_offset, d, r, t, dst) : 0;
+            bool hit = dst < d.R && in_rank[tok * d.R + dst] != 0;
+            long long row = hit ? recv_row(prefix, send_head, row_offset, d, r, t, dst) : 0;
+            // the handle comes from the caller: a row outside the destination's range is dropped
+            if (hit && (row < row_offset[dst] || row >= row_offset[dst + 1])) hit = false;
             const unsigned long long m = __ballot(hit);
             if (hit) {
                 const int p = n + __popcll(m & ((1ull << lane) - 1ull));
@@ -274,6 +276,7 @@ ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
     const size_t tok = static_cast<size_t>(r) * d.T + t;
     if (!in_rank[tok * d.R + dst]) return;
     const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+    if (row < row_offset[dst] || row >= row_offset[dst + 1]) return;
     const int El = d.E / d.R;
     if (recv_topk_idx)
         for (int k = 0; k < d.K; ++k) {

@@ -286,7 +286,7 @@ ll_scales_kernel(ScalesArgs a) {
     if (!a.recv_scales) return;
     const int n = seg_end[d.R - 1];
     for (int slot = tid; slot < n; slot += kLayoutThreads) {
-        const int t = t_next;
+        const int t = min(max(t_next, 0), d.T - 1); // written by the dispatch kernel; clamped so that a stale buffer cannot fault
         if (slot + kLayoutThreads < n) t_next = a.src_info[static_cast<size_t>(e) * d.N + slot + kLayoutThreads];
         int lo = 0, hi = d.R - 1; // first rank whose segment ends beyond `slot`
         while (lo < hi) {
@@ -400,6 +400,7 @@ ll_combine_kernel(CombineArgs a) {
             const int e = a.topk_idx[sel];
             long long row = a.row_map[sel];
             if (e < 0 || e >= d.E || pair_blocked(a.mask, d.R, r, e / d.El)) row = -1;
+            if (row >= static_cast<long long>(d.E) * d.N) row = -1; // a foreign handle must not make the kernel fault
             row_of_k[tid] = row;
             weight_of_k[tid] = a.topk_weights[sel];
         }
@@ -411,7 +412,9 @@ ll_combine_kernel(CombineArgs a) {
         long long row = -1;
         if (e >= 0 && e < d.E && !pair_blocked(a.mask, d.R, r, e / d.El)) {
             const long long lr = a.layout_range[static_cast<size_t>(e) * d.R + r];
-            const int n = static_cast<int>(lr & 0xffffffffll), begin = static_cast<int>(lr >> 32);
+            int n = static_cast<int>(lr & 0xffffffffll), begin = static_cast<int>(lr >> 32);
+            begin = min(max(begin, 0), d.N); // the handle comes from the caller: keep the search inside the expert
+            n = min(max(n, 0), d.N - begin);
             const int *seg = a.src_info + static_cast<size_t>(e) * d.N + begin;
             for (int i0 = 0; i0 < n && row < 0; i0 += kWaveSize) {
                 const int i = i0 + lane;
