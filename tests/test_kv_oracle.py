@@ -246,3 +246,16 @@ def test_config1_dram_loopback_bit_exact(cpu_agent):
     assert a.check_xfer_state(req2) == "DONE" and np.array_equal(back, src)
     for h in (req, req2, hl, hr, hb):
         h.release()
+
+
+def test_sorted_region_list_matches_reference_expectations():
+    """tests/cpp/sec_desc_list_check.cpp: the agent's registration list against the orderings
+    the reference's unit tests state for nixlSecDescList, and the covering search on top."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "sec_desc_list_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert proc.returncode == 0 and proc.stdout.strip() == "OK", proc.stdout + proc.stderr
