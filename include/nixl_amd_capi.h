@@ -77,6 +77,9 @@ typedef struct nixl_capi_xfer_dlist_handle_s *nixl_capi_xfer_dlist_handle_t;
 typedef struct nixl_capi_reg_dlist_s *nixl_capi_reg_dlist_t;
 typedef struct nixl_capi_xfer_req_s *nixl_capi_xfer_req_t;
 typedef struct nixl_capi_xfer_telemetry_s *nixl_capi_xfer_telemetry_t;
+typedef struct nixl_capi_string_list_s *nixl_capi_string_list_t;
+typedef struct nixl_capi_mem_list_s *nixl_capi_mem_list_t;
+typedef struct nixl_capi_param_iter_s *nixl_capi_param_iter_t;
 
 /* agent */
 nixl_capi_status_t nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent);
@@ -186,6 +189,57 @@ nixl_capi_status_t nixl_capi_xfer_dlist_handle_run_count(nixl_capi_xfer_dlist_ha
 /* Post, then poll until the request leaves NIXL_IN_PROG; returns the final status.
  * Saves one foreign-function round trip per poll in timing loops. */
 nixl_capi_status_t nixl_capi_post_and_wait(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl);
+
+/* Plugin and backend queries (reference wrapper.h:66-88,119-137).  Lists and iterators are
+ * owned by the caller and freed with their destroy function; strings stay valid as long as
+ * the object they came from. */
+nixl_capi_status_t
+nixl_capi_get_available_plugins(nixl_capi_agent_t agent, nixl_capi_string_list_t *plugins);
+nixl_capi_status_t
+nixl_capi_destroy_string_list(nixl_capi_string_list_t list);
+nixl_capi_status_t
+nixl_capi_string_list_size(nixl_capi_string_list_t list, size_t *size);
+nixl_capi_status_t
+nixl_capi_string_list_get(nixl_capi_string_list_t list, size_t index, const char **str);
+nixl_capi_status_t
+nixl_capi_get_plugin_params(nixl_capi_agent_t agent, const char *plugin_name, nixl_capi_mem_list_t *mems,
+                            nixl_capi_params_t *params);
+nixl_capi_status_t
+nixl_capi_get_backend_params(nixl_capi_agent_t agent, nixl_capi_backend_t backend, nixl_capi_mem_list_t *mems,
+                             nixl_capi_params_t *params);
+nixl_capi_status_t
+nixl_capi_destroy_mem_list(nixl_capi_mem_list_t list);
+nixl_capi_status_t
+nixl_capi_mem_list_is_empty(nixl_capi_mem_list_t list, bool *is_empty);
+nixl_capi_status_t
+nixl_capi_mem_list_size(nixl_capi_mem_list_t list, size_t *size);
+nixl_capi_status_t
+nixl_capi_mem_list_get(nixl_capi_mem_list_t list, size_t index, nixl_capi_mem_type_t *mem_type);
+nixl_capi_status_t
+nixl_capi_mem_type_to_string(nixl_capi_mem_type_t mem_type, const char **str);
+nixl_capi_status_t
+nixl_capi_params_is_empty(nixl_capi_params_t params, bool *is_empty);
+nixl_capi_status_t
+nixl_capi_params_create_iterator(nixl_capi_params_t params, nixl_capi_param_iter_t *iter);
+nixl_capi_status_t
+nixl_capi_params_iterator_next(nixl_capi_param_iter_t iter, const char **key, const char **value, bool *has_next);
+nixl_capi_status_t
+nixl_capi_params_destroy_iterator(nixl_capi_param_iter_t iter);
+
+/* Cost estimate and backend of a request (reference wrapper.h:271-287). */
+typedef enum {
+    NIXL_CAPI_COST_ANALYTICAL_BACKEND = 0,
+} nixl_capi_cost_t;
+
+nixl_capi_status_t
+nixl_capi_estimate_xfer_cost(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_opt_args_t opt_args,
+                             int64_t *duration_us, int64_t *err_margin_us, nixl_capi_cost_t *method);
+nixl_capi_status_t
+nixl_capi_query_xfer_backend(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_backend_t *backend);
+/* extension: the plugin name a backend handle was created from; the string is valid until
+ * the calling thread makes this call again */
+nixl_capi_status_t
+nixl_capi_backend_get_type(nixl_capi_backend_t backend, const char **type);
 
 #ifdef __cplusplus
 }

@@ -174,6 +174,24 @@ _CAPI_SIGS = {
     "nixl_capi_xfer_req_desc_count": [c_void_p, POINTER(c_size_t), POINTER(c_size_t)],
     "nixl_capi_xfer_req_get_desc": [c_void_p, c_size_t, POINTER(c_uint64), POINTER(c_uint64),
                                     POINTER(c_uint64)],
+    "nixl_capi_get_available_plugins": [c_void_p, POINTER(c_void_p)],
+    "nixl_capi_destroy_string_list": [c_void_p],
+    "nixl_capi_string_list_size": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_string_list_get": [c_void_p, c_size_t, POINTER(c_char_p)],
+    "nixl_capi_get_plugin_params": [c_void_p, c_char_p, POINTER(c_void_p), POINTER(c_void_p)],
+    "nixl_capi_get_backend_params": [c_void_p, c_void_p, POINTER(c_void_p), POINTER(c_void_p)],
+    "nixl_capi_destroy_mem_list": [c_void_p],
+    "nixl_capi_mem_list_is_empty": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_mem_list_size": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_mem_list_get": [c_void_p, c_size_t, POINTER(c_int)],
+    "nixl_capi_mem_type_to_string": [c_int, POINTER(c_char_p)],
+    "nixl_capi_params_is_empty": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_params_create_iterator": [c_void_p, POINTER(c_void_p)],
+    "nixl_capi_params_iterator_next": [c_void_p, POINTER(c_char_p), POINTER(c_char_p), POINTER(c_bool)],
+    "nixl_capi_params_destroy_iterator": [c_void_p],
+    "nixl_capi_estimate_xfer_cost": [c_void_p, c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int)],
+    "nixl_capi_query_xfer_backend": [c_void_p, c_void_p, POINTER(c_void_p)],
+    "nixl_capi_backend_get_type": [c_void_p, POINTER(c_char_p)],
     "nixl_capi_release_xfer_req": [c_void_p, c_void_p],
     "nixl_capi_destroy_xfer_req": [c_void_p],
 }

@@ -54,8 +54,19 @@ def _check(where, rc, ok=(0,)):
     return rc
 
 
+def _tensors_of(descs):
+    """The tensors in `descs` if it is a tensor or a list of tensors, else None."""
+    if hasattr(descs, "data_ptr"):
+        return [descs]
+    if not isinstance(descs, np.ndarray) and len(descs) and all(hasattr(d, "data_ptr") for d in descs):
+        return list(descs)
+    return None
+
+
 def _as_triples(descs):
     """Normalise a descriptor list to a C-contiguous (N, 3) uint64 array."""
+    if hasattr(descs, "data_ptr"):
+        descs = [descs]
     if isinstance(descs, np.ndarray):
         arr = descs
     else:
@@ -75,8 +86,9 @@ def _as_triples(descs):
 def _guess_mem(descs, mem_type):
     if mem_type is not None:
         return _MEM[mem_type]
-    if not isinstance(descs, np.ndarray) and len(descs) and hasattr(descs[0], "data_ptr"):
-        return _MEM[descs[0].device.type]
+    tensors = _tensors_of(descs)
+    if tensors:
+        return _MEM[tensors[0].device.type]
     raise ValueError("mem_type is required for raw address lists")
 
 
@@ -184,6 +196,8 @@ class nixl_agent:
     """Reference: nixl_agent, src/api/python/_api.py:189-296."""
 
     def __init__(self, agent_name, nixl_conf=None, plugin_dirs=()):
+        if not agent_name:
+            raise ValueError("agent name must not be empty")  # as the reference bindings do
         self._lib = _lib.agent_lib()
         self.name = agent_name
         conf = nixl_conf or nixl_agent_config(backends=())
@@ -227,6 +241,97 @@ class nixl_agent:
         finally:
             self._lib.nixl_capi_destroy_params(params)
 
+    # -- plugin and backend queries (reference: _api.py:308-389) ----------------------------
+    _MEM_NAMES = {0: "DRAM", 1: "VRAM", 2: "BLK", 3: "OBJ", 4: "FILE"}
+
+    def get_plugin_list(self):
+        lst = ctypes.c_void_p()
+        _check("get_plugin_list", self._lib.nixl_capi_get_available_plugins(self._h, ctypes.byref(lst)))
+        try:
+            n = ctypes.c_size_t()
+            self._lib.nixl_capi_string_list_size(lst, ctypes.byref(n))
+            out = []
+            for i in range(n.value):
+                s = ctypes.c_char_p()
+                self._lib.nixl_capi_string_list_get(lst, i, ctypes.byref(s))
+                out.append(s.value.decode())
+            return out
+        finally:
+            self._lib.nixl_capi_destroy_string_list(lst)
+
+    def _mems_and_params(self, rc, mems, params):
+        """Unpack and free the (memory list, parameters) pair of a query; an unknown name
+        gives two empty results, as in the reference (test_nixl_api.py:145-154)."""
+        if rc != 0:
+            return [], {}
+        try:
+            n = ctypes.c_size_t()
+            self._lib.nixl_capi_mem_list_size(mems, ctypes.byref(n))
+            mem_names = []
+            for i in range(n.value):
+                m = ctypes.c_int()
+                self._lib.nixl_capi_mem_list_get(mems, i, ctypes.byref(m))
+                mem_names.append(self._MEM_NAMES.get(m.value, "UNKNOWN"))
+            out = {}
+            empty = ctypes.c_bool()
+            self._lib.nixl_capi_params_is_empty(params, ctypes.byref(empty))
+            if not empty.value:
+                it = ctypes.c_void_p()
+                self._lib.nixl_capi_params_create_iterator(params, ctypes.byref(it))
+                more = ctypes.c_bool(True)
+                while more.value:
+                    k, v = ctypes.c_char_p(), ctypes.c_char_p()
+                    if self._lib.nixl_capi_params_iterator_next(it, ctypes.byref(k), ctypes.byref(v), ctypes.byref(more)) != 0:
+                        break
+                    out[k.value.decode()] = v.value.decode()
+                self._lib.nixl_capi_params_destroy_iterator(it)
+            return mem_names, out
+        finally:
+            self._lib.nixl_capi_destroy_mem_list(mems)
+            self._lib.nixl_capi_destroy_params(params)
+
+    def _plugin_query(self, name):
+        mems, params = ctypes.c_void_p(), ctypes.c_void_p()
+        rc = self._lib.nixl_capi_get_plugin_params(self._h, name.encode(), ctypes.byref(mems), ctypes.byref(params))
+        return self._mems_and_params(rc, mems, params)
+
+    def _backend_query(self, name):
+        if name not in self.backends:
+            return [], {}
+        mems, params = ctypes.c_void_p(), ctypes.c_void_p()
+        rc = self._lib.nixl_capi_get_backend_params(self._h, self.backends[name], ctypes.byref(mems), ctypes.byref(params))
+        return self._mems_and_params(rc, mems, params)
+
+    def get_plugin_mem_types(self, backend):
+        return self._plugin_query(backend)[0]
+
+    def get_plugin_params(self, backend):
+        return self._plugin_query(backend)[1]
+
+    def get_backend_mem_types(self, backend):
+        return self._backend_query(backend)[0]
+
+    def get_backend_params(self, backend):
+        return self._backend_query(backend)[1]
+
+    def estimate_xfer_cost(self, req_handle):
+        """Reference: _api.py:534-551.  (duration_us, err_margin_us, method)."""
+        d, e, m = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int()
+        _check("estimate_xfer_cost", self._lib.nixl_capi_estimate_xfer_cost(self._h, req_handle._handle, None, ctypes.byref(d),
+                                                                             ctypes.byref(e), ctypes.byref(m)))
+        return d.value, e.value, m.value
+
+    def query_xfer_backend(self, handle):
+        """Reference: _api.py:694-707: the name of the backend a request was bound to."""
+        b = ctypes.c_void_p()
+        _check("query_xfer_backend", self._lib.nixl_capi_query_xfer_backend(self._h, handle._handle, ctypes.byref(b)))
+        try:
+            name = ctypes.c_char_p()
+            _check("backend_get_type", self._lib.nixl_capi_backend_get_type(b, ctypes.byref(name)))
+            return name.value.decode()
+        finally:
+            self._lib.nixl_capi_destroy_backend(b)
+
     def _opt_args(self, backends=(), skip_desc_merge=False, notif_msg=b""):
         if not backends and not skip_desc_merge and not notif_msg:
             return None
@@ -247,13 +352,23 @@ class nixl_agent:
 
     # -- descriptors ------------------------------------------------------------------
     def get_xfer_descs(self, descs, mem_type=None):
+        """Reference: _api.py:999-1115.  Accepts a list of (addr, len, devId) tuples or an
+        (N, 3) array with a memory type, a tensor, or a list of tensors; a tensor that is not
+        contiguous cannot be described by one range and yields None."""
         if isinstance(descs, nixl_xfer_dlist):
             return descs
+        tensors = _tensors_of(descs)
+        if tensors and not all(t.is_contiguous() for t in tensors):
+            return None
         return nixl_xfer_dlist(_as_triples(descs), _guess_mem(descs, mem_type))
 
     def get_reg_descs(self, descs, mem_type=None):
+        """Reference: _api.py:1117-1230; same inputs as get_xfer_descs."""
         if isinstance(descs, nixl_reg_dlist):
             return descs
+        tensors = _tensors_of(descs)
+        if tensors and not all(t.is_contiguous() for t in tensors):
+            return None
         return nixl_reg_dlist(_as_triples(descs), _guess_mem(descs, mem_type))
 
     # -- registration -----------------------------------------------------------------

@@ -30,6 +30,15 @@ struct nixl_capi_reg_dlist_s {
 struct nixl_capi_xfer_req_s {
     nixlXferReqH *req;
 };
+struct nixl_capi_string_list_s {
+    std::vector<std::string> strings;
+};
+struct nixl_capi_mem_list_s {
+    nixl_mem_list_t mems;
+};
+struct nixl_capi_param_iter_s {
+    nixl_b_params_t::const_iterator it, end;
+};
 
 namespace {
 
@@ -440,6 +449,181 @@ nixl_capi_status_t
 nixl_capi_destroy_xfer_req(nixl_capi_xfer_req_t req) {
     if (!req) return NIXL_CAPI_ERROR_INVALID_PARAM;
     delete req; // the inner request was handed back by nixl_capi_release_xfer_req
+    return NIXL_CAPI_SUCCESS;
+}
+
+// ---- plugin and backend queries ---------------------------------------------------------------
+
+nixl_capi_status_t
+nixl_capi_get_available_plugins(nixl_capi_agent_t agent, nixl_capi_string_list_t *plugins) {
+    if (!agent || !plugins) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        std::vector<nixl_backend_t> names;
+        const nixl_status_t st = agent->inner->getAvailPlugins(names);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *plugins = new nixl_capi_string_list_s{std::move(names)};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_string_list(nixl_capi_string_list_t list) {
+    if (!list) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete list;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_string_list_size(nixl_capi_string_list_t list, size_t *size) {
+    if (!list || !size) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *size = list->strings.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_string_list_get(nixl_capi_string_list_t list, size_t index, const char **str) {
+    if (!list || !str || index >= list->strings.size()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *str = list->strings[index].c_str();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_get_plugin_params(nixl_capi_agent_t agent, const char *plugin_name, nixl_capi_mem_list_t *mems,
+                            nixl_capi_params_t *params) {
+    if (!agent || !plugin_name || !mems || !params) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_mem_list_t m;
+        nixl_b_params_t p;
+        const nixl_status_t st = agent->inner->getPluginParams(plugin_name, m, p);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *mems = new nixl_capi_mem_list_s{std::move(m)};
+        *params = new nixl_capi_params_s{std::move(p)};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_get_backend_params(nixl_capi_agent_t agent, nixl_capi_backend_t backend, nixl_capi_mem_list_t *mems,
+                             nixl_capi_params_t *params) {
+    if (!agent || !backend || !mems || !params) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_mem_list_t m;
+        nixl_b_params_t p;
+        const nixl_status_t st = agent->inner->getBackendParams(backend->backend, m, p);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *mems = new nixl_capi_mem_list_s{std::move(m)};
+        *params = new nixl_capi_params_s{std::move(p)};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_mem_list(nixl_capi_mem_list_t list) {
+    if (!list) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete list;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_mem_list_is_empty(nixl_capi_mem_list_t list, bool *is_empty) {
+    if (!list || !is_empty) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *is_empty = list->mems.empty();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_mem_list_size(nixl_capi_mem_list_t list, size_t *size) {
+    if (!list || !size) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *size = list->mems.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_mem_list_get(nixl_capi_mem_list_t list, size_t index, nixl_capi_mem_type_t *mem_type) {
+    if (!list || !mem_type || index >= list->mems.size()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *mem_type = static_cast<nixl_capi_mem_type_t>(list->mems[index]);
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_mem_type_to_string(nixl_capi_mem_type_t mem_type, const char **str) {
+    if (!str) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    static const char *const names[] = {"DRAM_SEG", "VRAM_SEG", "BLK_SEG", "OBJ_SEG", "FILE_SEG"};
+    if (mem_type < NIXL_CAPI_MEM_DRAM || mem_type > NIXL_CAPI_MEM_FILE) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *str = names[mem_type];
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_params_is_empty(nixl_capi_params_t params, bool *is_empty) {
+    if (!params || !is_empty) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *is_empty = params->params.empty();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_params_create_iterator(nixl_capi_params_t params, nixl_capi_param_iter_t *iter) {
+    if (!params || !iter) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *iter = new nixl_capi_param_iter_s{params->params.cbegin(), params->params.cend()};
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_params_iterator_next(nixl_capi_param_iter_t iter, const char **key, const char **value, bool *has_next) {
+    if (!iter || !key || !value || !has_next) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    if (iter->it == iter->end) {
+        *has_next = false;
+        return NIXL_CAPI_ERROR_INVALID_STATE;
+    }
+    *key = iter->it->first.c_str();
+    *value = iter->it->second.c_str();
+    ++iter->it;
+    *has_next = iter->it != iter->end;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_params_destroy_iterator(nixl_capi_param_iter_t iter) {
+    if (!iter) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete iter;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_estimate_xfer_cost(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_opt_args_t opt_args,
+                             int64_t *duration_us, int64_t *err_margin_us, nixl_capi_cost_t *method) {
+    if (!agent || !req_hndl || !duration_us || !err_margin_us || !method) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        std::chrono::microseconds duration{0}, margin{0};
+        nixl_cost_t how = nixl_cost_t::ANALYTICAL_BACKEND;
+        const nixl_status_t st =
+            agent->inner->estimateXferCost(req_hndl->req, duration, margin, how, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *duration_us = duration.count();
+        *err_margin_us = margin.count();
+        *method = static_cast<nixl_capi_cost_t>(how);
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_query_xfer_backend(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_hndl, nixl_capi_backend_t *backend) {
+    if (!agent || !req_hndl || !backend) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlBackendH *b = nullptr;
+        const nixl_status_t st = agent->inner->queryXferBackend(req_hndl->req, b);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *backend = new nixl_capi_backend_s{b};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_backend_get_type(nixl_capi_backend_t backend, const char **type) {
+    if (!backend || !backend->backend || !type) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    thread_local std::string name;
+    name = backend->backend->getType();
+    *type = name.c_str();
     return NIXL_CAPI_SUCCESS;
 }
 

@@ -259,3 +259,37 @@ def test_sorted_region_list_matches_reference_expectations():
         pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
     proc = subprocess.run([exe], capture_output=True, text=True, timeout=60)
     assert proc.returncode == 0 and proc.stdout.strip() == "OK", proc.stdout + proc.stderr
+
+
+def test_api_behaviour_of_the_reference_python_tests(cpu_agent, oracle_plugin_dir):
+    """Cases of the reference's test/python/test_nixl_api.py that concern one agent:
+    empty name (:90-93), unknown operation (:135-142), unknown plugin name gives empty
+    answers (:145-154) and cannot be created (:157-160), non-contiguous tensors (:358-371)."""
+    import torch
+    a = cpu_agent
+    with pytest.raises(ValueError):
+        nixl_agent("")
+    x = np.zeros(256, np.uint8)
+    reg = a.register_memory(np.array([[x.ctypes.data, x.nbytes, 0]], dtype=np.uint64), "DRAM")
+    l = a.get_xfer_descs(np.array([[x.ctypes.data, 64, 0]], dtype=np.uint64), "DRAM")
+    r = a.get_xfer_descs(np.array([[x.ctypes.data + 128, 64, 0]], dtype=np.uint64), "DRAM")
+    with pytest.raises(KeyError):
+        a.initialize_xfer("WR", l, r, a.name)
+    with pytest.raises(KeyError):
+        a.make_prepped_xfer("RD", None, [], None, [])
+    assert a.get_plugin_mem_types("UVX") == [] and a.get_plugin_params("UVX") == {}
+    assert a.get_backend_mem_types("UVX") == [] and a.get_backend_params("UVX") == {}
+    with pytest.raises(ag.NixlError) as err:
+        a.create_backend("UVX")
+    assert err.value.status == ag.NIXL_ERR_NOT_FOUND
+    # what a real plugin answers
+    assert "MEMCPY" in a.get_plugin_list()
+    assert a.get_plugin_mem_types("MEMCPY") == ["DRAM"] and a.get_plugin_params("MEMCPY") == {"threads": "1"}
+    assert a.get_backend_mem_types("MEMCPY") == ["DRAM"]
+    req = a.initialize_xfer("WRITE", l, r, a.name)
+    assert a.query_xfer_backend(req) == "MEMCPY"
+    req.release()
+    a.deregister_memory(reg)
+    cont = torch.arange(8).reshape(2, 4)
+    assert a.get_reg_descs(torch.transpose(cont, 0, 1)) is None and a.get_xfer_descs(torch.transpose(cont, 0, 1)) is None
+    assert a.get_xfer_descs(cont, "DRAM").descCount() == 1  # a single tensor, not only a list
