@@ -147,6 +147,57 @@ def run_kv(args):
     return out
 
 
+def run_small_descriptors(steps=20, warmup=3):
+    """Small-descriptor stress: 262 144 VRAM->VRAM descriptors with sizes log-uniform in
+    [512 B, 4 KiB] rounded to 16 B, random 16-byte-aligned offsets in two 4 GiB buffers,
+    destinations non-overlapping.  One request through the agent; HIP events on the launch
+    stream around every post."""
+    import torch
+    from nixl_amd import nixl_agent, nixl_agent_config
+    dev = torch.device("cuda:0")
+    n, buf_bytes = 262144, 4 << 30
+    rng = np.random.default_rng(2025)
+    lens = ((np.exp(rng.uniform(np.log(512), np.log(4096), n)).astype(np.int64) // 16) * 16).astype(np.uint64)
+    src = torch.zeros(buf_bytes, dtype=torch.uint8, device=dev)
+    dst = torch.zeros(buf_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.Stream(device=dev)
+    agent = nixl_agent("small", nixl_agent_config(backends=()))
+    agent.create_backend("HIP", {"stream": str(stream.cuda_stream)})
+    agent.register_memory([src, dst])
+    so = (rng.integers(0, (buf_bytes - 4096) // 16, n) * 16).astype(np.uint64)
+    do = (rng.permutation(buf_bytes // 8192)[:n] * 8192 + rng.integers(0, (8192 - 4096) // 16, n) * 16).astype(np.uint64)
+    zeros = np.zeros(n, dtype=np.uint64)
+    hl = agent.prep_xfer_dlist("", np.stack([np.uint64(src.data_ptr()) + so, lens, zeros], 1), "VRAM")
+    hr = agent.prep_xfer_dlist("small", np.stack([np.uint64(dst.data_ptr()) + do, lens, zeros], 1), "VRAM")
+    idx = np.arange(n)
+    req = agent.make_prepped_xfer("WRITE", hl, idx, hr, idx)
+    torch.cuda.synchronize()
+    times = []
+    for i in range(warmup + steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        state = agent.transfer(req)
+        e1.record(stream)
+        while state == "PROC":
+            state = agent.check_xfer_state(req)
+        if state != "DONE":
+            raise RuntimeError(f"transfer ended in state {state}")
+        e1.synchronize()
+        if i >= warmup:
+            times.append(e0.elapsed_time(e1) * 1e3)
+    payload = int(lens.sum())
+    us = float(np.mean(times))
+    for h in (req, hl, hr):
+        h.release()
+    agent.close()
+    del src, dst
+    torch.cuda.empty_cache()
+    gbps = 2 * payload / (us * 1e-6) / 1e9
+    return {"descriptors": n, "payload_bytes": payload, "avg_launch_us": round(us, 1), "achieved_GBps": round(gbps, 1),
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "ns_per_descriptor": round(us * 1e3 / n, 3),
+            "kernel": "copy_piece_kernel<true,4>"}
+
+
 def run_calibration_copy():
     """One launch of torch's element-wise add over 2^28 int32: reads exactly 1 GiB, writes 1 GiB."""
     import torch
@@ -222,6 +273,7 @@ def main():
     ap.add_argument("--block-bytes", type=int, default=32768, help="bytes per (layer, K|V) sub-block")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ep", action="store_true")
+    ap.add_argument("--no-small", action="store_true", help="skip the small-descriptor stress")
     ap.add_argument("--ep-iters", type=int, default=50, help="timed calls per expert-parallel kernel")
     ap.add_argument("--ep-warmup", type=int, default=20)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -268,6 +320,8 @@ def main():
             "value_GBps": round(kv16["value"], 1), "avg_launch_ms": kv16["roofline"]["avg_launch_ms"],
             "achieved_GBps": kv16["roofline"]["achieved"], "frac": kv16["roofline"]["frac"],
             "descriptors_per_request": kv16["kv"]["descriptors_per_request"]}
+    if not args.no_small:
+        line["kv"]["small_descriptor_stress"] = run_small_descriptors()
     if not args.no_ep:
         try:
             from nixl_amd import ep_bench
