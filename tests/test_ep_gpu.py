@@ -750,3 +750,36 @@ def test_ll_combine_logfmt(cuda):
     assert calc_diff(torch.from_numpy(g), torch.from_numpy(p)) < 1e-5
     ideal = x.float().numpy() * np.where(topk >= 0, w, 0).sum(axis=2, keepdims=True)
     assert calc_diff(torch.from_numpy(g), torch.from_numpy(ideal)) < 1e-5
+
+
+def test_ll_narrow_workgroups_give_the_same_bytes(cuda):
+    """nixl_amd_ep_ll_set_tuning: with workgroups of 64 and 128 lanes a token's row is split
+    over several workgroups in dispatch and combine; results must not change."""
+    k = _lib.ep_kernels()
+    R, T, H, K, E, M = 4, 9, 2048, 4, 8, 12
+    x, topk, w = make_world(123, R, T, H, K, E, drop=0.1, scale=2.0)
+    want = eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, True, fill=0x55)
+    try:
+        assert k.nixl_amd_ep_ll_set_tuning(100, 0) < 0 and k.nixl_amd_ep_ll_set_tuning(0, 2048) < 0
+        for lanes in (64, 128, 1024):
+            assert k.nixl_amd_ep_ll_set_tuning(lanes, lanes) == 0
+            rc, got = raw_ll_dispatch(cuda, x, topk, E, M, True)
+            assert rc == 0, _lib.kernels_error()
+            assert_dispatch_equal(got, want, True)
+            buf = Buffer(R, device=cuda)
+            td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+            rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+            valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+            y = torch.where(valid, rx, torch.zeros_like(rx))
+            for h in (handle, tuple(handle)):
+                for logfmt in (False, True):
+                    out, _, _ = buf.combine(y, td, wd, h, use_logfmt=logfmt)
+                    torch.cuda.synchronize()
+                    ref = eo.ll_combine(bits16(y).reshape(R, E // R, R * M, H), topk, w, handle[0].cpu().numpy(),
+                                        handle[1].cpu().numpy(), E, M, use_fma=True, use_logfmt=logfmt)
+                    if logfmt:
+                        assert np.mean(bits16(out).reshape(R, T, H) == ref) > 0.98
+                    else:
+                        assert np.array_equal(bits16(out).reshape(R, T, H), ref)
+    finally:
+        k.nixl_amd_ep_ll_set_tuning(1024, 1024)
