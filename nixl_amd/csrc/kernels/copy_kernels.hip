@@ -135,12 +135,13 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, i
 constexpr int kPieceLoads = 4;
 constexpr uint32_t kPieceUnits = kWaveSize * kPieceLoads; // 4 KiB
 
-template<bool NT, int LOADS>
-__global__ void __launch_bounds__(kWaveSize)
+template<bool NT, int LOADS, int WAVES>
+__global__ void __launch_bounds__(kWaveSize *WAVES)
 copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) {
-    const uint32_t lane = threadIdx.x;
-    const uint32_t p = blockIdx.x;
-    const PieceRec rec = recs[p]; // same address in every lane: a scalar load
+    const uint32_t lane = threadIdx.x & (kWaveSize - 1);
+    const uint32_t p = uniform(blockIdx.x * WAVES + threadIdx.x / kWaveSize);
+    if (p >= n_recs) return;
+    const PieceRec rec = recs[p]; // same address in every lane of the wave: a scalar load
     const uint64_t d = rec.dst + lane * 16u;
     const uint32_t units = rec.units; // >= 1
     // Loads are unconditional (a lane past the end re-reads the piece's last unit) so that
@@ -592,13 +593,16 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
         HIP_TRY(hipGetLastError());
     }
     if (plan->n_pieces) {
-        const dim3 grid(plan->n_pieces);
-        if (plan->nt)
-            hipLaunchKernelGGL((copy_piece_kernel<true, kPieceLoads>), grid, dim3(kWaveSize), 0, s, plan->piece_recs,
-                               plan->n_pieces);
-        else
-            hipLaunchKernelGGL((copy_piece_kernel<false, kPieceLoads>), grid, dim3(kWaveSize), 0, s, plan->piece_recs,
-                               plan->n_pieces);
+        const uint32_t w = static_cast<uint32_t>(plan->waves > 4 ? 4 : plan->waves);
+        const dim3 grid((plan->n_pieces + w - 1) / w), block(kWaveSize * w);
+#define NIXL_AMD_PIECE(NTV, WV) \
+    hipLaunchKernelGGL((copy_piece_kernel<NTV, kPieceLoads, WV>), grid, block, 0, s, plan->piece_recs, plan->n_pieces)
+        if (plan->nt) {
+            if (w == 1) NIXL_AMD_PIECE(true, 1); else if (w == 2) NIXL_AMD_PIECE(true, 2); else NIXL_AMD_PIECE(true, 4);
+        } else {
+            if (w == 1) NIXL_AMD_PIECE(false, 1); else if (w == 2) NIXL_AMD_PIECE(false, 2); else NIXL_AMD_PIECE(false, 4);
+        }
+#undef NIXL_AMD_PIECE
         HIP_TRY(hipGetLastError());
     }
     if (plan->mixed_wgs) {
