@@ -323,11 +323,8 @@ def main():
     if not args.no_small:
         line["kv"]["small_descriptor_stress"] = run_small_descriptors()
     if not args.no_ep:
-        try:
-            from nixl_amd import ep_bench
-            line["ep"] = ep_bench.run(args)
-        except ImportError:
-            line["ep"] = None
+        from nixl_amd import ep_bench
+        line["ep"] = ep_bench.run(args)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline()
         # the same path with the descriptor list split over the box's CPU share, reported beside
