@@ -369,8 +369,12 @@ ht_combine_kernel(uint16_t *__restrict__ combined,
 // (larger value wins, equal values go to the lower expert index).
 constexpr int kRouterMaxPerLane = 16; // E <= 1024
 
+// PL = experts a lane holds (a power of two >= ceil(E / 64)): the argmax rounds only walk
+// the slots that exist.
+template<int PL>
 __global__ void __launch_bounds__(256)
 router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, float *__restrict__ topk_w, int n_tokens, int E, int K) {
+    constexpr int kRouterMaxPerLane = PL; // shadows the global bound inside this kernel
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int token = blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
     if (token >= n_tokens) return;
@@ -592,8 +596,19 @@ nixl_amd_ep_router_topk(const float *logits,
     if (num_topk <= 0 || num_topk > 16 || num_topk > num_experts)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "router_topk: num_topk must be in [1, min(16, num_experts)]");
     if (num_tokens == 0) return NIXL_AMD_OK;
-    hipLaunchKernelGGL(router_kernel, dim3((num_tokens + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), logits,
-                       topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    const dim3 grid((num_tokens + 3) / 4), block(256);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int per_lane = (num_experts + kWaveSize - 1) / kWaveSize;
+    if (per_lane <= 1)
+        hipLaunchKernelGGL(router_kernel<1>, grid, block, 0, s, logits, topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    else if (per_lane <= 2)
+        hipLaunchKernelGGL(router_kernel<2>, grid, block, 0, s, logits, topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    else if (per_lane <= 4)
+        hipLaunchKernelGGL(router_kernel<4>, grid, block, 0, s, logits, topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    else if (per_lane <= 8)
+        hipLaunchKernelGGL(router_kernel<8>, grid, block, 0, s, logits, topk_idx, topk_weights, num_tokens, num_experts, num_topk);
+    else
+        hipLaunchKernelGGL(router_kernel<16>, grid, block, 0, s, logits, topk_idx, topk_weights, num_tokens, num_experts, num_topk);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }
