@@ -38,7 +38,8 @@
 
 namespace {
 
-constexpr int kLayoutThreads = 256;
+constexpr int kLayoutThreads = 1024; // one (token, k) per thread at 128 tokens x top-8
+constexpr int kScaleThreads = 256;
 constexpr int kLayoutLdsBytes = 32768;
 constexpr int kMaxTopk = 16; // reference limit, kernels/nixl_ep_ll.cu:412,421
 
@@ -243,7 +244,7 @@ struct ScalesArgs {
 constexpr int kScaleParts = 4; // workgroups per expert; 8 and 14 measured slower
 constexpr int kScaleBatch = 8;
 
-__global__ void __launch_bounds__(kLayoutThreads)
+__global__ void __launch_bounds__(kScaleThreads)
 ll_scales_kernel(ScalesArgs a) {
     extern __shared__ int seg_end[]; // [R] end of each source rank's segment of expert e
     const LlDims d = a.d;
@@ -253,7 +254,7 @@ ll_scales_kernel(ScalesArgs a) {
     if (!a.recv_scales && part != 0) return; // metadata only: one workgroup per expert is enough
     // the first row's source token is fetched before its validity is known (always in bounds)
     int t_next = a.src_info[static_cast<size_t>(e) * d.N + min(tid, d.N - 1)];
-    for (int r = tid; r < d.R; r += kLayoutThreads)
+    for (int r = tid; r < d.R; r += kScaleThreads)
         seg_end[r] = a.send_count[r * d.E + e];
     __syncthreads();
     if (tid < kWaveSize) {
@@ -285,9 +286,9 @@ ll_scales_kernel(ScalesArgs a) {
     __syncthreads();
     if (!a.recv_scales) return;
     const int n = seg_end[d.R - 1];
-    for (int slot = tid; slot < n; slot += kLayoutThreads) {
+    for (int slot = tid; slot < n; slot += kScaleThreads) {
         const int t = min(max(t_next, 0), d.T - 1); // written by the dispatch kernel; clamped so that a stale buffer cannot fault
-        if (slot + kLayoutThreads < n) t_next = a.src_info[static_cast<size_t>(e) * d.N + slot + kLayoutThreads];
+        if (slot + kScaleThreads < n) t_next = a.src_info[static_cast<size_t>(e) * d.N + slot + kScaleThreads];
         int lo = 0, hi = d.R - 1; // first rank whose segment ends beyond `slot`
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
@@ -623,7 +624,7 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
     sa.d = d;
     sa.use_ue8m0 = use_ue8m0;
     sa.parts = kScaleParts;
-    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * sa.parts), dim3(kLayoutThreads),
+    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * sa.parts), dim3(kScaleThreads),
                        static_cast<size_t>(d.R) * sizeof(int), s, sa);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
