@@ -84,6 +84,9 @@ using chrono_period_us_t = std::chrono::microseconds;
 inline constexpr uint16_t default_comm_port = 8888;
 
 #define NIXL_INIT_AGENT ""
+// Agent name of a placeholder entry in a remote memory-view list
+// (src/api/cpp/nixl_types.h:305, src/infra/nixl_descriptors.cpp:30).
+extern const std::string nixl_null_agent;
 
 namespace nixlEnumStrings {
 

@@ -80,6 +80,8 @@ typedef struct nixl_capi_xfer_telemetry_s *nixl_capi_xfer_telemetry_t;
 typedef struct nixl_capi_string_list_s *nixl_capi_string_list_t;
 typedef struct nixl_capi_mem_list_s *nixl_capi_mem_list_t;
 typedef struct nixl_capi_param_iter_s *nixl_capi_param_iter_t;
+typedef struct nixl_capi_remote_dlist_s *nixl_capi_remote_dlist_t;
+typedef struct nixl_capi_mem_view_s *nixl_capi_mem_view_t;
 
 /* agent */
 nixl_capi_status_t nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent);
@@ -240,6 +242,26 @@ nixl_capi_query_xfer_backend(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req_h
  * the calling thread makes this call again */
 nixl_capi_status_t
 nixl_capi_backend_get_type(nixl_capi_backend_t backend, const char **type);
+
+/* Memory views for kernels that move data themselves (reference wrapper.h:358-445).  The
+ * handle value is what device code receives as nixlMemViewH (nixl_amd_device.h): with the
+ * HIP backend a device pointer.  remote_agent NULL adds the placeholder entry that keeps
+ * the indices of later entries. */
+nixl_capi_status_t
+nixl_capi_prep_mem_view_local(nixl_capi_agent_t agent, nixl_capi_xfer_dlist_t descs, nixl_capi_mem_view_t *mvh,
+                              nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t
+nixl_capi_prep_mem_view_remote(nixl_capi_agent_t agent, nixl_capi_remote_dlist_t descs, nixl_capi_mem_view_t *mvh,
+                               nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t
+nixl_capi_create_remote_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_remote_dlist_t *dlist);
+nixl_capi_status_t
+nixl_capi_destroy_remote_dlist(nixl_capi_remote_dlist_t dlist);
+nixl_capi_status_t
+nixl_capi_remote_dlist_add_desc(nixl_capi_remote_dlist_t dlist, uintptr_t addr, size_t len, uint64_t dev_id,
+                                const char *remote_agent);
+nixl_capi_status_t
+nixl_capi_release_mem_view(nixl_capi_agent_t agent, nixl_capi_mem_view_t mvh);
 
 #ifdef __cplusplus
 }

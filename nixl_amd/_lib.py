@@ -192,6 +192,12 @@ _CAPI_SIGS = {
     "nixl_capi_estimate_xfer_cost": [c_void_p, c_void_p, c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int)],
     "nixl_capi_query_xfer_backend": [c_void_p, c_void_p, POINTER(c_void_p)],
     "nixl_capi_backend_get_type": [c_void_p, POINTER(c_char_p)],
+    "nixl_capi_prep_mem_view_local": [c_void_p, c_void_p, POINTER(c_void_p), c_void_p],
+    "nixl_capi_prep_mem_view_remote": [c_void_p, c_void_p, POINTER(c_void_p), c_void_p],
+    "nixl_capi_create_remote_dlist": [c_int, POINTER(c_void_p)],
+    "nixl_capi_destroy_remote_dlist": [c_void_p],
+    "nixl_capi_remote_dlist_add_desc": [c_void_p, c_size_t, c_size_t, c_uint64, c_char_p],
+    "nixl_capi_release_mem_view": [c_void_p, c_void_p],
     "nixl_capi_release_xfer_req": [c_void_p, c_void_p],
     "nixl_capi_destroy_xfer_req": [c_void_p],
 }

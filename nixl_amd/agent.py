@@ -153,6 +153,32 @@ class nixl_reg_dlist:
             self._h = None
 
 
+class nixl_remote_dlist:
+    """Owned nixl_remote_dlist_t: (addr, len, devId, agent name) entries; an agent name of
+    None is the placeholder that keeps later indices (reference: nixlRemoteDList,
+    src/bindings/python/nixl_bindings.cpp; wrapper.h:404-433)."""
+
+    def __init__(self, entries, mem):
+        self._lib = _lib.agent_lib()
+        self.mem = mem
+        self.entries = list(entries)
+        h = ctypes.c_void_p()
+        _check("create_remote_dlist", self._lib.nixl_capi_create_remote_dlist(mem, ctypes.byref(h)))
+        self._h = h
+        for a, l, d, name in self.entries:
+            _check("remote_dlist_add_desc",
+                   self._lib.nixl_capi_remote_dlist_add_desc(h, int(a), int(l), int(d),
+                                                             None if name is None else name.encode()))
+
+    def descCount(self):
+        return len(self.entries)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.nixl_capi_destroy_remote_dlist(self._h)
+            self._h = None
+
+
 class nixl_prepped_dlist_handle:
     """Reference: _api.py:49-86."""
 
@@ -332,6 +358,28 @@ class nixl_agent:
         finally:
             self._lib.nixl_capi_destroy_backend(b)
 
+    def prep_mem_view(self, dlist, *, backends=None):
+        """Reference: _api.py:728-759.  A local (nixl_xfer_dlist) or remote
+        (nixl_remote_dlist) list becomes a table that device code indexes; returns the handle
+        as an integer (with the HIP backend: the table's device address)."""
+        if isinstance(dlist, nixl_remote_dlist):
+            call, what = self._lib.nixl_capi_prep_mem_view_remote, "prep_mem_view(remote)"
+        elif isinstance(dlist, nixl_xfer_dlist):
+            call, what = self._lib.nixl_capi_prep_mem_view_local, "prep_mem_view(local)"
+        else:
+            raise TypeError("prep_mem_view takes a nixl_xfer_dlist or a nixl_remote_dlist")
+        o = self._opt_args(backends or ())
+        mvh = ctypes.c_void_p()
+        try:
+            _check(what, call(self._h, dlist._h, ctypes.byref(mvh), o))
+        finally:
+            self._free_opt(o)
+        return int(mvh.value)
+
+    def release_mem_view(self, mvh):
+        """Reference: _api.py:761-768."""
+        _check("release_mem_view", self._lib.nixl_capi_release_mem_view(self._h, ctypes.c_void_p(int(mvh))))
+
     def _opt_args(self, backends=(), skip_desc_merge=False, notif_msg=b""):
         if not backends and not skip_desc_merge and not notif_msg:
             return None
@@ -361,6 +409,15 @@ class nixl_agent:
         if tensors and not all(t.is_contiguous() for t in tensors):
             return None
         return nixl_xfer_dlist(_as_triples(descs), _guess_mem(descs, mem_type))
+
+    def get_remote_descs(self, descs, mem_type=None):
+        """Reference: _api.py:1082-1113: a list of (addr, len, devId, agent name) tuples with a
+        mandatory memory type, or a remote list passed along; anything else yields None."""
+        if isinstance(descs, nixl_remote_dlist):
+            return descs
+        if not descs or not isinstance(descs[0], tuple) or mem_type is None or len(descs[0]) != 4:
+            return None
+        return nixl_remote_dlist(descs, _MEM[mem_type])
 
     def get_reg_descs(self, descs, mem_type=None):
         """Reference: _api.py:1117-1230; same inputs as get_xfer_descs."""

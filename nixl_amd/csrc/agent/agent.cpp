@@ -175,6 +175,19 @@ nixlMemSection::populate(const nixl_xfer_dlist_t &query, nixlBackendEngine *back
     return NIXL_SUCCESS;
 }
 
+// reference: src/infra/nixl_memory_section.cpp:186-205
+nixl_status_t
+nixlMemSection::addElement(const nixlRemoteDesc &query,
+                           nixlBackendEngine *backend,
+                           nixl_remote_meta_dlist_t &resp) const {
+    const auto sec = sections.find({resp.getType(), backend});
+    if (sec == sections.end()) return NIXL_ERR_NOT_FOUND;
+    const int at = sec->second.coveringIndex(query);
+    if (at < 0) return NIXL_ERR_UNKNOWN;
+    resp.addDesc(nixlRemoteMetaDesc(query.addr, query.len, query.devId, sec->second[at].metadataP));
+    return NIXL_SUCCESS;
+}
+
 // reference: src/infra/nixl_memory_section.cpp:106-184
 nixl_status_t
 nixlMemSection::populate(const nixl_xfer_dlist_t &query,
@@ -239,7 +252,11 @@ nixlMemSection::populate(const nixl_xfer_dlist_t &query,
 // Agent
 // =====================================================================================
 
+const std::string nixl_null_agent = "NULL_AGENT";
+
 nixlAgentData::~nixlAgentData() {
+    for (const auto &[view, engine] : mvhToEngine)
+        engine->releaseMemView(view);
     // Deregister whatever the application left registered, then destroy engines through
     // the plugin that made them (reference: src/infra/nixl_memory_section.cpp:416-423).
     for (auto &[key, list] : localSection_.sections)
@@ -254,6 +271,18 @@ nixlAgentData::slotOf(const nixl_backend_t &type) const {
     for (const auto &s : engines_)
         if (s->engine->getType() == type) return s.get();
     return nullptr;
+}
+
+std::vector<nixlBackendEngine *>
+nixlAgentData::backendsFor(const nixl_opt_args_t *extra, const nixlMemSection &section, nixl_mem_t mem) const {
+    std::vector<nixlBackendEngine *> out;
+    if (extra && !extra->backends.empty()) {
+        for (const nixlBackendH *h : extra->backends)
+            out.push_back(h->engine);
+    } else if (const auto *avail = section.backendsFor(mem)) {
+        out.assign(avail->begin(), avail->end());
+    }
+    return out;
 }
 
 nixlAgent::nixlAgent(const std::string &name, const nixlAgentConfig &cfg)
@@ -926,18 +955,105 @@ nixlAgent::releasedDlistH(nixlDlistH *dlist_hndl) const {
 
 // ---- outside the transfer path -----------------------------------------------------------
 
+// reference: src/core/nixl_agent.cpp:1906-1976
 nixl_status_t
-nixlAgent::prepMemView(const nixl_remote_dlist_t &, nixlMemViewH &, const nixl_opt_args_t *) const {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgent::prepMemView(const nixl_remote_dlist_t &dlist,
+                       nixlMemViewH &mvh,
+                       const nixl_opt_args_t *extra_params) const {
+    mvh = nullptr;
+    const nixl_mem_t mem = dlist.getType();
+    nixl_remote_meta_dlist_t resolved(mem);
+    nixlBackendEngine *engine = nullptr;
+    nixl_opt_b_args_t opt;
+    if (extra_params) opt.customParam = extra_params->customParam;
+
+    std::shared_lock guard(data->lock);
+    for (const nixlRemoteDesc &desc : dlist) {
+        if (desc.remoteAgent == nixl_null_agent) {
+            resolved.addDesc(nixlRemoteMetaDesc(nixl_null_agent));
+            continue;
+        }
+        const auto it = data->remoteSections_.find(desc.remoteAgent);
+        if (it == data->remoteSections_.end()) {
+            NIXL_ERROR_FUNC << "metadata for remote agent '" << desc.remoteAgent << "' not found";
+            return NIXL_ERR_NOT_FOUND;
+        }
+        if (engine) {
+            // The first resolvable descriptor fixed the engine; the rest must resolve there.
+            const nixl_status_t st = it->second.addElement(desc, engine, resolved);
+            if (st != NIXL_SUCCESS) return st;
+            continue;
+        }
+        for (nixlBackendEngine *b : data->backendsFor(extra_params, it->second, mem)) {
+            if (it->second.addElement(desc, b, resolved) == NIXL_SUCCESS) {
+                engine = b;
+                break;
+            }
+        }
+        if (!engine) break;
+    }
+    if (!engine) {
+        NIXL_ERROR_FUNC << "no backend can build this list of remote memory descriptors";
+        return NIXL_ERR_NOT_FOUND;
+    }
+
+    const nixl_status_t st = engine->prepMemView(resolved, mvh, &opt);
+    if (st == NIXL_SUCCESS) {
+        std::lock_guard<std::mutex> views(data->mvhLock);
+        data->mvhToEngine.emplace(mvh, engine);
+    }
+    return st;
 }
 
+// reference: src/core/nixl_agent.cpp:1978-2018
 nixl_status_t
-nixlAgent::prepMemView(const nixl_local_dlist_t &, nixlMemViewH &, const nixl_opt_args_t *) const {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgent::prepMemView(const nixl_local_dlist_t &dlist,
+                       nixlMemViewH &mvh,
+                       const nixl_opt_args_t *extra_params) const {
+    mvh = nullptr;
+    const nixl_mem_t mem = dlist.getType();
+    nixl_meta_dlist_t resolved(mem);
+    nixlBackendEngine *engine = nullptr;
+    nixl_opt_b_args_t opt;
+    if (extra_params) opt.customParam = extra_params->customParam;
+
+    std::shared_lock guard(data->lock);
+    for (nixlBackendEngine *b : data->backendsFor(extra_params, data->localSection_, mem)) {
+        if (data->localSection_.populate(dlist, b, resolved) == NIXL_SUCCESS) {
+            engine = b;
+            break;
+        }
+    }
+    if (!engine) {
+        NIXL_ERROR_FUNC << "no backend can build this list of local memory descriptors";
+        return NIXL_ERR_NOT_FOUND;
+    }
+
+    const nixl_status_t st = engine->prepMemView(resolved, mvh, &opt);
+    if (st == NIXL_SUCCESS) {
+        std::lock_guard<std::mutex> views(data->mvhLock);
+        data->mvhToEngine.emplace(mvh, engine);
+    }
+    return st;
 }
 
+// reference: src/core/nixl_agent.cpp:2020-2036
 void
-nixlAgent::releaseMemView(nixlMemViewH) const {}
+nixlAgent::releaseMemView(nixlMemViewH mvh) const {
+    std::shared_lock guard(data->lock);
+    nixlBackendEngine *engine = nullptr;
+    {
+        std::lock_guard<std::mutex> views(data->mvhLock);
+        const auto it = data->mvhToEngine.find(mvh);
+        if (it == data->mvhToEngine.end()) {
+            NIXL_WARN << "invalid memory view handle: " << mvh;
+            return;
+        }
+        engine = it->second;
+        data->mvhToEngine.erase(it);
+    }
+    engine->releaseMemView(mvh);
+}
 
 nixl_status_t
 nixlAgent::getNotifs(nixl_notifs_t &, const nixl_opt_args_t *) {

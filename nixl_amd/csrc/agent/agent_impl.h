@@ -17,6 +17,7 @@
 #include <array>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <set>
 #include <shared_mutex>
 #include <string>
@@ -124,6 +125,9 @@ public:
     // Same, compressed into stride runs.
     nixl_status_t
     populate(const nixl_xfer_dlist_t &query, nixlBackendEngine *backend, nixl_stride_dlist_t &resp) const;
+    // Resolve one remote descriptor and append it (memory views).
+    nixl_status_t
+    addElement(const nixlRemoteDesc &query, nixlBackendEngine *backend, nixl_remote_meta_dlist_t &resp) const;
 
     std::map<nixl_section_key_t, nixlSecDescList> sections;
     std::array<std::set<nixlBackendEngine *>, FILE_SEG + 1> memToBackend;
@@ -194,8 +198,17 @@ public:
     // Only the agent itself can be a "remote" here (loopback).
     std::unordered_map<std::string, nixlMemSection> remoteSections_;
 
+    // Which engine made each live memory view (src/core/agent_data.h mvhToEngine).
+    std::unordered_map<nixlMemViewH, nixlBackendEngine *> mvhToEngine;
+    // Guards mvhToEngine alone, so that views can be made under the shared lock.
+    std::mutex mvhLock;
+
     engineSlot *
     slotOf(const nixl_backend_t &type) const;
+    // Candidate engines for a section and memory type: the caller's choice, else every
+    // engine that holds registrations of that type (src/core/nixl_agent.cpp getBackends).
+    std::vector<nixlBackendEngine *>
+    backendsFor(const nixl_opt_args_t *extra, const nixlMemSection &section, nixl_mem_t mem) const;
 };
 
 #endif

@@ -21,6 +21,9 @@ struct nixl_capi_opt_args_s {
 struct nixl_capi_xfer_dlist_s {
     nixl_xfer_dlist_t *dlist;
 };
+struct nixl_capi_remote_dlist_s {
+    nixl_remote_dlist_t *dlist;
+};
 struct nixl_capi_xfer_dlist_handle_s {
     nixlDlistH *handle;
 };
@@ -625,6 +628,68 @@ nixl_capi_backend_get_type(nixl_capi_backend_t backend, const char **type) {
     name = backend->backend->getType();
     *type = name.c_str();
     return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_prep_mem_view_local(nixl_capi_agent_t agent, nixl_capi_xfer_dlist_t descs, nixl_capi_mem_view_t *mvh,
+                              nixl_capi_opt_args_t opt_args) {
+    if (!agent || !descs || !mvh) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlMemViewH view = nullptr;
+        const nixl_status_t st = agent->inner->prepMemView(*descs->dlist, view, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *mvh = static_cast<nixl_capi_mem_view_t>(view);
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_prep_mem_view_remote(nixl_capi_agent_t agent, nixl_capi_remote_dlist_t descs, nixl_capi_mem_view_t *mvh,
+                               nixl_capi_opt_args_t opt_args) {
+    if (!agent || !descs || !mvh) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixlMemViewH view = nullptr;
+        const nixl_status_t st = agent->inner->prepMemView(*descs->dlist, view, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *mvh = static_cast<nixl_capi_mem_view_t>(view);
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_create_remote_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_remote_dlist_t *dlist) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        *dlist = new nixl_capi_remote_dlist_s{new nixl_remote_dlist_t(memOf(mem_type))};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_remote_dlist(nixl_capi_remote_dlist_t dlist) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete dlist->dlist;
+    delete dlist;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_remote_dlist_add_desc(nixl_capi_remote_dlist_t dlist, uintptr_t addr, size_t len, uint64_t dev_id,
+                                const char *remote_agent) {
+    if (!dlist) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        dlist->dlist->addDesc(nixlRemoteDesc(addr, len, dev_id, remote_agent ? remote_agent : nixl_null_agent));
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_release_mem_view(nixl_capi_agent_t agent, nixl_capi_mem_view_t mvh) {
+    if (!agent || !mvh) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        agent->inner->releaseMemView(static_cast<nixlMemViewH>(mvh));
+        return NIXL_CAPI_SUCCESS;
+    });
 }
 
 } // extern "C"

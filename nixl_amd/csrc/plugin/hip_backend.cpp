@@ -1,9 +1,11 @@
 #include "hip_backend.h"
 
 #include <cstdlib>
+#include <cstring>
 
 #include "backend/backend_plugin.h"
 #include "common/nixl_log.h"
+#include "nixl_amd_device.h"
 
 namespace {
 
@@ -73,6 +75,10 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
 
 nixlHipEngine::~nixlHipEngine() {
     reapRetired(true);
+    for (const auto &[table, device] : memViews_) {
+        (void)hipSetDevice(device);
+        (void)hipFree(table);
+    }
     for (size_t i = 0; i < streams_.size(); ++i) {
         if (!streams_[i]) continue;
         (void)hipSetDevice(static_cast<int>(i / streamsPerDevice_));
@@ -328,6 +334,109 @@ nixlHipEngine::estimateXferCost(const nixl_xfer_op_t &,
     err_margin = std::chrono::microseconds(static_cast<long>(us * 0.5));
     method = nixl_cost_t::ANALYTICAL_BACKEND;
     return NIXL_SUCCESS;
+}
+
+// ---- memory views --------------------------------------------------------------------
+
+nixl_status_t
+nixlHipEngine::buildMemView(const std::vector<viewEntry> &entries, uint32_t kind, nixlMemViewH &mvh) const {
+    mvh = nullptr;
+    if (entries.empty()) return NIXL_ERR_INVALID_PARAM;
+
+    std::vector<uint64_t> image(2 + 2 * entries.size());
+    nixl_amd_mem_view_t head{};
+    head.magic = NIXL_AMD_MEM_VIEW_MAGIC;
+    head.kind = kind;
+    head.count = entries.size();
+    static_assert(sizeof(head) == 2 * sizeof(uint64_t) && sizeof(nixl_amd_mem_view_entry_t) == 2 * sizeof(uint64_t));
+    std::memcpy(image.data(), &head, sizeof(head));
+
+    int device = -1;
+    for (size_t i = 0; i < entries.size(); ++i) {
+        const viewEntry &e = entries[i];
+        nixl_amd_mem_view_entry_t out{0, 0};
+        if (e.md) {
+            if (!e.md->contains(e.addr, e.len)) {
+                NIXL_ERROR << "HIP backend: memory view entry " << i << " is outside its registered region";
+                return NIXL_ERR_INVALID_PARAM;
+            }
+            // One table serves the kernels of one device; pinned host memory is reachable
+            // from any of them.
+            if (e.md->mem == VRAM_SEG) {
+                if (device < 0) device = e.md->device;
+                if (e.md->device != device) {
+                    NIXL_ERROR << "HIP backend: memory view spans devices " << device << " and "
+                               << e.md->device;
+                    return NIXL_ERR_NOT_SUPPORTED;
+                }
+            }
+            out.addr = e.addr;
+            out.len = e.len;
+        }
+        std::memcpy(&image[2 + 2 * i], &out, sizeof(out));
+    }
+    if (device < 0 && hipGetDevice(&device) != hipSuccess) return NIXL_ERR_BACKEND;
+
+    void *table = nullptr;
+    const size_t bytes = image.size() * sizeof(uint64_t);
+    if (!hipOk(hipSetDevice(device), "hipSetDevice") || !hipOk(hipMalloc(&table, bytes), "hipMalloc"))
+        return NIXL_ERR_BACKEND;
+    // Synchronous copy: the table is complete when the handle is handed out, whichever
+    // stream the application launches its kernels on.
+    if (!hipOk(hipMemcpy(table, image.data(), bytes, hipMemcpyHostToDevice), "hipMemcpy")) {
+        (void)hipFree(table);
+        return NIXL_ERR_BACKEND;
+    }
+    {
+        std::lock_guard<std::mutex> lock(memViewsMutex_);
+        memViews_.emplace(table, device);
+    }
+    mvh = table;
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::prepMemView(const nixl_meta_dlist_t &descs, nixlMemViewH &mvh, const nixl_opt_b_args_t *) const {
+    std::vector<viewEntry> entries;
+    entries.reserve(static_cast<size_t>(descs.descCount()));
+    for (const nixlMetaDesc &d : descs) {
+        const auto *md = static_cast<const nixlHipMD *>(d.metadataP);
+        if (!md) return NIXL_ERR_INVALID_PARAM;
+        entries.push_back({d.addr, d.len, md});
+    }
+    return buildMemView(entries, NIXL_AMD_MEM_VIEW_LOCAL, mvh);
+}
+
+nixl_status_t
+nixlHipEngine::prepMemView(const nixl_remote_meta_dlist_t &descs,
+                           nixlMemViewH &mvh,
+                           const nixl_opt_b_args_t *) const {
+    std::vector<viewEntry> entries;
+    entries.reserve(static_cast<size_t>(descs.descCount()));
+    for (const nixlRemoteMetaDesc &d : descs) {
+        // A descriptor without registration data is a placeholder that keeps the indices
+        // of the entries after it (the agent adds one for the null agent).
+        entries.push_back({d.addr, d.len, static_cast<const nixlHipMD *>(d.metadataP)});
+    }
+    return buildMemView(entries, NIXL_AMD_MEM_VIEW_REMOTE, mvh);
+}
+
+void
+nixlHipEngine::releaseMemView(nixlMemViewH mvh) const {
+    int device = 0;
+    {
+        std::lock_guard<std::mutex> lock(memViewsMutex_);
+        const auto it = memViews_.find(mvh);
+        if (it == memViews_.end()) {
+            NIXL_WARN << "HIP backend: unknown memory view handle " << mvh;
+            return;
+        }
+        device = it->second;
+        memViews_.erase(it);
+    }
+    // hipFree waits for the device, so a kernel still reading the table finishes first.
+    (void)hipSetDevice(device);
+    (void)hipFree(mvh);
 }
 
 // ---- plugin entry points -------------------------------------------------------------

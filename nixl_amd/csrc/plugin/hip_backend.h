@@ -13,6 +13,7 @@
 #include <atomic>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "backend/backend_engine.h"
@@ -121,6 +122,20 @@ public:
     nixl_status_t
     releaseReqH(nixlBackendReqH *handle) const override;
 
+    // Memory views for kernels that move data themselves: the handle is a device pointer
+    // to a table of {address, length} entries (layout in nixl_amd_device.h), checked here
+    // against the registrations (shape of src/plugins/ucx/ucx_backend.cpp prepMemView).
+    nixl_status_t
+    prepMemView(const nixl_remote_meta_dlist_t &descs,
+                nixlMemViewH &mvh,
+                const nixl_opt_b_args_t *opt_args = nullptr) const override;
+    nixl_status_t
+    prepMemView(const nixl_meta_dlist_t &descs,
+                nixlMemViewH &mvh,
+                const nixl_opt_b_args_t *opt_args = nullptr) const override;
+    void
+    releaseMemView(nixlMemViewH mvh) const override;
+
     nixl_status_t
     estimateXferCost(const nixl_xfer_op_t &operation,
                      const nixl_meta_dlist_t &local,
@@ -137,6 +152,13 @@ private:
     pickStream(int device) const;
     void
     reapRetired(bool wait) const;
+    struct viewEntry {
+        uintptr_t addr;
+        size_t len;
+        const nixlHipMD *md; // null for a placeholder entry
+    };
+    nixl_status_t
+    buildMemView(const std::vector<viewEntry> &entries, uint32_t kind, nixlMemViewH &mvh) const;
 
     int numDevices_ = 0;
     int streamsPerDevice_ = 1;
@@ -150,6 +172,9 @@ private:
     // Requests released while their kernel was still running; freed once it has finished.
     mutable std::vector<nixlHipReqH *> retired_;
     mutable std::mutex retiredMutex_;
+    // Live memory-view tables: device pointer -> owning device.
+    mutable std::unordered_map<void *, int> memViews_;
+    mutable std::mutex memViewsMutex_;
 };
 
 #endif

@@ -408,6 +408,65 @@ def test_raw_south_bound_api_from_cpp(cuda):
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
 
 
+def test_device_memory_view_calls_from_hip(cuda):
+    """Memory views and the device-side put / counter add / get-pointer calls over them,
+    driven from a HIP program through nixlAgent (tests/cpp/mem_view_device_api.hip; the
+    scenarios of the reference's test/gtest/device_api/single_write_test.cu plus ragged
+    spans against memcpy, ordering of a counter after puts, and refusals)."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "mem_view_device_api")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    env = dict(os.environ, NIXL_PLUGIN_DIR=_lib.PLUGIN_DIR)
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=120, env=env)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
+def test_memory_view_tables_from_python(cuda):
+    """prep_mem_view / release_mem_view of the Python API (reference _api.py:728-768): the
+    handle is the device address of a table {magic, kind, count, (addr, len)...}; a remote
+    list may carry a placeholder; lists that name unregistered memory or an unknown agent
+    are refused."""
+    import torch
+    from nixl_amd.agent import NixlError
+
+    class _DeviceWords:
+        def __init__(self, ptr, n):
+            self.__cuda_array_interface__ = {"shape": (n,), "typestr": "<i8", "data": (ptr, False), "version": 2}
+
+    a = nixl_agent("viewer", nixl_agent_config(backends=()))
+    a.create_backend("HIP")
+    x = torch.zeros(1 << 16, dtype=torch.uint8, device=cuda)
+    y = torch.zeros(1 << 14, dtype=torch.uint8, device=cuda)
+    a.register_memory([x, y])
+    local = a.get_xfer_descs([(x.data_ptr() + 256, 1024, 0), (y.data_ptr(), 1 << 14, 0)], "VRAM")
+    remote = a.get_remote_descs([(y.data_ptr() + 64, 128, 0, "viewer"), (0, 0, 0, None),
+                                 (x.data_ptr(), 1 << 16, 0, "viewer")], "VRAM")
+    assert a.get_remote_descs([(1, 2, 3)], "VRAM") is None and a.get_remote_descs([(1, 2, 3, "v")]) is None
+    lv = a.prep_mem_view(local)
+    rv = a.prep_mem_view(remote, backends=["HIP"])
+    assert lv and rv and lv != rv
+    magic = 0x5649584C
+    got = torch.as_tensor(_DeviceWords(lv, 2 + 2 * 2), device=cuda).cpu().tolist()
+    assert got == [magic | (0 << 32), 2, x.data_ptr() + 256, 1024, y.data_ptr(), 1 << 14]
+    got = torch.as_tensor(_DeviceWords(rv, 2 + 2 * 3), device=cuda).cpu().tolist()
+    assert got == [magic | (1 << 32), 3, y.data_ptr() + 64, 128, 0, 0, x.data_ptr(), 1 << 16]
+    a.release_mem_view(rv)
+    a.release_mem_view(lv)
+
+    z = torch.zeros(4096, dtype=torch.uint8, device=cuda)  # never registered
+    with pytest.raises(NixlError):
+        a.prep_mem_view(a.get_xfer_descs([(z.data_ptr(), 4096, 0)], "VRAM"))
+    with pytest.raises(NixlError):
+        a.prep_mem_view(a.get_xfer_descs([(y.data_ptr(), (1 << 14) + 1, 0)], "VRAM"))
+    with pytest.raises(NixlError):
+        a.prep_mem_view(a.get_remote_descs([(x.data_ptr(), 64, 0, "nobody")], "VRAM"))
+    with pytest.raises(TypeError):
+        a.prep_mem_view([(x.data_ptr(), 64, 0)])
+
+
 def test_requests_from_several_threads(cuda):
     """The reference calls prepXfer / postXfer / checkXfer / releaseReqH concurrently from
     several threads, one request each (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:
