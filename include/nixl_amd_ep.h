@@ -153,6 +153,13 @@ nixl_amd_ep_get_dispatch_layout(const int32_t *topk_idx,
  *   recv_row_offset          [R + 1] int64 or NULL (no reference counterpart): exclusive prefix
  *                            of the per-destination row totals, the form ht_dispatch and
  *                            ht_combine take; its last entry is the row count of recv_x
+ *   recv_counter             [R dst] int32 or NULL: rows each destination receives
+ *
+ * recv_counter and recv_expert_count are what the host needs to size the receive tensors; no
+ * later kernel reads them.  As the reference's moe_recv_counter_mapped and
+ * moe_recv_expert_counter_mapped (kernels/api.cuh:82,87; csrc/nixl_ep.cpp:762-800) they may
+ * point to pinned host memory: the host presets them to -1 and polls until every entry is
+ * non-negative, instead of copying them back.
  */
 int
 nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
@@ -162,6 +169,7 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
                                int *gbl_channel_prefix_matrix,
                                int *send_head,
                                int64_t *recv_row_offset,
+                               int *recv_counter,
                                int num_tokens,
                                int num_ranks,
                                int num_experts,

@@ -21,23 +21,24 @@ namespace {
 constexpr int kScanThreads = 1024;
 
 // Exclusive prefix of `v` over the workgroup (blockDim.x == kScanThreads); `total` gets the sum.
-__device__ __forceinline__ int
-block_exclusive_scan(int v, int *wave_sums, int &total) {
+template<typename V>
+__device__ __forceinline__ V
+block_exclusive_scan(V v, V *wave_sums, V &total) {
     const int lane = threadIdx.x & (kWaveSize - 1), wave = threadIdx.x / kWaveSize;
-    int incl = v;
+    V incl = v;
 #pragma unroll
     for (int off = 1; off < kWaveSize; off <<= 1) {
-        const int up = __shfl_up(incl, off);
+        const V up = __shfl_up(incl, off);
         if (lane >= off) incl += up;
     }
     __syncthreads(); // wave_sums may still be read from a previous call
     if (lane == kWaveSize - 1) wave_sums[wave] = incl;
     __syncthreads();
     constexpr int kWaves = kScanThreads / kWaveSize;
-    int before = 0, sum = 0;
+    V before = 0, sum = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-        const int s = wave_sums[w];
+        const V s = wave_sums[w];
         if (w < wave) before += s;
         sum += s;
     }
@@ -103,7 +104,7 @@ ht_scan_kernel(const uint8_t *__restrict__ in_rank,
     int pos = block_exclusive_scan(mine, wave_sums, total);
     for (int t = t0; t < t1; ++t) {
         const bool hit = in_rank[(static_cast<size_t>(src) * T + t) * R + d] != 0;
-        send_head[(static_cast<size_t>(src) * T + t) * R + d] = hit ? pos : -1;
+        __builtin_nontemporal_store(hit ? pos : -1, &send_head[(static_cast<size_t>(src) * T + t) * R + d]);
         pos += hit;
         // `pos` is now the number of hits in tokens [0, t]; a channel's inclusive prefix
         // is that number at the channel's last token.
@@ -118,6 +119,147 @@ ht_scan_kernel(const uint8_t *__restrict__ in_rank,
             channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = total;
 }
 
+// The same for up to 8 ranks and fewer than 65 536 tokens, which is every shipping
+// configuration.  A workgroup owns one chunk of kScanThreads tokens of one source rank, one
+// token per thread, and handles all destinations at once with four 16-bit counters to a
+// 64-bit word: it first counts the hits of the chunks before its own (a reduction; chunks do
+// not wait for each other), then scans its own.  A thread writes the R positions of its
+// token as one run, a wave consecutive runs.  The positions are stored non-temporally: the
+// row kernel that follows reads them from every XCD, and lines left dirty in the writer's L2
+// made those reads slow (+45 us on 8 x 4096 tokens).  grid = R * ceil(T / kScanThreads).
+constexpr int kPackedScanRanks = 8;
+constexpr int kPackedScanMaxTokens = 65535;
+
+struct PackedCounts {
+    unsigned long long lo, hi; // destinations 0..3 and 4..7, 16 bits each
+};
+
+__device__ __forceinline__ int
+packed_field(const PackedCounts &c, int d) {
+    return static_cast<int>(((d < 4 ? c.lo : c.hi) >> (16 * (d & 3))) & 0xffffu);
+}
+
+__device__ __forceinline__ PackedCounts
+packed_hits(const uint8_t *flags, int t, int R) {
+    PackedCounts hit{0, 0};
+    if (R == 8) {
+        const unsigned long long f = *reinterpret_cast<const unsigned long long *>(flags + static_cast<size_t>(t) * 8);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            hit.lo |= static_cast<unsigned long long>(((f >> (8 * d)) & 0xffu) != 0) << (16 * d);
+            hit.hi |= static_cast<unsigned long long>(((f >> (8 * (d + 4))) & 0xffu) != 0) << (16 * d);
+        }
+    } else {
+        for (int d = 0; d < R; ++d) {
+            const unsigned long long bit = flags[static_cast<size_t>(t) * R + d] != 0;
+            if (d < 4)
+                hit.lo |= bit << (16 * d);
+            else
+                hit.hi |= bit << (16 * (d - 4));
+        }
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kScanThreads)
+ht_scan_packed_kernel(const uint8_t *__restrict__ in_rank,
+                      int *__restrict__ send_head,
+                      int *__restrict__ channel_prefix,
+                      int T,
+                      int R,
+                      int C) {
+    constexpr int kWaves = kScanThreads / kWaveSize;
+    __shared__ PackedCounts wave_sums[kWaves], wave_before[kWaves];
+    const int chunks = (T + kScanThreads - 1) / kScanThreads;
+    const int src = blockIdx.x / chunks, base = (blockIdx.x % chunks) * kScanThreads;
+    const int tid = threadIdx.x, lane = tid & (kWaveSize - 1), wave = tid / kWaveSize;
+    const int per_channel = (T + C - 1) / C;
+    const uint8_t *flags = in_rank + static_cast<size_t>(src) * T * R;
+    const int t = base + tid;
+
+    // own token first, so that its load overlaps the count of the earlier chunks
+    PackedCounts hit{0, 0};
+    if (t < T) hit = packed_hits(flags, t, R);
+    PackedCounts earlier{0, 0};
+    for (int u = tid; u < base; u += kScanThreads) {
+        const PackedCounts h = packed_hits(flags, u, R);
+        earlier.lo += h.lo;
+        earlier.hi += h.hi;
+    }
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+        earlier.lo += __shfl_xor(earlier.lo, off);
+        earlier.hi += __shfl_xor(earlier.hi, off);
+    }
+    PackedCounts incl = hit; // inclusive scan inside the wave
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+        const unsigned long long ulo = __shfl_up(incl.lo, off), uhi = __shfl_up(incl.hi, off);
+        if (lane >= off) {
+            incl.lo += ulo;
+            incl.hi += uhi;
+        }
+    }
+    if (lane == kWaveSize - 1) wave_sums[wave] = incl;
+    if (lane == 0) wave_before[wave] = earlier;
+    __syncthreads();
+    // second level by the first wave: wave_sums[w] becomes the hits before wave w (earlier
+    // chunks included), wave_before[0] the grand total up to the end of this chunk
+    if (wave == 0) {
+        PackedCounts s{0, 0}, e{0, 0};
+        if (lane < kWaves) {
+            s = wave_sums[lane];
+            e = wave_before[lane];
+        }
+        PackedCounts run = s;
+#pragma unroll
+        for (int off = 1; off < kWaves; off <<= 1) {
+            const unsigned long long ulo = __shfl_up(run.lo, off), uhi = __shfl_up(run.hi, off);
+            if (lane >= off) {
+                run.lo += ulo;
+                run.hi += uhi;
+            }
+        }
+#pragma unroll
+        for (int off = kWaves / 2; off > 0; off >>= 1) {
+            e.lo += __shfl_xor(e.lo, off);
+            e.hi += __shfl_xor(e.hi, off);
+        }
+        if (lane < kWaves) wave_sums[lane] = PackedCounts{run.lo - s.lo + e.lo, run.hi - s.hi + e.hi};
+        if (lane == kWaves - 1) wave_before[0] = PackedCounts{run.lo + e.lo, run.hi + e.hi};
+    }
+    __syncthreads();
+    const PackedCounts before = wave_sums[wave], total = wave_before[0];
+    incl.lo += before.lo; // hits in tokens [0, t]
+    incl.hi += before.hi;
+    if (t < T) {
+        int out[kPackedScanRanks];
+#pragma unroll
+        for (int d = 0; d < kPackedScanRanks; ++d)
+            out[d] = packed_field(hit, d) ? packed_field(incl, d) - 1 : -1;
+        int *dst = send_head + (static_cast<size_t>(src) * T + t) * R;
+        if (R == 8) {
+            st16_nt(dst, make_uint4(out[0], out[1], out[2], out[3]));
+            st16_nt(dst + 4, make_uint4(out[4], out[5], out[6], out[7]));
+        } else {
+#pragma unroll
+            for (int d = 0; d < kPackedScanRanks; ++d)
+                if (d < R) __builtin_nontemporal_store(out[d], dst + d);
+        }
+        if ((t + 1) % per_channel == 0 || t + 1 == T) {
+            const int c = t / per_channel;
+            for (int d = 0; d < R; ++d)
+                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = packed_field(incl, d);
+        }
+    }
+    // channels that start at or beyond T are empty: they repeat the grand total, which the
+    // workgroup of the last chunk knows
+    if (tid == 0 && base + kScanThreads >= T)
+        for (int c = (T + per_channel - 1) / per_channel; c < C; ++c)
+            for (int d = 0; d < R; ++d)
+                channel_prefix[(static_cast<size_t>(src) * R + d) * C + c] = packed_field(total, d);
+}
+
 // ---- notify, part 2: receive-side prefix over source ranks, aligned per-expert counts
 // (kernels/nixl_ep_ht.cu:295-314) and where each destination's rows start in the
 // concatenated outputs.  One workgroup. ------------------------------------------------------
@@ -127,6 +269,7 @@ ht_prefix_kernel(const int *__restrict__ channel_prefix,
                  int *__restrict__ recv_rank_prefix,
                  int *__restrict__ recv_expert_count,
                  long long *__restrict__ row_offset,
+                 int *__restrict__ recv_counter,
                  int R,
                  int E,
                  int C,
@@ -146,6 +289,7 @@ ht_prefix_kernel(const int *__restrict__ channel_prefix,
             total += channel_prefix[(static_cast<size_t>(r) * R + tid) * C + (C - 1)];
             recv_rank_prefix[tid * R + r] = total;
         }
+        if (recv_counter) recv_counter[tid] = total;
     }
     if (row_offset) {
         // exclusive prefix of the per-destination totals in 64 bits
@@ -479,6 +623,7 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
                                int *gbl_channel_prefix_matrix,
                                int *send_head,
                                int64_t *recv_row_offset,
+                               int *recv_counter,
                                int num_tokens,
                                int num_ranks,
                                int num_experts,
@@ -493,13 +638,21 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
         !gbl_channel_prefix_matrix || !send_head)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_notify_dispatch: null pointer argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(ht_scan_kernel, dim3(static_cast<unsigned>(num_ranks) * num_ranks), dim3(kScanThreads), 0, s, is_token_in_rank, send_head,
-                       gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
+    // the packed kernel reads 8 flag bytes and writes 16-byte pieces at a time
+    const bool aligned = reinterpret_cast<uintptr_t>(is_token_in_rank) % 8 == 0 && reinterpret_cast<uintptr_t>(send_head) % 16 == 0;
+    if (num_ranks <= kPackedScanRanks && num_tokens <= kPackedScanMaxTokens && aligned)
+        hipLaunchKernelGGL(ht_scan_packed_kernel,
+                           dim3(static_cast<unsigned>(num_ranks) * ((num_tokens + kScanThreads - 1) / kScanThreads)),
+                           dim3(kScanThreads), 0, s,
+                           is_token_in_rank, send_head, gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
+    else
+        hipLaunchKernelGGL(ht_scan_kernel, dim3(static_cast<unsigned>(num_ranks) * num_ranks), dim3(kScanThreads), 0, s,
+                           is_token_in_rank, send_head, gbl_channel_prefix_matrix, num_tokens, num_ranks, num_channels);
     HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(ht_prefix_kernel, dim3(1), dim3(kScanThreads), 0, s, gbl_channel_prefix_matrix,
                        num_tokens_per_expert, recv_gbl_rank_prefix_sum, recv_expert_count,
-                       reinterpret_cast<long long *>(recv_row_offset), num_ranks, num_experts, num_channels,
-                       expert_alignment);
+                       reinterpret_cast<long long *>(recv_row_offset), recv_counter, num_ranks, num_experts,
+                       num_channels, expert_alignment);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
 }

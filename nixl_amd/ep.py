@@ -12,7 +12,9 @@ only owns the memory and the stream; all work is done by the HIP kernels behind
 include/nixl_amd_ep.h, and nothing here falls back to torch ops.
 """
 import ctypes
+import time
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -77,6 +79,10 @@ class Buffer:
         self.mask_buffer = torch.zeros((self.num_ranks, self.num_ranks), dtype=torch.int32, device=self.device)
         self._mask_active = False
         self._workspace = None
+        # Normal-mode dispatch sizes its receive tensors for the worst case, and so avoids
+        # waiting for the counts before it launches, while that takes no more than this.
+        self.ht_recv_worst_case_limit = 16 << 30
+        self.cpu_timeout_secs = 100  # NUM_CPU_TIMEOUT_SECS, csrc/kernels/configs.cuh
 
     # -- life cycle and sizing helpers kept for callers written against the reference ------
     def destroy(self):
@@ -180,12 +186,21 @@ class Buffer:
     def _mask_ptr(self):
         return _ptr(self.mask_buffer) if self._mask_active else None
 
-    def _host_counts(self, n):
-        """Pinned host buffers for the counts normal-mode dispatch reads back."""
-        if getattr(self, "_pinned_counts", None) is None or self._pinned_counts[1].numel() != n:
-            self._pinned_counts = (torch.empty(1, dtype=torch.int64, pin_memory=True),
-                                   torch.empty(n, dtype=torch.int32, pin_memory=True))
-        return self._pinned_counts
+    def _mapped_counts(self, n):
+        """Pinned host words that the count kernel writes and the host polls, as a numpy view."""
+        if getattr(self, "_mapped_tensor", None) is None or self._mapped_tensor.numel() != n:
+            self._mapped_tensor = torch.empty(n, dtype=torch.int32, pin_memory=True)
+            self._mapped_view = self._mapped_tensor.numpy()
+        return self._mapped_view
+
+    def _wait_counts(self, mapped, num_ranks):
+        """Polls until the GPU has written every count (reference: csrc/nixl_ep.cpp:779-797,
+        same time-out); returns the total number of rows."""
+        deadline = time.monotonic() + self.cpu_timeout_secs
+        while int(mapped.min()) < 0:
+            if time.monotonic() > deadline:
+                raise EPError("timeout (dispatch CPU): the receive counts never arrived")
+        return int(mapped[:num_ranks].sum(dtype=np.int64))
 
     def _get_workspace(self, nbytes):
         if self._workspace is None or self._workspace.numel() < nbytes:
@@ -350,31 +365,40 @@ class Buffer:
         E = num_tokens_per_expert.shape[1]
         El = E // R
         prefix = torch.empty((R, R), dtype=torch.int32, device=dev)
-        expert_count = torch.empty((R, El), dtype=torch.int32, device=dev)
         chan = torch.empty((R, R, num_channels), dtype=torch.int32, device=dev)
         send_head = torch.empty((R, T, R), dtype=torch.int32, device=dev)
         row_offset = torch.empty(R + 1, dtype=torch.int64, device=dev)
+        # The counts the host needs go straight to pinned host memory, preset to -1 and polled
+        # below, as in the reference (csrc/nixl_ep.cpp:762-800).
+        mapped = self._mapped_counts(R + R * El)
+        mapped.fill(-1)
+        recv_counter_ptr = ctypes.c_void_p(self._mapped_tensor.data_ptr())
+        expert_count_ptr = ctypes.c_void_p(self._mapped_tensor.data_ptr() + 4 * R)
         _check(self._k.nixl_amd_ep_ht_notify_dispatch(_ptr(is_token_in_rank), _ptr(num_tokens_per_expert), _ptr(prefix),
-                                                      _ptr(expert_count), _ptr(chan), _ptr(send_head), _ptr(row_offset),
-                                                      T, R, E, num_channels, expert_alignment, _stream()),
-               "ht_notify_dispatch")
-        # The reference blocks here too, until the GPU has published the receive counts
-        # through host-mapped memory (csrc/nixl_ep.cpp:762-800), to size recv_x.  One
-        # synchronisation brings both the row total and the per-expert counts to the host.
-        host_total, host_counts = self._host_counts(R * El)
-        host_total.copy_(row_offset[-1:], non_blocking=True)
-        host_counts.copy_(expert_count.view(-1), non_blocking=True)
-        torch.cuda.current_stream(dev).synchronize()
-        total = int(host_total[0])
-        expert_count_list = host_counts.view(R, El).tolist()
-        recv_x = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
-        recv_topk_idx = torch.empty((total, K), dtype=torch.int32, device=dev)
-        recv_topk_weights = torch.empty((total, K), dtype=torch.float32, device=dev)
-        recv_src_meta = torch.empty((total, 2), dtype=torch.int32, device=dev)
+                                                      expert_count_ptr, _ptr(chan), _ptr(send_head), _ptr(row_offset),
+                                                      recv_counter_ptr, T, R, E, num_channels, expert_alignment,
+                                                      _stream()), "ht_notify_dispatch")
+        # The reference waits here, because it sizes recv_x from the counts.  With 288 GB of
+        # HBM the receive side can be sized for the worst case instead (every set entry of
+        # is_token_in_rank is one row, so R*T*R rows bound the total): the row kernels are
+        # queued right behind the count kernels, the GPU never idles through the host round
+        # trip, and the host only waits for the counts to cut the views.
+        capacity = R * T * R
+        ahead = capacity * (H * 2 + K * 8 + 8) <= self.ht_recv_worst_case_limit
+        rows = capacity if ahead else self._wait_counts(mapped, R)
+        recv_x = torch.empty((rows, H), dtype=torch.bfloat16, device=dev)
+        recv_topk_idx = torch.empty((rows, K), dtype=torch.int32, device=dev)
+        recv_topk_weights = torch.empty((rows, K), dtype=torch.float32, device=dev)
+        recv_src_meta = torch.empty((rows, 2), dtype=torch.int32, device=dev)
         _check(self._k.nixl_amd_ep_ht_dispatch(_ptr(recv_x), _ptr(recv_topk_idx), _ptr(recv_topk_weights),
                                                _ptr(recv_src_meta), _ptr(x), _ptr(topk_idx), _ptr(topk_weights),
                                                _ptr(is_token_in_rank), _ptr(prefix), _ptr(send_head), _ptr(row_offset),
                                                T, H, K, R, E, _stream()), "ht_dispatch")
+        if ahead:
+            total = self._wait_counts(mapped, R)
+            recv_x, recv_topk_idx = recv_x[:total], recv_topk_idx[:total]
+            recv_topk_weights, recv_src_meta = recv_topk_weights[:total], recv_src_meta[:total]
+        expert_count_list = mapped[R:].reshape(R, El).tolist()
         out_handle = (is_token_in_rank, prefix, chan, recv_src_meta, send_head, row_offset)
         return recv_x, recv_topk_idx, recv_topk_weights, expert_count_list, out_handle, EventOverlap(None)
 

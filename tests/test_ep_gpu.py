@@ -392,7 +392,9 @@ def zipf_topk(rng, R, T, K, E, s=1.2):
     return topk, (w / w.sum(2, keepdims=True)).astype(np.float32)
 
 
-@pytest.mark.parametrize("shape", [(4, 37, 256, 4, 16, 5, 8), (8, 300, 1024, 8, 64, 10, 1), (2, 1500, 512, 2, 4, 3, 4)])
+# 16 ranks take the per-pair scan kernel, up to 8 the packed one (2500 tokens: three chunks)
+@pytest.mark.parametrize("shape", [(4, 37, 256, 4, 16, 5, 8), (8, 300, 1024, 8, 64, 10, 1), (2, 1500, 512, 2, 4, 3, 4),
+                                   (16, 50, 256, 4, 32, 3, 1), (8, 2500, 128, 3, 16, 7, 2), (5, 1030, 128, 2, 10, 4, 1)])
 def test_ht_pipeline_matches_oracle(cuda, shape):
     R, T, H, K, E, C, align = shape
     x, topk, w = make_world(3 * R, R, T, H, K, E)
@@ -439,6 +441,27 @@ def test_ht_pipeline_matches_oracle(cuda, shape):
                                      o["row_offset"], ob0, ob1)
         assert np.array_equal(bits16(comb).reshape(R, T, H), want)
         assert np.array_equal(comb_w.cpu().numpy(), want_w)
+
+
+def test_ht_dispatch_sized_ahead_equals_sized_exactly(cuda):
+    """Normal-mode dispatch either sizes its receive tensors for the worst case and launches
+    before the counts reach the host, or (past a byte limit) waits for the counts as the
+    reference does (csrc/nixl_ep.cpp:762-800).  Both give the same tensors."""
+    R, T, H, K, E, C = 4, 211, 512, 3, 16, 4
+    x, topk, w = make_world(77, R, T, H, K, E)
+    xd, td, wd = x.to(cuda), torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    outs = []
+    for limit in (16 << 30, 0):
+        buf = Buffer(R, low_latency_mode=False, device=cuda)
+        buf.ht_recv_worst_case_limit = limit
+        per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(td, E)
+        outs.append(buf.ht_dispatch(xd, num_tokens_per_rank=per_rank, is_token_in_rank=in_rank,
+                                    num_tokens_per_expert=per_expert, topk_idx=td, topk_weights=wd, num_channels=C))
+    torch.cuda.synchronize()
+    (ax, ai, aw, al, ah, _), (bx, bi, bw, bl, bh, _) = outs
+    assert ax.shape == bx.shape and ax.shape[0] == int(ah[5][-1]) and ax.is_contiguous()
+    assert torch.equal(ax.view(torch.int16), bx.view(torch.int16)) and torch.equal(ai, bi) and torch.equal(aw, bw)
+    assert al == bl and torch.equal(ah[3], bh[3]) and torch.equal(ah[5], bh[5])
 
 
 def test_config5_full_size_properties(cuda):
