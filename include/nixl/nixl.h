@@ -93,7 +93,7 @@ public:
     nixl_status_t
     releasedDlistH(nixlDlistH *dlist_hndl) const;
 
-    // Control-plane members outside the transfer path: always NIXL_ERR_NOT_SUPPORTED.
+    // Memory views for kernels that move data themselves.
     nixl_status_t
     prepMemView(const nixl_remote_dlist_t &dlist,
                 nixlMemViewH &mvh,
@@ -110,12 +110,22 @@ public:
     genNotif(const std::string &remote_agent,
              const nixl_blob_t &msg,
              const nixl_opt_args_t *extra_params = nullptr) const;
+    // Metadata exchange by hand: the blob of one agent, in the reference's wire format,
+    // is given to another agent by whatever means the application has.  The side channels
+    // of the reference (sockets, ETCD: sendLocalMD, fetchRemoteMD, invalidateLocalMD) are not
+    // offered.
     nixl_status_t
     getLocalMD(nixl_blob_t &str) const;
+    nixl_status_t
+    getLocalPartialMD(const nixl_reg_dlist_t &descs,
+                      nixl_blob_t &str,
+                      const nixl_opt_args_t *extra_params = nullptr) const;
     nixl_status_t
     loadRemoteMD(const nixl_blob_t &remote_metadata, std::string &agent_name);
     nixl_status_t
     invalidateRemoteMD(const std::string &remote_agent);
+    nixl_status_t
+    checkRemoteMD(const std::string remote_name, const nixl_xfer_dlist_t &descs) const;
 };
 
 #endif // NIXL_AMD_AGENT_API_H

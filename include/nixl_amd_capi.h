@@ -82,6 +82,7 @@ typedef struct nixl_capi_mem_list_s *nixl_capi_mem_list_t;
 typedef struct nixl_capi_param_iter_s *nixl_capi_param_iter_t;
 typedef struct nixl_capi_remote_dlist_s *nixl_capi_remote_dlist_t;
 typedef struct nixl_capi_mem_view_s *nixl_capi_mem_view_t;
+typedef struct nixl_capi_notif_map_s *nixl_capi_notif_map_t;
 
 /* agent */
 nixl_capi_status_t nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent);
@@ -107,6 +108,8 @@ nixl_capi_status_t nixl_capi_opt_args_add_backend(nixl_capi_opt_args_t args, nix
 nixl_capi_status_t nixl_capi_opt_args_set_notif_msg(nixl_capi_opt_args_t args, const void *data, size_t len);
 nixl_capi_status_t nixl_capi_opt_args_set_has_notif(nixl_capi_opt_args_t args, bool has_notif);
 nixl_capi_status_t nixl_capi_opt_args_set_skip_desc_merge(nixl_capi_opt_args_t args, bool skip_merge);
+/* extension: nixl_opt_args_t::includeConnInfo, read by get_local_partial_md */
+nixl_capi_status_t nixl_capi_opt_args_set_include_conn_info(nixl_capi_opt_args_t args, bool include);
 
 /* descriptor lists */
 nixl_capi_status_t nixl_capi_create_xfer_dlist(nixl_capi_mem_type_t mem_type, nixl_capi_xfer_dlist_t *dlist);
@@ -262,6 +265,48 @@ nixl_capi_remote_dlist_add_desc(nixl_capi_remote_dlist_t dlist, uintptr_t addr, 
                                 const char *remote_agent);
 nixl_capi_status_t
 nixl_capi_release_mem_view(nixl_capi_agent_t agent, nixl_capi_mem_view_t mvh);
+
+/* Metadata exchange by hand and notifications between agents (reference wrapper.h:131-151,
+ * 228, 254-263, 327-332).  get_local_md / get_local_partial_md return a malloc'ed copy of
+ * the blob, which the caller releases with free() (or nixl_capi_free_buffer); load_remote_md
+ * returns the peer's name the same way.  The blob is in the reference's wire format. */
+nixl_capi_status_t
+nixl_capi_get_local_md(nixl_capi_agent_t agent, void **data, size_t *len);
+nixl_capi_status_t
+nixl_capi_get_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, void **data, size_t *len,
+                               nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t
+nixl_capi_load_remote_md(nixl_capi_agent_t agent, const void *data, size_t len, char **agent_name);
+nixl_capi_status_t
+nixl_capi_invalidate_remote_md(nixl_capi_agent_t agent, const char *remote_agent);
+nixl_capi_status_t
+nixl_capi_check_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_xfer_dlist_t descs);
+nixl_capi_status_t
+nixl_capi_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args);
+/* extension: releases a buffer handed out by the calls above */
+nixl_capi_status_t
+nixl_capi_free_buffer(void *data);
+
+nixl_capi_status_t
+nixl_capi_create_notif_map(nixl_capi_notif_map_t *notif_map);
+nixl_capi_status_t
+nixl_capi_destroy_notif_map(nixl_capi_notif_map_t notif_map);
+nixl_capi_status_t
+nixl_capi_get_notifs(nixl_capi_agent_t agent, nixl_capi_notif_map_t notif_map, nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t
+nixl_capi_gen_notif(nixl_capi_agent_t agent, const char *remote_agent, const void *data, size_t len,
+                    nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t
+nixl_capi_notif_map_size(nixl_capi_notif_map_t map, size_t *size);
+nixl_capi_status_t
+nixl_capi_notif_map_get_agent_at(nixl_capi_notif_map_t map, size_t index, const char **agent_name);
+nixl_capi_status_t
+nixl_capi_notif_map_get_notifs_size(nixl_capi_notif_map_t map, const char *agent_name, size_t *size);
+nixl_capi_status_t
+nixl_capi_notif_map_get_notif(nixl_capi_notif_map_t map, const char *agent_name, size_t index, const void **data,
+                              size_t *len);
+nixl_capi_status_t
+nixl_capi_notif_map_clear(nixl_capi_notif_map_t map);
 
 #ifdef __cplusplus
 }

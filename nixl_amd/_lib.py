@@ -198,6 +198,23 @@ _CAPI_SIGS = {
     "nixl_capi_destroy_remote_dlist": [c_void_p],
     "nixl_capi_remote_dlist_add_desc": [c_void_p, c_size_t, c_size_t, c_uint64, c_char_p],
     "nixl_capi_release_mem_view": [c_void_p, c_void_p],
+    "nixl_capi_opt_args_set_include_conn_info": [c_void_p, c_bool],
+    "nixl_capi_get_local_md": [c_void_p, POINTER(c_void_p), POINTER(c_size_t)],
+    "nixl_capi_get_local_partial_md": [c_void_p, c_void_p, POINTER(c_void_p), POINTER(c_size_t), c_void_p],
+    "nixl_capi_load_remote_md": [c_void_p, c_char_p, c_size_t, POINTER(c_void_p)],
+    "nixl_capi_invalidate_remote_md": [c_void_p, c_char_p],
+    "nixl_capi_check_remote_md": [c_void_p, c_char_p, c_void_p],
+    "nixl_capi_make_connection": [c_void_p, c_char_p, c_void_p],
+    "nixl_capi_free_buffer": [c_void_p],
+    "nixl_capi_create_notif_map": [POINTER(c_void_p)],
+    "nixl_capi_destroy_notif_map": [c_void_p],
+    "nixl_capi_get_notifs": [c_void_p, c_void_p, c_void_p],
+    "nixl_capi_gen_notif": [c_void_p, c_char_p, c_char_p, c_size_t, c_void_p],
+    "nixl_capi_notif_map_size": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_notif_map_get_agent_at": [c_void_p, c_size_t, POINTER(c_char_p)],
+    "nixl_capi_notif_map_get_notifs_size": [c_void_p, c_char_p, POINTER(c_size_t)],
+    "nixl_capi_notif_map_get_notif": [c_void_p, c_char_p, c_size_t, POINTER(c_void_p), POINTER(c_size_t)],
+    "nixl_capi_notif_map_clear": [c_void_p],
     "nixl_capi_release_xfer_req": [c_void_p, c_void_p],
     "nixl_capi_destroy_xfer_req": [c_void_p],
 }

@@ -238,6 +238,7 @@ class nixl_agent:
         _check("create_agent", self._lib.nixl_capi_create_configured_agent(agent_name.encode(), ctypes.byref(cfg), ctypes.byref(h)))
         self._h = h
         self.backends = {}
+        self.notifs = {}  # what update_notifs / check_remote_xfer_done have not handed out yet
         self.nixl_ops = {"WRITE": 1, "READ": 0}
         for b in conf.backends:
             self.create_backend(b)
@@ -358,6 +359,107 @@ class nixl_agent:
         finally:
             self._lib.nixl_capi_destroy_backend(b)
 
+    # -- metadata and notifications between agents ------------------------------------------
+    def _take_buffer(self, data, size):
+        try:
+            return ctypes.string_at(data, size.value)
+        finally:
+            self._lib.nixl_capi_free_buffer(data)
+
+    def get_agent_metadata(self):
+        """Reference: _api.py:856-862.  The agent's metadata blob, in the reference's wire
+        format; hand it to another agent's add_remote_agent by any means."""
+        data, size = ctypes.c_void_p(), ctypes.c_size_t()
+        _check("get_agent_metadata", self._lib.nixl_capi_get_local_md(self._h, ctypes.byref(data), ctypes.byref(size)))
+        return self._take_buffer(data, size)
+
+    def get_partial_agent_metadata(self, descs, inc_conn_info=False, backends=()):
+        """Reference: _api.py:864-884.  Metadata of the listed registrations only (an empty
+        list: connection info only)."""
+        o = self._opt_args(backends, include_conn_info=inc_conn_info)
+        data, size = ctypes.c_void_p(), ctypes.c_size_t()
+        try:
+            _check("get_partial_agent_metadata",
+                   self._lib.nixl_capi_get_local_partial_md(self._h, descs._h, ctypes.byref(data), ctypes.byref(size), o))
+        finally:
+            self._free_opt(o)
+        return self._take_buffer(data, size)
+
+    def add_remote_agent(self, metadata):
+        """Reference: _api.py:886-897.  Returns the peer's name."""
+        name = ctypes.c_void_p()
+        _check("add_remote_agent", self._lib.nixl_capi_load_remote_md(self._h, bytes(metadata), len(metadata), ctypes.byref(name)))
+        try:
+            return ctypes.string_at(name).decode()
+        finally:
+            self._lib.nixl_capi_free_buffer(name)
+
+    def remove_remote_agent(self, agent):
+        """Reference: _api.py:899-907."""
+        _check("remove_remote_agent", self._lib.nixl_capi_invalidate_remote_md(self._h, agent.encode()))
+
+    def check_remote_metadata(self, agent, descs=None):
+        """Reference: _api.py:976-992."""
+        return self._lib.nixl_capi_check_remote_md(self._h, agent.encode(), descs._h if descs is not None else None) == 0
+
+    def make_connection(self, remote_agent, backends=()):
+        """Reference: _api.py:471-481."""
+        o = self._opt_args(backends)
+        try:
+            _check("make_connection", self._lib.nixl_capi_make_connection(self._h, remote_agent.encode(), o))
+        finally:
+            self._free_opt(o)
+
+    def _drain_notifs(self, into, backends=()):
+        m = ctypes.c_void_p()
+        _check("create_notif_map", self._lib.nixl_capi_create_notif_map(ctypes.byref(m)))
+        o = self._opt_args(backends)
+        try:
+            _check("get_notifs", self._lib.nixl_capi_get_notifs(self._h, m, o))
+            n = ctypes.c_size_t()
+            self._lib.nixl_capi_notif_map_size(m, ctypes.byref(n))
+            for i in range(n.value):
+                name = ctypes.c_char_p()
+                self._lib.nixl_capi_notif_map_get_agent_at(m, i, ctypes.byref(name))
+                count = ctypes.c_size_t()
+                self._lib.nixl_capi_notif_map_get_notifs_size(m, name.value, ctypes.byref(count))
+                msgs = into.setdefault(name.value.decode(), [])
+                for j in range(count.value):
+                    data, size = ctypes.c_void_p(), ctypes.c_size_t()
+                    self._lib.nixl_capi_notif_map_get_notif(m, name.value, j, ctypes.byref(data), ctypes.byref(size))
+                    msgs.append(ctypes.string_at(data, size.value))
+        finally:
+            self._free_opt(o)
+            self._lib.nixl_capi_destroy_notif_map(m)
+        return into
+
+    def get_new_notifs(self, backends=()):
+        """Reference: _api.py:770-783: {agent name: [messages]} that arrived since the last call."""
+        return self._drain_notifs({}, backends)
+
+    def update_notifs(self, backends=()):
+        """Reference: _api.py:785-799: like get_new_notifs, accumulated in self.notifs."""
+        return self._drain_notifs(self.notifs, backends)
+
+    def check_remote_xfer_done(self, remote_agent_name, lookup_tag, backends=(), tag_is_prefix=True):
+        """Reference: _api.py:801-838: looks for one message of `remote_agent_name` that starts
+        with (or contains) the tag, and removes just that one."""
+        self._drain_notifs(self.notifs, backends)
+        for msg in self.notifs.get(remote_agent_name, []):
+            if (tag_is_prefix and msg.startswith(lookup_tag)) or (not tag_is_prefix and lookup_tag in msg):
+                self.notifs[remote_agent_name].remove(msg)
+                return True
+        return False
+
+    def send_notif(self, remote_agent_name, notif_msg, backend=None):
+        """Reference: _api.py:840-854."""
+        msg = notif_msg.encode() if isinstance(notif_msg, str) else bytes(notif_msg)
+        o = self._opt_args([backend] if backend else ())
+        try:
+            _check("send_notif", self._lib.nixl_capi_gen_notif(self._h, remote_agent_name.encode(), msg, len(msg), o))
+        finally:
+            self._free_opt(o)
+
     def prep_mem_view(self, dlist, *, backends=None):
         """Reference: _api.py:728-759.  A local (nixl_xfer_dlist) or remote
         (nixl_remote_dlist) list becomes a table that device code indexes; returns the handle
@@ -380,8 +482,8 @@ class nixl_agent:
         """Reference: _api.py:761-768."""
         _check("release_mem_view", self._lib.nixl_capi_release_mem_view(self._h, ctypes.c_void_p(int(mvh))))
 
-    def _opt_args(self, backends=(), skip_desc_merge=False, notif_msg=b""):
-        if not backends and not skip_desc_merge and not notif_msg:
+    def _opt_args(self, backends=(), skip_desc_merge=False, notif_msg=b"", include_conn_info=False):
+        if not backends and not skip_desc_merge and not notif_msg and not include_conn_info:
             return None
         o = ctypes.c_void_p()
         _check("create_opt_args", self._lib.nixl_capi_create_opt_args(ctypes.byref(o)))
@@ -389,6 +491,8 @@ class nixl_agent:
             self._lib.nixl_capi_opt_args_add_backend(o, self.backends[b])
         if skip_desc_merge:
             self._lib.nixl_capi_opt_args_set_skip_desc_merge(o, True)
+        if include_conn_info:
+            self._lib.nixl_capi_opt_args_set_include_conn_info(o, True)
         if notif_msg:
             self._lib.nixl_capi_opt_args_set_notif_msg(o, notif_msg, len(notif_msg))
             self._lib.nixl_capi_opt_args_set_has_notif(o, True)

@@ -9,6 +9,7 @@
 #include <mutex>
 
 #include "agent_impl.h"
+#include "serdes.h"
 #include "common/nixl_log.h"
 
 namespace fs = std::filesystem;
@@ -257,6 +258,13 @@ const std::string nixl_null_agent = "NULL_AGENT";
 nixlAgentData::~nixlAgentData() {
     for (const auto &[view, engine] : mvhToEngine)
         engine->releaseMemView(view);
+    // Peers' descriptors were loaded into the backends; hand them back
+    // (reference: ~nixlRemoteSection, src/infra/nixl_memory_section.cpp:554-561).
+    std::vector<std::string> peers;
+    for (const auto &kv : remoteSections_)
+        if (kv.first != name_) peers.push_back(kv.first);
+    for (const std::string &peer : peers)
+        dropRemote(peer);
     // Deregister whatever the application left registered, then destroy engines through
     // the plugin that made them (reference: src/infra/nixl_memory_section.cpp:416-423).
     for (auto &[key, list] : localSection_.sections)
@@ -363,9 +371,9 @@ nixlAgent::createBackend(const nixl_backend_t &type, const nixl_b_params_t &para
         NIXL_ERROR_FUNC << "backend initialization error for '" << type << "'";
         return drop(NIXL_ERR_BACKEND);
     }
+    std::string conn;
     if (engine->supportsRemote()) {
         // A remote-capable backend must also carry notifications and connection info.
-        std::string conn;
         if (!engine->supportsNotif()) return drop(NIXL_ERR_BACKEND);
         const nixl_status_t st = engine->getConnInfo(conn);
         if (st != NIXL_SUCCESS) return drop(st);
@@ -377,6 +385,8 @@ nixlAgent::createBackend(const nixl_backend_t &type, const nixl_b_params_t &para
             return drop(st);
         }
     }
+    if (engine->supportsRemote()) data->connMd_[type] = conn;
+    if (engine->supportsNotif()) data->notifEngines.push_back(engine);
     for (nixl_mem_t m : engine->getSupportedMems())
         data->memToBackend[m].push_back(engine);
 
@@ -409,6 +419,16 @@ registerWithBackend(nixlAgentData &d, const nixl_reg_dlist_t &descs, nixlBackend
                 backend->deregisterMem(entry.metadataP);
                 break;
             }
+        }
+        if (backend->supportsRemote()) {
+            // what a peer needs to address this region; travels in getLocalMD
+            st = backend->getPublicData(entry.metadataP, entry.metaBlob);
+            if (st != NIXL_SUCCESS) {
+                if (local && mirror.metadataP != entry.metadataP) backend->unloadMD(mirror.metadataP);
+                backend->deregisterMem(entry.metadataP);
+                break;
+            }
+            mirror.metaBlob = entry.metaBlob;
         }
         mine.push_back(entry);
         if (local) self.push_back(mirror);
@@ -552,16 +572,46 @@ nixlAgent::queryMem(const nixl_reg_dlist_t &descs,
 
 // reference: src/core/nixl_agent.cpp:563-618 (only the agent itself is a known peer here)
 nixl_status_t
-nixlAgent::makeConnection(const std::string &remote_agent, const nixl_opt_args_t *) {
+nixlAgent::makeConnection(const std::string &remote_agent, const nixl_opt_args_t *extra_params) {
     std::unique_lock guard(data->lock);
-    if (remote_agent != data->name_) return NIXL_ERR_NOT_FOUND;
-    nixl_status_t st = NIXL_ERR_BACKEND;
-    for (const auto &s : data->engines_) {
-        if (!s->engine->supportsLocal()) continue;
-        st = s->engine->connect(remote_agent);
-        if (st != NIXL_SUCCESS) return st;
+    if (remote_agent == data->name_) {
+        // the agent's own backends, as at creation
+        nixl_status_t st = NIXL_ERR_BACKEND;
+        for (const auto &s : data->engines_) {
+            if (!s->engine->supportsLocal()) continue;
+            st = s->engine->connect(remote_agent);
+            if (st != NIXL_SUCCESS) return st;
+        }
+        return st;
     }
-    return st;
+    const auto peer = data->remoteBackends_.find(remote_agent);
+    if (peer == data->remoteBackends_.end() || peer->second.empty()) {
+        NIXL_ERROR_FUNC << "metadata for remote agent '" << remote_agent << "' not found";
+        return NIXL_ERR_NOT_FOUND;
+    }
+    std::set<nixl_backend_t> types;
+    if (extra_params && !extra_params->backends.empty())
+        for (const nixlBackendH *h : extra_params->backends)
+            types.insert(h->getType());
+    else
+        for (const auto &kv : peer->second)
+            types.insert(kv.first);
+    int made = 0;
+    for (const nixl_backend_t &type : types) {
+        nixlAgentData::engineSlot *slot = data->slotOf(type);
+        if (!slot) continue;
+        const nixl_status_t st = slot->engine->connect(remote_agent);
+        if (st != NIXL_SUCCESS) {
+            NIXL_ERROR_FUNC << "connect('" << remote_agent << "') failed on backend '" << type << "' with status " << st;
+            return st;
+        }
+        ++made;
+    }
+    if (made == 0) {
+        NIXL_ERROR_FUNC << "no common backend to connect with '" << remote_agent << "'";
+        return NIXL_ERR_BACKEND;
+    }
+    return NIXL_SUCCESS;
 }
 
 // reference: src/core/nixl_agent.cpp:620-687
@@ -1055,27 +1105,380 @@ nixlAgent::releaseMemView(nixlMemViewH mvh) const {
     engine->releaseMemView(mvh);
 }
 
+// ---- notifications ------------------------------------------------------------------------
+
+// reference: src/core/nixl_agent.cpp:1322-1380
 nixl_status_t
-nixlAgent::getNotifs(nixl_notifs_t &, const nixl_opt_args_t *) {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgent::getNotifs(nixl_notifs_t &notif_map, const nixl_opt_args_t *extra_params) {
+    std::unique_lock guard(data->lock);
+    std::vector<nixlBackendEngine *> engines;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (const nixlBackendH *h : extra_params->backends)
+            if (h->engine->supportsNotif()) engines.push_back(h->engine);
+    } else {
+        engines = data->notifEngines;
+    }
+    if (engines.empty()) {
+        NIXL_ERROR_FUNC << "no specified or potential backend supports notifications";
+        return NIXL_ERR_BACKEND;
+    }
+    // Best effort: an error of one backend is reported, the others are still drained.
+    nixl_status_t worst = NIXL_SUCCESS;
+    for (nixlBackendEngine *e : engines) {
+        notif_list_t fresh;
+        const nixl_status_t st = e->getNotifs(fresh);
+        if (st < 0) {
+            NIXL_ERROR_FUNC << "backend '" << e->getType() << "' returned error status " << st
+                            << " while getting notifications";
+            worst = st;
+        }
+        for (auto &[from, msg] : fresh)
+            notif_map[from].push_back(std::move(msg));
+    }
+    return worst;
+}
+
+// reference: src/core/nixl_agent.cpp:1382-1444
+nixl_status_t
+nixlAgent::genNotif(const std::string &remote_agent, const nixl_blob_t &msg, const nixl_opt_args_t *extra_params) const {
+    std::shared_lock guard(data->lock);
+    std::vector<nixlBackendEngine *> engines;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (const nixlBackendH *h : extra_params->backends)
+            if (h->engine->supportsNotif()) engines.push_back(h->engine);
+    } else {
+        engines = data->notifEngines;
+    }
+    if (engines.empty()) {
+        NIXL_ERROR_FUNC << "no specified or potential backend supports notifications";
+        return NIXL_ERR_BACKEND;
+    }
+    if (remote_agent == data->name_) {
+        for (nixlBackendEngine *e : engines)
+            if (e->supportsLocal()) return e->genNotif(remote_agent, msg);
+        NIXL_ERROR_FUNC << "no specified or potential backend can send intra-agent notifications";
+        return NIXL_ERR_NOT_FOUND;
+    }
+    const auto peer = data->remoteBackends_.find(remote_agent);
+    if (peer != data->remoteBackends_.end())
+        for (nixlBackendEngine *e : engines)
+            if (peer->second.count(e->getType())) return e->genNotif(remote_agent, msg);
+    NIXL_ERROR_FUNC << "no specified or potential backend could send the inter-agent notifications";
+    return NIXL_ERR_NOT_FOUND;
+}
+
+// ---- metadata -----------------------------------------------------------------------------
+
+namespace {
+
+// A section list on the wire: "nixlSecElms" count, then per (memory type, backend) a "bknd"
+// name and the descriptor list as a registration list whose blobs are the backends' public
+// data (reference: serializeSections, src/infra/nixl_memory_section.cpp:333-363;
+// nixlDescList<T>::serialize, src/infra/nixl_descriptors.cpp:236-282).
+using section_pick_t = std::vector<std::pair<nixl_section_key_t, std::vector<const nixlSectionDesc *>>>;
+
+nixl_status_t
+writeSections(nixlSerDes &sd, const section_pick_t &picked) {
+    const size_t count = picked.size();
+    nixl_status_t st = sd.addBuf("nixlSecElms", &count, sizeof(count));
+    for (const auto &[key, descs] : picked) {
+        if (st != NIXL_SUCCESS) break;
+        const nixl_mem_t mem = key.first;
+        const size_t n = descs.size();
+        st = sd.addStr("bknd", key.second->getType());
+        if (st == NIXL_SUCCESS) st = sd.addStr("nixlDList", "nixlSDList");
+        if (st == NIXL_SUCCESS) st = sd.addBuf("t", &mem, sizeof(mem));
+        if (st == NIXL_SUCCESS) st = sd.addBuf("n", &n, sizeof(n));
+        for (const nixlSectionDesc *d : descs) {
+            if (st != NIXL_SUCCESS) break;
+            st = sd.addStr("", static_cast<const nixlBasicDesc *>(d)->serialize() + d->metaBlob);
+        }
+    }
+    return st;
+}
+
+// The inverse for one list (reference: nixlDescList<T>::nixlDescList(nixlSerDes *),
+// src/infra/nixl_descriptors.cpp:141-190).  An empty result means a malformed list.
+nixl_reg_dlist_t
+readRegList(nixlSerDes &sd) {
+    nixl_reg_dlist_t out(DRAM_SEG);
+    if (sd.getStr("nixlDList") != "nixlSDList") return out;
+    nixl_mem_t mem;
+    size_t n = 0;
+    if (sd.getBuf("t", &mem, sizeof(mem)) != NIXL_SUCCESS || mem < DRAM_SEG || mem > FILE_SEG) return out;
+    if (sd.getBuf("n", &n, sizeof(n)) != NIXL_SUCCESS) return out;
+    nixl_reg_dlist_t list(mem);
+    for (size_t i = 0; i < n; ++i) {
+        const std::string item = sd.getStr("");
+        if (item.size() < sizeof(nixlBasicDesc)) return out;
+        list.addDesc(nixlBlobDesc(item));
+    }
+    return list;
 }
 
 nixl_status_t
-nixlAgent::genNotif(const std::string &, const nixl_blob_t &, const nixl_opt_args_t *) const {
-    return NIXL_ERR_NOT_SUPPORTED;
+writeHeader(nixlSerDes &sd, const std::string &name, const std::vector<std::pair<nixl_backend_t, nixl_blob_t>> &conns) {
+    const size_t count = conns.size();
+    nixl_status_t st = sd.addStr("Agent", name);
+    if (st == NIXL_SUCCESS) st = sd.addBuf("Conns", &count, sizeof(count));
+    for (const auto &[type, info] : conns) {
+        if (st == NIXL_SUCCESS) st = sd.addStr("t", type);
+        if (st == NIXL_SUCCESS) st = sd.addStr("c", info);
+    }
+    if (st == NIXL_SUCCESS) st = sd.addStr("", "MemSection");
+    return st;
+}
+
+} // namespace
+
+// reference: src/core/nixl_agent.cpp:1446-1507
+nixl_status_t
+nixlAgent::getLocalMD(nixl_blob_t &str) const {
+    std::shared_lock guard(data->lock);
+    if (data->connMd_.empty()) {
+        NIXL_ERROR_FUNC << "no backends support remote operations";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    nixlSerDes sd;
+    std::vector<std::pair<nixl_backend_t, nixl_blob_t>> conns(data->connMd_.begin(), data->connMd_.end());
+    if (writeHeader(sd, data->name_, conns) != NIXL_SUCCESS) return NIXL_ERR_UNKNOWN;
+
+    section_pick_t picked;
+    for (const auto &[key, list] : data->localSection_.sections) {
+        if (!key.second->supportsRemote()) continue;
+        std::vector<const nixlSectionDesc *> descs;
+        for (size_t i = 0; i < list.size(); ++i)
+            descs.push_back(&list[i]);
+        picked.emplace_back(key, std::move(descs));
+    }
+    const nixl_status_t st = writeSections(sd, picked);
+    if (st != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "serialization failed";
+        return st;
+    }
+    str = sd.exportStr();
+    return NIXL_SUCCESS;
+}
+
+// reference: src/core/nixl_agent.cpp:1509-1602, src/infra/nixl_memory_section.cpp:370-413
+nixl_status_t
+nixlAgent::getLocalPartialMD(const nixl_reg_dlist_t &descs, nixl_blob_t &str, const nixl_opt_args_t *extra_params) const {
+    std::shared_lock guard(data->lock);
+    std::vector<nixlBackendEngine *> wanted;
+    if (extra_params && !extra_params->backends.empty()) {
+        for (const nixlBackendH *h : extra_params->backends)
+            wanted.push_back(h->engine);
+    } else if (!descs.isEmpty()) {
+        wanted = data->memToBackend[descs.getType()];
+        if (wanted.empty()) {
+            NIXL_ERROR_FUNC << "no available backends for mem type '" << descs.getType() << "'";
+            return NIXL_ERR_NOT_FOUND;
+        }
+    } else {
+        for (const auto &slot : data->engines_)
+            wanted.push_back(slot->engine);
+    }
+    // Best effort: a backend without connection info does not support remote operation.
+    std::vector<nixlBackendEngine *> selected;
+    std::vector<std::pair<nixl_backend_t, nixl_blob_t>> conns;
+    for (nixlBackendEngine *b : wanted) {
+        const auto it = data->connMd_.find(b->getType());
+        if (it == data->connMd_.end()) continue;
+        selected.push_back(b);
+        conns.emplace_back(it->first, it->second);
+    }
+    if (selected.empty() && descs.descCount() > 0) {
+        NIXL_ERROR_FUNC << "no backends support the requested descriptors";
+        return NIXL_ERR_BACKEND;
+    }
+    // Connection info travels only on request, or when no descriptors were named.
+    if (!((extra_params && extra_params->includeConnInfo) || descs.descCount() == 0)) conns.clear();
+
+    nixlSerDes sd;
+    if (writeHeader(sd, data->name_, conns) != NIXL_SUCCESS) return NIXL_ERR_UNKNOWN;
+    section_pick_t picked;
+    if (!descs.isEmpty()) {
+        for (nixlBackendEngine *b : selected) {
+            const nixl_section_key_t key{descs.getType(), b};
+            const auto sec = data->localSection_.sections.find(key);
+            if (sec == data->localSection_.sections.end()) continue;
+            std::vector<const nixlSectionDesc *> found;
+            for (const nixlBlobDesc &d : descs) {
+                const int i = sec->second.indexOf(d);
+                if (i < 0) {
+                    NIXL_ERROR_FUNC << "serialization failed";
+                    return NIXL_ERR_NOT_FOUND;
+                }
+                found.push_back(&sec->second[static_cast<size_t>(i)]);
+            }
+            picked.emplace_back(key, std::move(found));
+        }
+    }
+    const nixl_status_t st = writeSections(sd, picked);
+    if (st != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "serialization failed";
+        return st;
+    }
+    str = sd.exportStr();
+    return NIXL_SUCCESS;
 }
 
 nixl_status_t
-nixlAgent::getLocalMD(nixl_blob_t &) const {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgentData::dropRemote(const std::string &remote_name) {
+    const auto sec = remoteSections_.find(remote_name);
+    if (sec == remoteSections_.end()) return NIXL_ERR_NOT_FOUND;
+    for (auto &[key, list] : sec->second.sections)
+        for (size_t i = 0; i < list.size(); ++i)
+            key.second->unloadMD(list[i].metadataP);
+    remoteSections_.erase(sec);
+    const auto peer = remoteBackends_.find(remote_name);
+    if (peer != remoteBackends_.end()) {
+        for (const auto &kv : peer->second)
+            if (engineSlot *slot = slotOf(kv.first)) slot->engine->disconnect(remote_name);
+        remoteBackends_.erase(peer);
+    }
+    return NIXL_SUCCESS;
 }
 
+// reference: src/core/nixl_agent.cpp:1604-1683 (blob), :1746-1785 (connection info),
+// :1787-1799 and src/infra/nixl_memory_section.cpp:430-505 (sections)
 nixl_status_t
-nixlAgent::loadRemoteMD(const nixl_blob_t &, std::string &) {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgent::loadRemoteMD(const nixl_blob_t &remote_metadata, std::string &agent_name) {
+    std::unique_lock guard(data->lock);
+    nixlSerDes sd;
+    if (sd.importStr(remote_metadata) != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "failed to deserialize remote metadata";
+        return NIXL_ERR_MISMATCH;
+    }
+    const std::string remote = sd.getStr("Agent");
+    if (remote.empty()) {
+        NIXL_ERROR_FUNC << "error in deserializing remote agent name";
+        return NIXL_ERR_MISMATCH;
+    }
+    if (remote == data->name_) {
+        NIXL_ERROR_FUNC << "remote agent name same as local agent, no need to load metadata";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    size_t conn_cnt = 0;
+    if (sd.getBuf("Conns", &conn_cnt, sizeof(conn_cnt)) != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "error getting connection count";
+        return NIXL_ERR_MISMATCH;
+    }
+
+    size_t usable = 0;
+    for (size_t i = 0; i < conn_cnt; ++i) {
+        const nixl_backend_t type = sd.getStr("t");
+        const nixl_blob_t info = sd.getStr("c");
+        if (type.empty() || info.empty()) {
+            NIXL_ERROR_FUNC << "failed to deserialize remote metadata";
+            return NIXL_ERR_MISMATCH;
+        }
+        nixlAgentData::engineSlot *slot = data->slotOf(type);
+        if (!slot || !slot->engine->supportsRemote()) continue; // not a common backend
+        auto &known = data->remoteBackends_[remote];
+        const auto seen = known.find(type);
+        if (seen != known.end()) {
+            // the same connection info again is fine; a different one is not accepted
+            if (seen->second != info) return NIXL_ERR_NOT_ALLOWED;
+            ++usable;
+            continue;
+        }
+        const nixl_status_t st = slot->engine->loadRemoteConnInfo(remote, info);
+        if (st == NIXL_SUCCESS) {
+            known.emplace(type, info);
+            ++usable;
+        } else {
+            if (known.empty()) data->remoteBackends_.erase(remote);
+            if (st != NIXL_ERR_NOT_SUPPORTED) {
+                NIXL_ERROR_FUNC << "error loading connection info for backend '" << type << "' with status " << st;
+                return st;
+            }
+        }
+    }
+    if (usable == 0 && conn_cnt > 0) {
+        NIXL_ERROR_FUNC << "no common backend found";
+        return NIXL_ERR_BACKEND;
+    }
+    if (sd.getStr("") != "MemSection") {
+        NIXL_ERROR_FUNC << "failed to deserialize remote metadata";
+        return NIXL_ERR_MISMATCH;
+    }
+
+    size_t sections = 0;
+    nixl_status_t st = sd.getBuf("nixlSecElms", &sections, sizeof(sections));
+    nixlMemSection &target = data->remoteSections_[remote];
+    for (size_t i = 0; st == NIXL_SUCCESS && i < sections; ++i) {
+        const nixl_backend_t type = sd.getStr("bknd");
+        if (type.empty()) {
+            st = NIXL_ERR_INVALID_PARAM;
+            break;
+        }
+        const nixl_reg_dlist_t regions = readRegList(sd);
+        if (regions.isEmpty()) {
+            st = NIXL_ERR_NOT_FOUND;
+            break;
+        }
+        nixlAgentData::engineSlot *slot = data->slotOf(type);
+        if (!slot) continue; // a backend this agent does not have
+        nixlBackendEngine *backend = slot->engine;
+        if (!backend->supportsRemote()) {
+            st = NIXL_ERR_UNKNOWN;
+            break;
+        }
+        const nixl_mem_t mem = regions.getType();
+        nixlSecDescList &list = target.sections[{mem, backend}];
+        target.memToBackend[mem].insert(backend);
+        std::vector<nixlSectionDesc> fresh;
+        for (const nixlBlobDesc &region : regions) {
+            const int at = list.indexOf(region);
+            if (at >= 0) {
+                // already known: the published data must not have changed
+                if (list[static_cast<size_t>(at)].metaBlob != region.metaInfo) st = NIXL_ERR_NOT_ALLOWED;
+                if (st != NIXL_SUCCESS) break;
+                continue;
+            }
+            nixlSectionDesc entry(region.addr, region.len, region.devId, nullptr);
+            st = backend->loadRemoteMD(region, mem, remote, entry.metadataP);
+            if (st != NIXL_SUCCESS) break;
+            entry.metaBlob = region.metaInfo;
+            fresh.push_back(std::move(entry));
+        }
+        // what was loaded is kept in the list either way, so that a failure unloads it below
+        list.add(std::move(fresh));
+    }
+    if (st != NIXL_SUCCESS) {
+        NIXL_ERROR_FUNC << "error loading remote metadata for agent '" << remote << "' with status " << st;
+        data->dropRemote(remote);
+        return st;
+    }
+    agent_name = remote;
+    return NIXL_SUCCESS;
 }
 
+// reference: src/core/nixl_agent.cpp:1801-1836
 nixl_status_t
-nixlAgent::invalidateRemoteMD(const std::string &) {
-    return NIXL_ERR_NOT_SUPPORTED;
+nixlAgent::invalidateRemoteMD(const std::string &remote_agent) {
+    std::unique_lock guard(data->lock);
+    if (remote_agent == data->name_) {
+        NIXL_ERROR_FUNC << "agent '" << data->name_ << "' cannot invalidate itself";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    return data->dropRemote(remote_agent);
+}
+
+// reference: src/core/nixl_agent.cpp:1862-1887
+nixl_status_t
+nixlAgent::checkRemoteMD(const std::string remote_name, const nixl_xfer_dlist_t &descs) const {
+    std::shared_lock guard(data->lock);
+    const auto sec = data->remoteSections_.find(remote_name);
+    if (sec == data->remoteSections_.end()) return NIXL_ERR_NOT_FOUND;
+    if (descs.isEmpty()) return NIXL_SUCCESS;
+    const auto peer = data->remoteBackends_.find(remote_name);
+    if (peer == data->remoteBackends_.end()) return NIXL_ERR_NOT_FOUND;
+    nixl_meta_dlist_t scratch(descs.getType());
+    for (const auto &kv : peer->second) {
+        nixlAgentData::engineSlot *slot = data->slotOf(kv.first);
+        if (slot && sec->second.populate(descs, slot->engine, scratch) == NIXL_SUCCESS) return NIXL_SUCCESS;
+    }
+    return NIXL_ERR_NOT_FOUND;
 }

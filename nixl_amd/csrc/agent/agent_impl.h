@@ -195,8 +195,20 @@ public:
     std::array<std::vector<nixlBackendEngine *>, FILE_SEG + 1> memToBackend;
 
     nixlMemSection localSection_;
-    // Only the agent itself can be a "remote" here (loopback).
+    // The agent itself (loopback, filled at registration) and every peer whose metadata
+    // was loaded.
     std::unordered_map<std::string, nixlMemSection> remoteSections_;
+    // Connection info of every remote-capable backend of this agent, by backend type
+    // (what getLocalMD publishes), and what each peer published, as loaded
+    // (src/core/agent_data.h:57-66).
+    std::unordered_map<nixl_backend_t, nixl_blob_t> connMd_;
+    std::unordered_map<std::string, std::unordered_map<nixl_backend_t, nixl_blob_t>> remoteBackends_;
+    std::vector<nixlBackendEngine *> notifEngines;
+
+    // Drops a peer's sections (unloading every descriptor from its backend) and
+    // disconnects its backends.  The caller holds the lock exclusively.
+    nixl_status_t
+    dropRemote(const std::string &remote_name);
 
     // Which engine made each live memory view (src/core/agent_data.h mvhToEngine).
     std::unordered_map<nixlMemViewH, nixlBackendEngine *> mvhToEngine;

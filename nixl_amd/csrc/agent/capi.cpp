@@ -1,7 +1,10 @@
 // extern "C" façade over nixlAgent (declared in include/nixl_amd_capi.h).
 #include "nixl_amd_capi.h"
 
+#include <cstdlib>
+#include <cstring>
 #include <exception>
+#include <iterator>
 #include <thread>
 
 #include "agent_impl.h"
@@ -20,6 +23,9 @@ struct nixl_capi_opt_args_s {
 };
 struct nixl_capi_xfer_dlist_s {
     nixl_xfer_dlist_t *dlist;
+};
+struct nixl_capi_notif_map_s {
+    nixl_notifs_t notifs;
 };
 struct nixl_capi_remote_dlist_s {
     nixl_remote_dlist_t *dlist;
@@ -207,6 +213,13 @@ nixl_capi_status_t
 nixl_capi_opt_args_set_skip_desc_merge(nixl_capi_opt_args_t args, bool skip_merge) {
     if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
     args->args.skipDescMerge = skip_merge;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_include_conn_info(nixl_capi_opt_args_t args, bool include) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.includeConnInfo = include;
     return NIXL_CAPI_SUCCESS;
 }
 
@@ -690,6 +703,158 @@ nixl_capi_release_mem_view(nixl_capi_agent_t agent, nixl_capi_mem_view_t mvh) {
         agent->inner->releaseMemView(static_cast<nixlMemViewH>(mvh));
         return NIXL_CAPI_SUCCESS;
     });
+}
+
+namespace {
+
+nixl_capi_status_t
+copyOut(const std::string &blob, void **data, size_t *len) {
+    void *copy = std::malloc(blob.size() ? blob.size() : 1);
+    if (!copy) return NIXL_CAPI_ERROR_BACKEND;
+    std::memcpy(copy, blob.data(), blob.size());
+    *data = copy;
+    *len = blob.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+} // namespace
+
+nixl_capi_status_t
+nixl_capi_get_local_md(nixl_capi_agent_t agent, void **data, size_t *len) {
+    if (!agent || !data || !len) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_blob_t blob;
+        const nixl_status_t st = agent->inner->getLocalMD(blob);
+        if (st != NIXL_SUCCESS) return fold(st);
+        return copyOut(blob, data, len);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_get_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, void **data, size_t *len,
+                               nixl_capi_opt_args_t opt_args) {
+    if (!agent || !descs || !data || !len) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        nixl_blob_t blob;
+        const nixl_status_t st = agent->inner->getLocalPartialMD(*descs->dlist, blob, opt_args ? &opt_args->args : nullptr);
+        if (st != NIXL_SUCCESS) return fold(st);
+        return copyOut(blob, data, len);
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_load_remote_md(nixl_capi_agent_t agent, const void *data, size_t len, char **agent_name) {
+    if (!agent || !data || !len || !agent_name) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        std::string name;
+        const nixl_status_t st = agent->inner->loadRemoteMD(nixl_blob_t(static_cast<const char *>(data), len), name);
+        if (st != NIXL_SUCCESS) return fold(st);
+        *agent_name = ::strdup(name.c_str());
+        return *agent_name ? NIXL_CAPI_SUCCESS : NIXL_CAPI_ERROR_BACKEND;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_invalidate_remote_md(nixl_capi_agent_t agent, const char *remote_agent) {
+    if (!agent || !remote_agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->invalidateRemoteMD(remote_agent)); });
+}
+
+nixl_capi_status_t
+nixl_capi_check_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_xfer_dlist_t descs) {
+    if (!agent || !remote_name) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        // no list: only ask whether the peer's metadata is present
+        static const nixl_xfer_dlist_t none(DRAM_SEG);
+        return fold(agent->inner->checkRemoteMD(remote_name, descs ? *descs->dlist : none));
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !remote_agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->makeConnection(remote_agent, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_free_buffer(void *data) {
+    std::free(data);
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_create_notif_map(nixl_capi_notif_map_t *notif_map) {
+    if (!notif_map) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        *notif_map = new nixl_capi_notif_map_s;
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_notif_map(nixl_capi_notif_map_t notif_map) {
+    if (!notif_map) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete notif_map;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_get_notifs(nixl_capi_agent_t agent, nixl_capi_notif_map_t notif_map, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !notif_map) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->getNotifs(notif_map->notifs, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_gen_notif(nixl_capi_agent_t agent, const char *remote_agent, const void *data, size_t len,
+                    nixl_capi_opt_args_t opt_args) {
+    if (!agent || !remote_agent || (len && !data)) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        const nixl_blob_t msg(static_cast<const char *>(data), len);
+        return fold(agent->inner->genNotif(remote_agent, msg, opt_args ? &opt_args->args : nullptr));
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_notif_map_size(nixl_capi_notif_map_t map, size_t *size) {
+    if (!map || !size) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *size = map->notifs.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_notif_map_get_agent_at(nixl_capi_notif_map_t map, size_t index, const char **agent_name) {
+    if (!map || !agent_name || index >= map->notifs.size()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    auto it = map->notifs.begin();
+    std::advance(it, index);
+    *agent_name = it->first.c_str();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_notif_map_get_notifs_size(nixl_capi_notif_map_t map, const char *agent_name, size_t *size) {
+    if (!map || !agent_name || !size) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    const auto it = map->notifs.find(agent_name);
+    if (it == map->notifs.end()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *size = it->second.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_notif_map_get_notif(nixl_capi_notif_map_t map, const char *agent_name, size_t index, const void **data,
+                              size_t *len) {
+    if (!map || !agent_name || !data || !len) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    const auto it = map->notifs.find(agent_name);
+    if (it == map->notifs.end() || index >= it->second.size()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *data = it->second[index].data();
+    *len = it->second[index].size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_notif_map_clear(nixl_capi_notif_map_t map) {
+    if (!map) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    map->notifs.clear();
+    return NIXL_CAPI_SUCCESS;
 }
 
 } // extern "C"

@@ -1,7 +1,11 @@
 #include "hip_backend.h"
 
+#include <unistd.h>
+
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <unordered_map>
 
 #include "backend/backend_plugin.h"
 #include "common/nixl_log.h"
@@ -28,6 +32,22 @@ hipOk(hipError_t e, const char *what) {
     NIXL_ERROR << "HIP backend: " << what << " failed: " << hipGetErrorString(e);
     return false;
 }
+
+// Engines of this process by agent name: how a notification reaches another agent's queue.
+std::mutex g_registryMutex;
+std::unordered_map<std::string, const nixlHipEngine *> g_registry;
+
+// What a peer needs to address a region (getPublicData / loadRemoteMD).
+struct PublicRegion {
+    uint64_t magic;
+    uint64_t addr;
+    uint64_t len;
+    int64_t pid;
+    int32_t device;
+    int32_t mem;
+};
+constexpr uint64_t kRegionMagic = 0x314e474552504948ull; // "HIPREGN1"
+constexpr const char *kConnPrefix = "HIP1:pid=";
 
 } // namespace
 
@@ -71,9 +91,16 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     }
     numDevices_ = n;
     streams_.assign(static_cast<size_t>(n) * streamsPerDevice_, nullptr);
+    std::lock_guard<std::mutex> lock(g_registryMutex);
+    g_registry[localAgent] = this;
 }
 
 nixlHipEngine::~nixlHipEngine() {
+    {
+        std::lock_guard<std::mutex> lock(g_registryMutex);
+        const auto it = g_registry.find(localAgent);
+        if (it != g_registry.end() && it->second == this) g_registry.erase(it);
+    }
     reapRetired(true);
     for (const auto &[table, device] : memViews_) {
         (void)hipSetDevice(device);
@@ -115,9 +142,10 @@ nixlHipEngine::reapRetired(bool wait) const {
             else
                 finished = (hipEventQuery(r->done) != hipErrorNotReady);
         }
-        if (finished)
+        if (finished) {
+            deliverPending(r);
             delete r;
-        else
+        } else
             retired_[keep++] = r;
     }
     retired_.resize(keep);
@@ -194,13 +222,12 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
     handle = nullptr;
     reapRetired(false);
 
-    if (remote_agent != localAgent) {
-        NIXL_ERROR << "HIP backend: only loopback transfers are supported (agent '" << localAgent
-                   << "', remote '" << remote_agent << "')";
-        return NIXL_ERR_INVALID_PARAM;
+    if (!knowsAgent(remote_agent)) {
+        NIXL_ERROR << "HIP backend: agent '" << remote_agent << "' is neither this agent ('" << localAgent
+                   << "') nor a peer whose connection info was loaded";
+        return NIXL_ERR_NOT_FOUND;
     }
     if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
-    if (opt_args && opt_args->hasNotif) return NIXL_ERR_NOT_SUPPORTED;
     const int n = local.descCount();
     if (n == 0 || n != remote.descCount()) {
         NIXL_ERROR << "HIP backend: descriptor count mismatch (local " << n << ", remote "
@@ -264,14 +291,20 @@ nixl_status_t
 nixlHipEngine::postXfer(const nixl_xfer_op_t &,
                         const nixl_meta_dlist_t &,
                         const nixl_meta_dlist_t &,
-                        const std::string &,
+                        const std::string &remote_agent,
                         nixlBackendReqH *&handle,
                         const nixl_opt_b_args_t *opt_args) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req || !req->plan) return NIXL_ERR_INVALID_PARAM;
-    if (opt_args && opt_args->hasNotif) return NIXL_ERR_NOT_SUPPORTED;
     if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
     if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
+    // the notification of an earlier post that nobody polled to completion goes out first
+    deliverPending(req);
+    if (opt_args && opt_args->hasNotif) {
+        req->notifPending = true;
+        req->notifTarget = remote_agent;
+        req->notifMsg = opt_args->notifMsg;
+    }
 
     if (nixl_amd_copy_plan_launch(req->plan, req->stream) != NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
@@ -289,7 +322,11 @@ nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
     if (!req->posted) return NIXL_SUCCESS; // nothing outstanding
     if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
     const hipError_t e = hipEventQuery(req->done);
-    if (e == hipSuccess) return NIXL_SUCCESS;
+    if (e == hipSuccess) {
+        // the peer learns of the transfer only after its bytes have landed
+        deliverPending(req);
+        return NIXL_SUCCESS;
+    }
     if (e == hipErrorNotReady) return NIXL_IN_PROG;
     NIXL_ERROR << "HIP backend: transfer failed: " << hipGetErrorString(e);
     return NIXL_ERR_BACKEND;
@@ -307,7 +344,129 @@ nixlHipEngine::releaseReqH(nixlBackendReqH *handle) const {
         retired_.push_back(req);
         return NIXL_SUCCESS;
     }
+    if (req->posted) deliverPending(req);
     delete req;
+    return NIXL_SUCCESS;
+}
+
+// ---- peers in this process, notifications ------------------------------------------------
+
+bool
+nixlHipEngine::knowsAgent(const std::string &name) const {
+    if (name == localAgent) return true;
+    std::lock_guard<std::mutex> lock(peersMutex_);
+    return std::find(peers_.begin(), peers_.end(), name) != peers_.end();
+}
+
+void
+nixlHipEngine::deliverPending(nixlHipReqH *req) const {
+    if (!req->notifPending) return;
+    req->notifPending = false;
+    if (genNotif(req->notifTarget, req->notifMsg) != NIXL_SUCCESS)
+        NIXL_WARN << "HIP backend: notification for agent '" << req->notifTarget << "' could not be delivered";
+}
+
+nixl_status_t
+nixlHipEngine::getConnInfo(std::string &str) const {
+    str = kConnPrefix + std::to_string(static_cast<long long>(getpid()));
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::loadRemoteConnInfo(const std::string &remote_agent, const std::string &remote_conn_info) {
+    const size_t n = std::strlen(kConnPrefix);
+    if (remote_conn_info.compare(0, n, kConnPrefix) != 0) return NIXL_ERR_MISMATCH;
+    char *end = nullptr;
+    const long long pid = std::strtoll(remote_conn_info.c_str() + n, &end, 10);
+    if (end == remote_conn_info.c_str() + n || *end != '\0') return NIXL_ERR_MISMATCH;
+    if (pid != static_cast<long long>(getpid())) {
+        // Its addresses mean nothing here without IPC memory handles.
+        NIXL_WARN << "HIP backend: agent '" << remote_agent << "' lives in process " << pid
+                  << "; only agents of this process are reachable";
+        return NIXL_ERR_NOT_SUPPORTED;
+    }
+    std::lock_guard<std::mutex> lock(peersMutex_);
+    if (std::find(peers_.begin(), peers_.end(), remote_agent) == peers_.end()) peers_.push_back(remote_agent);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::connect(const std::string &remote_agent) {
+    return knowsAgent(remote_agent) ? NIXL_SUCCESS : NIXL_ERR_NOT_FOUND;
+}
+
+nixl_status_t
+nixlHipEngine::disconnect(const std::string &remote_agent) {
+    if (remote_agent == localAgent) return NIXL_SUCCESS;
+    std::lock_guard<std::mutex> lock(peersMutex_);
+    const auto it = std::find(peers_.begin(), peers_.end(), remote_agent);
+    if (it == peers_.end()) return NIXL_ERR_NOT_FOUND;
+    peers_.erase(it);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::getPublicData(const nixlBackendMD *meta, std::string &str) const {
+    const auto *md = static_cast<const nixlHipMD *>(meta);
+    if (!md) return NIXL_ERR_INVALID_PARAM;
+    PublicRegion region{};
+    region.magic = kRegionMagic;
+    region.addr = md->addr;
+    region.len = md->len;
+    region.pid = static_cast<int64_t>(getpid());
+    region.device = md->device;
+    region.mem = static_cast<int32_t>(md->mem);
+    str.assign(reinterpret_cast<const char *>(&region), sizeof(region));
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::loadRemoteMD(const nixlBlobDesc &input,
+                            const nixl_mem_t &nixl_mem,
+                            const std::string &remote_agent,
+                            nixlBackendMD *&output) {
+    output = nullptr;
+    if (!knowsAgent(remote_agent)) return NIXL_ERR_NOT_FOUND;
+    PublicRegion region{};
+    if (input.metaInfo.size() != sizeof(region)) return NIXL_ERR_MISMATCH;
+    std::memcpy(&region, input.metaInfo.data(), sizeof(region));
+    if (region.magic != kRegionMagic || region.pid != static_cast<int64_t>(getpid())) return NIXL_ERR_MISMATCH;
+    if (region.addr != input.addr || region.len != input.len || region.mem != static_cast<int32_t>(nixl_mem) ||
+        region.len == 0 || region.device < 0 || region.device >= numDevices_) {
+        NIXL_ERROR << "HIP backend: published data of agent '" << remote_agent << "' does not match its descriptor";
+        return NIXL_ERR_MISMATCH;
+    }
+    output = new nixlHipMD(region.addr, region.len, region.device, nixl_mem, /*of_peer=*/true);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::unloadMD(nixlBackendMD *input) {
+    // loadLocalMD hands out the registration itself, which deregisterMem frees
+    const auto *md = static_cast<const nixlHipMD *>(input);
+    if (md && md->ofPeer) delete md;
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::genNotif(const std::string &remote_agent, const std::string &msg) const {
+    std::lock_guard<std::mutex> registry(g_registryMutex);
+    const auto it = g_registry.find(remote_agent);
+    if (it == g_registry.end()) return NIXL_ERR_NOT_FOUND;
+    const nixlHipEngine *target = it->second;
+    std::lock_guard<std::mutex> lock(target->notifMutex_);
+    target->notifs_.emplace_back(localAgent, msg);
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
+nixlHipEngine::getNotifs(notif_list_t &notif_list) {
+    // transfers released while in flight may have finished since
+    reapRetired(false);
+    std::lock_guard<std::mutex> lock(notifMutex_);
+    for (auto &n : notifs_)
+        notif_list.push_back(std::move(n));
+    notifs_.clear();
     return NIXL_SUCCESS;
 }
 

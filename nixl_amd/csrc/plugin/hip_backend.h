@@ -1,5 +1,5 @@
-// nixlHipEngine: a local-only NIXL backend for VRAM<->VRAM descriptor transfers on one
-// AMD GPU.  It fills the same slot as the reference's local backends (shape of
+// nixlHipEngine: a NIXL backend for VRAM<->VRAM descriptor transfers on one AMD GPU, between
+// the regions of one agent (loopback) or of several agents that live in the same process.  It fills the same slot as the reference's local backends (shape of
 // src/plugins/posix/posix_backend.h:78-158; request life-cycle split of
 // src/plugins/cuda_gds/gds_backend.cpp:159-391): prepXfer lowers the two descriptor
 // lists once into a device-resident copy plan, postXfer enqueues one kernel launch and
@@ -22,17 +22,19 @@
 // Registration record returned by registerMem and handed back in nixlMetaDesc::metadataP.
 class nixlHipMD : public nixlBackendMD {
 public:
-    nixlHipMD(uintptr_t addr_, size_t len_, int device_, nixl_mem_t mem_)
-        : nixlBackendMD(true),
+    nixlHipMD(uintptr_t addr_, size_t len_, int device_, nixl_mem_t mem_, bool of_peer = false)
+        : nixlBackendMD(!of_peer),
           addr(addr_),
           len(len_),
           device(device_),
-          mem(mem_) {}
+          mem(mem_),
+          ofPeer(of_peer) {}
 
     const uintptr_t addr;
     const size_t len;
     const int device; // HIP device whose kernels may touch the region
     const nixl_mem_t mem;
+    const bool ofPeer; // made by loadRemoteMD from a peer's published data; unloadMD frees it
 
     bool
     contains(uintptr_t a, size_t l) const noexcept {
@@ -48,6 +50,10 @@ public:
     int device = 0;
     bool posted = false;
     size_t bytes = 0;
+    // A notification that is due once the posted transfer has finished.
+    bool notifPending = false;
+    std::string notifTarget;
+    std::string notifMsg;
 
     ~nixlHipReqH() override;
 };
@@ -57,9 +63,11 @@ public:
     explicit nixlHipEngine(const nixlBackendInitParams *init_params);
     ~nixlHipEngine() override;
 
+    // "Remote" means another agent of this process: its regions are plain addresses here.
+    // An agent in another process would need IPC memory handles, which are left out.
     bool
     supportsRemote() const override {
-        return false;
+        return true;
     }
 
     bool
@@ -69,7 +77,7 @@ public:
 
     bool
     supportsNotif() const override {
-        return false;
+        return true;
     }
 
     nixl_mem_list_t
@@ -83,19 +91,28 @@ public:
     deregisterMem(nixlBackendMD *meta) override;
 
     nixl_status_t
-    connect(const std::string &) override {
-        return NIXL_SUCCESS;
-    }
+    connect(const std::string &remote_agent) override;
+    nixl_status_t
+    disconnect(const std::string &remote_agent) override;
+    nixl_status_t
+    unloadMD(nixlBackendMD *input) override;
 
     nixl_status_t
-    disconnect(const std::string &) override {
-        return NIXL_SUCCESS;
-    }
+    getPublicData(const nixlBackendMD *meta, std::string &str) const override;
+    nixl_status_t
+    getConnInfo(std::string &str) const override;
+    nixl_status_t
+    loadRemoteConnInfo(const std::string &remote_agent, const std::string &remote_conn_info) override;
+    nixl_status_t
+    loadRemoteMD(const nixlBlobDesc &input,
+                 const nixl_mem_t &nixl_mem,
+                 const std::string &remote_agent,
+                 nixlBackendMD *&output) override;
 
     nixl_status_t
-    unloadMD(nixlBackendMD *) override {
-        return NIXL_SUCCESS;
-    }
+    getNotifs(notif_list_t &notif_list) override;
+    nixl_status_t
+    genNotif(const std::string &remote_agent, const std::string &msg) const override;
 
     nixl_status_t
     loadLocalMD(nixlBackendMD *input, nixlBackendMD *&output) override {
@@ -152,6 +169,10 @@ private:
     pickStream(int device) const;
     void
     reapRetired(bool wait) const;
+    bool
+    knowsAgent(const std::string &name) const;
+    void
+    deliverPending(nixlHipReqH *req) const;
     struct viewEntry {
         uintptr_t addr;
         size_t len;
@@ -172,6 +193,12 @@ private:
     // Requests released while their kernel was still running; freed once it has finished.
     mutable std::vector<nixlHipReqH *> retired_;
     mutable std::mutex retiredMutex_;
+    // Peers whose connection info was loaded (agents of this process).
+    mutable std::mutex peersMutex_;
+    std::vector<std::string> peers_;
+    // Notifications other agents (or this one) left for this agent.
+    mutable std::mutex notifMutex_;
+    mutable notif_list_t notifs_;
     // Live memory-view tables: device pointer -> owning device.
     mutable std::unordered_map<void *, int> memViews_;
     mutable std::mutex memViewsMutex_;

@@ -87,7 +87,11 @@ main(int argc, char **argv) {
     params.syncMode = nixl_thread_sync_t::NIXL_THREAD_SYNC_NONE;
     nixlBackendEngine *engine = plugin->create_engine(&params);
     REQUIRE(engine && !engine->getInitErr());
-    REQUIRE(engine->supportsLocal() && !engine->supportsRemote() && !engine->supportsNotif());
+    // remote = other agents of this process; a remote-capable backend must carry notifications
+    REQUIRE(engine->supportsLocal() && engine->supportsRemote() && engine->supportsNotif());
+    std::string conn;
+    REQUIRE(engine->getConnInfo(conn) == NIXL_SUCCESS && !conn.empty());
+    REQUIRE(engine->connect("stranger") == NIXL_ERR_NOT_FOUND);
     REQUIRE(engine->connect(agent) == NIXL_SUCCESS);
 
     // 48 descriptors of 20 KiB + one of 4 KiB + 16 B + one odd-sized one, local -> remote

@@ -236,12 +236,103 @@ def test_plugin_rejects_what_it_cannot_do(hip_agent, cuda):
     with pytest.raises(ag.NixlError):
         a.register_memory(np.array([[host.ctypes.data, 4096, 0]], dtype=np.uint64), "VRAM")
     a.register_memory([t])
-    # notifications are not supported by a local-only backend
+    # an agent nobody introduced
     ld = a.get_xfer_descs(_descs(t, [0], [16]), "VRAM")
     rd = a.get_xfer_descs(_descs(t, [2048], [16]), "VRAM")
     with pytest.raises(ag.NixlError) as e:
-        a.initialize_xfer("WRITE", ld, rd, "agent", notif_msg=b"n")
-    assert e.value.status == ag.NIXL_ERR_BACKEND
+        a.initialize_xfer("WRITE", ld, rd, "stranger")
+    assert e.value.status == ag.NIXL_ERR_NOT_FOUND
+
+
+def test_two_agents_in_one_process(cuda):
+    """Two agents with a HIP backend each exchange metadata by hand (get_agent_metadata /
+    add_remote_agent, the reference's wire format) and move VRAM between their regions: WRITE
+    with a notification that the target sees once the bytes have landed, READ, prepared lists,
+    a device memory view over the peer's region, removal of the peer (reference cases:
+    test/python/test_nixl_api.py:56-70,163-186,385-412; examples/cpp/nixl_example.cpp)."""
+    import torch
+    a = nixl_agent("initiator", nixl_agent_config(backends=()))
+    b = nixl_agent("target", nixl_agent_config(backends=()))
+    a.create_backend("HIP")
+    b.create_backend("HIP")
+    n = 8 << 20
+    g = torch.Generator(device="cpu").manual_seed(3)
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g).to(cuda)
+    dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
+    a.register_memory([src])
+    b.register_memory([dst])
+    torch.cuda.synchronize()
+    md = b.get_agent_metadata()
+    assert md.startswith(b"nixlSerDes|Agent") and b"HIP1:pid=" in md and b"bknd" in md
+    assert a.add_remote_agent(md) == "target"
+    assert b.add_remote_agent(a.get_agent_metadata()) == "initiator"
+    a.make_connection("target")
+    assert a.check_remote_metadata("target", a.get_xfer_descs(_descs(dst, [4096], [4096]), "VRAM"))
+    assert not a.check_remote_metadata("target", a.get_xfer_descs(_descs(src, [4096], [4096]), "VRAM"))
+
+    blk = 32768
+    idx = np.random.default_rng(5).permutation(n // blk)
+    offs_src = [int(i) * blk for i in range(n // blk)]
+    offs_dst = [int(i) * blk for i in idx]
+    lens = [blk] * (n // blk)
+    h = a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(src, offs_src, lens), "VRAM"),
+                          a.get_xfer_descs(_descs(dst, offs_dst, lens), "VRAM"), "target", b"blocks 0..255")
+    state = a.transfer(h)
+    while state == "PROC":
+        state = a.check_xfer_state(h)
+    assert state == "DONE"
+    # the message is queued when the initiator sees the transfer complete, so the bytes are there
+    assert b.get_new_notifs() == {"initiator": [b"blocks 0..255"]}
+    want = torch.empty_like(src).view(-1, blk)
+    want[torch.from_numpy(idx).to(cuda)] = src.view(-1, blk)
+    assert torch.equal(dst, want.view(-1))
+    a.release_xfer_handle(h)
+
+    # READ: the target's bytes come back into a scratch region of the initiator
+    back = torch.zeros(1 << 20, dtype=torch.uint8, device=cuda)
+    a.register_memory([back])
+    torch.cuda.synchronize()
+    h = a.initialize_xfer("READ", a.get_xfer_descs(_descs(back, [0], [1 << 20]), "VRAM"),
+                          a.get_xfer_descs(_descs(dst, [3 << 20], [1 << 20]), "VRAM"), "target")
+    assert a.transfer_and_wait(h) == "DONE"
+    assert torch.equal(back, dst[3 << 20:4 << 20])
+    assert b.get_new_notifs() == {}
+    a.release_xfer_handle(h)
+
+    # prepared lists on both sides, a subset of indices, and a released-in-flight notification
+    local = a.prep_xfer_dlist("NIXL_INIT_AGENT", a.get_xfer_descs(_descs(src, offs_src[:64], lens[:64]), "VRAM"))
+    remote = a.prep_xfer_dlist("target", a.get_xfer_descs(_descs(dst, offs_src[:64], lens[:64]), "VRAM"))
+    h = a.make_prepped_xfer("WRITE", local, list(range(0, 64, 2)), remote, list(range(1, 64, 2)), b"released early")
+    assert a.transfer(h) in ("PROC", "DONE")
+    a.release_xfer_handle(h)  # may still be running: the backend keeps it, and its message, until it has finished
+    torch.cuda.synchronize()
+    # the message leaves when the initiator's backend next looks at its released requests
+    assert a.get_new_notifs() == {}
+    assert b.check_remote_xfer_done("initiator", b"released")
+    for i in range(0, 64, 2):
+        assert torch.equal(dst[(i + 1) * blk:(i + 2) * blk], src[i * blk:(i + 1) * blk])
+
+    # standalone messages both ways, and to oneself
+    a.send_notif("target", b"ping")
+    b.send_notif("initiator", b"pong")
+    a.send_notif("initiator", b"note to self")
+    assert b.get_new_notifs() == {"initiator": [b"ping"]}
+    assert a.get_new_notifs() == {"target": [b"pong"], "initiator": [b"note to self"]}
+
+    # a memory view over the peer's region resolves through the loaded metadata
+    view = a.prep_mem_view(a.get_remote_descs([(dst.data_ptr() + 256, 4096, 0, "target")], "VRAM"))
+    assert view
+    a.release_mem_view(view)
+
+    a.remove_remote_agent("target")
+    with pytest.raises(ag.NixlError) as e:
+        a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(src, [0], [64]), "VRAM"),
+                          a.get_xfer_descs(_descs(dst, [0], [64]), "VRAM"), "target")
+    assert e.value.status == ag.NIXL_ERR_NOT_FOUND
+    with pytest.raises(ag.NixlError):
+        a.send_notif("target", b"gone")
+    a.close()
+    b.close()
 
 
 def test_release_while_in_flight_does_not_block_or_corrupt(hip_agent, cuda):

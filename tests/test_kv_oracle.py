@@ -284,7 +284,7 @@ def test_api_behaviour_of_the_reference_python_tests(cpu_agent, oracle_plugin_di
     assert err.value.status == ag.NIXL_ERR_NOT_FOUND
     # what a real plugin answers
     assert "MEMCPY" in a.get_plugin_list()
-    assert a.get_plugin_mem_types("MEMCPY") == ["DRAM"] and a.get_plugin_params("MEMCPY") == {"threads": "1"}
+    assert a.get_plugin_mem_types("MEMCPY") == ["DRAM"] and a.get_plugin_params("MEMCPY") == {"threads": "1", "peer_agents": "0"}
     assert a.get_backend_mem_types("MEMCPY") == ["DRAM"]
     req = a.initialize_xfer("WRITE", l, r, a.name)
     assert a.query_xfer_backend(req) == "MEMCPY"
