@@ -4,7 +4,7 @@
 Mirrors the reference benchmark's flags, loops and report
 (benchmark/nixlbench/src/utils/utils.cpp:48-140 flags, :1295-1420 report;
 benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:1707-1831 transfer loop) for the one
-mode a local-only backend can run in: one agent whose transfers target itself, the way the
+mode that needs no second process: one agent whose transfers target itself, the way the
 reference runs storage backends (nixl_worker.cpp:1857).  For every block size from
 --start_block_size to --max_block_size (doubling) and every batch size from
 --start_batch_size to --max_batch_size (doubling): warm up, then run --num_iter transfers of
