@@ -5,7 +5,8 @@
 // workers, each with its own pair of views, :424-499; a remote list with a null-agent
 // placeholder and nixlGetPtr, :502-556), followed by what a loopback implementation has to
 // get right on its own: ragged and misaligned spans against memcpy on the host, counter
-// increments ordered after puts, and refusals that leave memory untouched.
+// increments ordered after puts, refusals that leave memory untouched, and the reference's
+// own arrangement of a sender and a receiver agent that exchange metadata.
 //
 // usage: mem_view_device_api; prints "OK" and exits 0 on success.
 #include <hip/hip_runtime.h>
@@ -483,6 +484,90 @@ main() {
         REQUIRE(agent.prepMemView(localList({reg}), mvh) == NIXL_SUCCESS && mvh);
         HIP_OK(hipFree(stray));
         std::printf("host refusals\n");
+    }
+
+    // 8. sender and receiver as two agents of this process, as in the reference's fixture
+    //    (single_write_test.cu:170-265: a backend each, metadata exchanged both ways); the
+    //    remote view names the receiver, the put lands in the receiver's registration, and a
+    //    counter in the receiver's memory tells it so
+    {
+        const std::string sender_name = "sender", receiver_name = "receiver";
+        nixlAgent sender(sender_name, nixlAgentConfig(false)), receiver(receiver_name, nixlAgentConfig(false));
+        nixlBackendH *sb = nullptr, *rb = nullptr;
+        REQUIRE(sender.createBackend("HIP", params, sb) == NIXL_SUCCESS);
+        REQUIRE(receiver.createBackend("HIP", params, rb) == NIXL_SUCCESS);
+        constexpr size_t size = 64 * 1024;
+        Buffer src = makeRegistered(sender, size), dst = makeRegistered(receiver, size), flag = makeRegistered(receiver, 64);
+        std::vector<uint32_t> host(size / 4);
+        for (size_t i = 0; i < host.size(); ++i)
+            host[i] = 0xDEADBEEF ^ static_cast<uint32_t>(i * 2654435761u);
+        HIP_OK(hipMemcpy(src.ptr, host.data(), size, hipMemcpyHostToDevice));
+
+        nixlMemViewH dst_mvh = nullptr;
+        // before the metadata is loaded the receiver is unknown to the sender
+        REQUIRE(sender.prepMemView(remoteList({dst, flag}, receiver_name), dst_mvh) == NIXL_ERR_NOT_FOUND);
+        nixl_blob_t md;
+        std::string loaded;
+        REQUIRE(receiver.getLocalMD(md) == NIXL_SUCCESS);
+        REQUIRE(sender.loadRemoteMD(md, loaded) == NIXL_SUCCESS && loaded == receiver_name);
+        REQUIRE(sender.getLocalMD(md) == NIXL_SUCCESS);
+        REQUIRE(receiver.loadRemoteMD(md, loaded) == NIXL_SUCCESS && loaded == sender_name);
+
+        nixlMemViewH src_mvh = nullptr;
+        REQUIRE(sender.prepMemView(localList({src}), src_mvh) == NIXL_SUCCESS);
+        REQUIRE(sender.prepMemView(remoteList({dst, flag}, receiver_name), dst_mvh) == NIXL_SUCCESS);
+        // the receiver's buffers are not the sender's own registrations
+        nixlMemViewH wrong = nullptr;
+        REQUIRE(sender.prepMemView(localList({dst}), wrong) == NIXL_ERR_NOT_FOUND);
+        REQUIRE(sender.prepMemView(remoteList({dst}, sender_name), wrong) == NIXL_ERR_NOT_FOUND);
+
+        HIP_OK(hipMemset(dev_out, 0, 2 * sizeof(int)));
+        HIP_OK(hipDeviceSynchronize());
+        constexpr unsigned groups = 4;
+        putThenCountKernel<<<groups, 256>>>(src_mvh, dst_mvh, size / groups, 1, dev_out);
+        HIP_OK(hipGetLastError());
+        HIP_OK(hipDeviceSynchronize());
+        int bad = -1;
+        HIP_OK(hipMemcpy(&bad, dev_out, sizeof(bad), hipMemcpyDeviceToHost));
+        REQUIRE(bad == 0);
+        uint64_t count = 0;
+        HIP_OK(hipMemcpy(&count, flag.ptr, sizeof(count), hipMemcpyDeviceToHost));
+        REQUIRE(count == groups);
+        std::vector<uint32_t> got(size / 4);
+        HIP_OK(hipMemcpy(got.data(), dst.ptr, size, hipMemcpyDeviceToHost));
+        REQUIRE(got == host);
+
+        // host-initiated transfer between the same two agents, with a notification
+        HIP_OK(hipMemset(dst.ptr, 0, size));
+        HIP_OK(hipDeviceSynchronize());
+        nixl_xfer_dlist_t l(VRAM_SEG), r(VRAM_SEG);
+        l.addDesc(nixlBasicDesc(reinterpret_cast<uintptr_t>(src.ptr), size, 0));
+        r.addDesc(nixlBasicDesc(reinterpret_cast<uintptr_t>(dst.ptr), size, 0));
+        nixl_opt_args_t with_notif;
+        with_notif.notifMsg = "landed";
+        with_notif.hasNotif = true;
+        nixlXferReqH *req = nullptr;
+        REQUIRE(sender.createXferReq(NIXL_WRITE, l, r, receiver_name, req, &with_notif) == NIXL_SUCCESS);
+        nixl_status_t st = sender.postXferReq(req);
+        while (st == NIXL_IN_PROG)
+            st = sender.getXferStatus(req);
+        REQUIRE(st == NIXL_SUCCESS);
+        nixl_notifs_t notifs;
+        REQUIRE(receiver.getNotifs(notifs) == NIXL_SUCCESS);
+        REQUIRE(notifs.size() == 1 && notifs[sender_name].size() == 1 && notifs[sender_name][0] == "landed");
+        HIP_OK(hipMemcpy(got.data(), dst.ptr, size, hipMemcpyDeviceToHost));
+        REQUIRE(got == host);
+        REQUIRE(sender.releaseXferReq(req) == NIXL_SUCCESS);
+
+        // once the receiver is invalidated, no new view of it can be made
+        sender.releaseMemView(dst_mvh);
+        sender.releaseMemView(src_mvh);
+        REQUIRE(sender.invalidateRemoteMD(receiver_name) == NIXL_SUCCESS);
+        REQUIRE(sender.prepMemView(remoteList({dst}, receiver_name), dst_mvh) == NIXL_ERR_NOT_FOUND);
+        dropRegistered(sender, src);
+        dropRegistered(receiver, dst);
+        dropRegistered(receiver, flag);
+        std::printf("two agents\n");
     }
 
     HIP_OK(hipFree(dev_out));
