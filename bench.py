@@ -210,6 +210,37 @@ def run_calibration_copy():
     torch.cuda.empty_cache()
 
 
+def run_ep_cpu_baseline(seconds=10.0, threads=1):
+    """Scalar CPU restatement of the low-latency kernels (the oracle) on `threads` host
+    threads, on a bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8,
+    fp8."""
+    from oracle import ep_oracle as eo
+    R, T, H, K, E, M = 4, 128, 7168, 8, 32, 128
+    rng = np.random.default_rng(4)
+    x = eo.f32_to_bf16(rng.standard_normal((R, T, H)).astype(np.float32))
+    logits = rng.standard_normal((R * T, E)).astype(np.float32)
+    topk, w = eo.router(logits, K)
+    topk, w = topk.reshape(R, T, K), w.reshape(R, T, K)
+    t0 = time.perf_counter()
+    n = 0
+    d_us, c_us = [], []
+    while time.perf_counter() - t0 < seconds or n < 2:
+        a = time.perf_counter()
+        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True, threads=threads)
+        b = time.perf_counter()
+        y = np.zeros((R, E // R, R * M, H), np.uint16)
+        c = time.perf_counter()
+        eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M, threads=threads)
+        d = time.perf_counter()
+        d_us.append((b - a) * 1e6)
+        c_us.append((d - c) * 1e6)
+        n += 1
+    return {"dispatch_us": round(float(np.mean(d_us)), 1), "combine_us": round(float(np.mean(c_us)), 1),
+            "cores": threads, "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
+                      "(1/8 of the GPU workload's tokens)"}
+
+
 def run_cpu_baseline(seconds=12.0, threads=1):
     """Reference-shaped CPU path: one agent, loopback, DRAM->DRAM, one memcpy per descriptor
     (the semantics of the reference's UCX loopback puts, src/plugins/ucx/ucx_backend.cpp:
@@ -325,6 +356,11 @@ def main():
     if not args.no_ep:
         from nixl_amd import ep_bench
         line["ep"] = ep_bench.run(args)
+        if not args.no_cpu_baseline:
+            line["ep"]["cpu_baseline"] = run_ep_cpu_baseline()
+            many = min(16, os.cpu_count() or 1)
+            if many > 1:
+                line["ep"]["cpu_baseline"]["all_cores"] = run_ep_cpu_baseline(seconds=4.0, threads=many)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline()
         # the same path with the descriptor list split over the box's CPU share, reported beside

@@ -7,9 +7,6 @@ cache), warm-ups first, first sample dropped, average / min / max reported.  Byt
 are the algorithmic ones: each input row read once, each output row written once
 (reference formula for the low-latency mode: tests/elastic/elastic.py:424-432).
 """
-import os
-import time
-
 import numpy as np
 import torch
 
@@ -154,45 +151,9 @@ def run_normal(dev, warmup=5, iters=20):
     }
 
 
-def run_cpu_baseline(seconds=10.0, threads=1):
-    """Scalar CPU restatement of the low-latency kernels (the oracle) on `threads` host
-    threads, on a bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8,
-    fp8."""
-    from oracle import ep_oracle as eo
-    R, T, H, K, E, M = 4, 128, 7168, 8, 32, 128
-    rng = np.random.default_rng(4)
-    x = eo.f32_to_bf16(rng.standard_normal((R, T, H)).astype(np.float32))
-    logits = rng.standard_normal((R * T, E)).astype(np.float32)
-    topk, w = eo.router(logits, K)
-    topk, w = topk.reshape(R, T, K), w.reshape(R, T, K)
-    t0 = time.perf_counter()
-    n = 0
-    d_us, c_us = [], []
-    while time.perf_counter() - t0 < seconds or n < 2:
-        a = time.perf_counter()
-        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True, threads=threads)
-        b = time.perf_counter()
-        y = np.zeros((R, E // R, R * M, H), np.uint16)
-        c = time.perf_counter()
-        eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M, threads=threads)
-        d = time.perf_counter()
-        d_us.append((b - a) * 1e6)
-        c_us.append((d - c) * 1e6)
-        n += 1
-    return {"dispatch_us": round(float(np.mean(d_us)), 1), "combine_us": round(float(np.mean(c_us)), 1),
-            "cores": threads, "kind": "port", "host_cpus": os.cpu_count(),
-            "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
-                      "(1/8 of the GPU workload's tokens)"}
-
-
 def run(args):
     dev = torch.device("cuda:0")
     warmup, iters = getattr(args, "ep_warmup", 20), getattr(args, "ep_iters", 50)
     out = {"low_latency": run_low_latency(dev, warmup, iters),
            "normal": run_normal(dev, max(warmup // 4, 1), max(iters // 2, 1))}
-    if not getattr(args, "no_cpu_baseline", False):
-        out["cpu_baseline"] = run_cpu_baseline()
-        many = min(16, os.cpu_count() or 1)
-        if many > 1:
-            out["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=4.0, threads=many)
     return out
