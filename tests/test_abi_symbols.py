@@ -91,3 +91,23 @@ def test_agent_members_exported():
     syms = _exported("libnixl_amd_agent.so", demangle=True)
     missing = [m for m in sorted(members) if f"nixlAgent::{m}(" not in syms]
     assert not missing, missing
+
+
+def test_product_code_never_reaches_for_the_cpu_oracle():
+    """The oracle is test infrastructure: nothing in the package imports it, no product source
+    names it, and no product library links it."""
+    pkg = os.path.join(ROOT, "nixl_amd")
+    offenders = []
+    for base, _dirs, files in os.walk(pkg):
+        if "__pycache__" in base or os.path.join(pkg, "lib") in base:
+            continue
+        for f in files:
+            if not f.endswith((".py", ".cpp", ".h", ".hip", "Makefile")):
+                continue
+            text = open(os.path.join(base, f), errors="replace").read()
+            if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "liboracle" in text or "oracle/" in text:
+                offenders.append(os.path.join(base, f))
+    assert not offenders, offenders
+    for lib in ("libnixl_amd_kernels.so", "libnixl_amd_agent.so", os.path.join("plugins", "libplugin_HIP.so")):
+        out = subprocess.run(["readelf", "-d", os.path.join(LIB, lib)], check=True, capture_output=True, text=True).stdout
+        assert "oracle" not in out.lower() and "MEMCPY" not in out, lib
