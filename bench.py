@@ -90,17 +90,24 @@ def run_kv(args):
     prep_ms = (time.perf_counter() - t0) * 1e3
     assert gather.desc_count() == (n_desc, n_desc * blk)
 
+    post_us, xfer_us = [], []  # wall clock of the post call and of post -> completion, as nixlbench splits them
+
     def step(events=None):
         for req in (gather, scatter):
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
+            w0 = time.perf_counter()
             state = agent.transfer(req)
+            w1 = time.perf_counter()
             if events is not None:
                 e1.record(stream)
                 events.append((e0, e1))
             while state == "PROC":
                 state = agent.check_xfer_state(req)
+            if events is not None:
+                post_us.append((w1 - w0) * 1e6)
+                xfer_us.append((time.perf_counter() - w0) * 1e6)
             if state != "DONE":
                 raise RuntimeError(f"transfer ended in state {state}")
 
@@ -134,10 +141,14 @@ def run_kv(args):
                      "traffic": MEASURED_TRAFFIC_BYTES.get((n_sel, pool_blocks, blk)),
                      "kernel": "copy_uniform_kernel<1,true,1>",
                      "avg_launch_ms": round(avg_launch_ms, 4),
+                     "min_launch_ms": round(float(np.min(kernel_ms)), 4),
+                     "p99_launch_ms": round(float(np.percentile(kernel_ms, 99)), 4),
                      "gather_ms": round(float(np.mean(kernel_ms[0::2])), 4),
                      "scatter_ms": round(float(np.mean(kernel_ms[1::2])), 4),
                      "algorithmic_bytes_per_launch": algorithmic_bytes_per_launch},
-        "kv": {"descriptors_per_request": n_desc, "descriptor_bytes": blk, "prep_ms": round(prep_ms, 2)},
+        "kv": {"descriptors_per_request": n_desc, "descriptor_bytes": blk, "prep_ms": round(prep_ms, 2),
+               "post_us": {"avg": round(float(np.mean(post_us)), 1), "p99": round(float(np.percentile(post_us, 99)), 1)},
+               "xfer_us": {"avg": round(float(np.mean(xfer_us)), 1), "p99": round(float(np.percentile(xfer_us, 99)), 1)}},
     }
     for h in (gather, scatter, h_src, h_stg_r, h_stg_l, h_dst):
         h.release()
@@ -239,6 +250,41 @@ def run_ep_cpu_baseline(seconds=10.0, threads=1):
             "cores": threads, "kind": "port", "host_cpus": os.cpu_count(),
             "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
                       "(1/8 of the GPU workload's tokens)"}
+
+
+def run_posix_analogue(seconds=4.0):
+    """What the reference's POSIX backend does with a descriptor list, without the plugin: one
+    pwrite per descriptor from DRAM into a file, then one pread per descriptor back
+    (src/plugins/posix/posix_backend.cpp: local DRAM, remote FILE only).  The file lives in
+    /dev/shm, so this is memory to memory through the kernel's file layer: a labelled
+    substitute, not a KV-to-KV copy.  4096 descriptors x 16 KiB (BASELINE config 1)."""
+    n, blk = 4096, 16384
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, n * blk, dtype=np.uint8)
+    back = np.zeros_like(src)
+    order = rng.permutation(n)
+    path = f"/dev/shm/nixl_amd_bench_{os.getpid()}.bin"
+    fd = os.open(path, os.O_RDWR | os.O_CREAT | os.O_TRUNC, 0o600)
+    try:
+        os.ftruncate(fd, n * blk)
+        src_v, back_v = memoryview(src), memoryview(back)
+        t0 = time.perf_counter()
+        rounds = 0
+        while time.perf_counter() - t0 < seconds or rounds == 0:
+            for i, j in enumerate(order):
+                os.pwrite(fd, src_v[i * blk:(i + 1) * blk], int(j) * blk)
+            for i, j in enumerate(order):
+                os.preadv(fd, [back_v[i * blk:(i + 1) * blk]], int(j) * blk)
+            rounds += 1
+        wall = time.perf_counter() - t0
+        if not np.array_equal(src, back):
+            raise RuntimeError("POSIX analogue: bytes read back differ")
+    finally:
+        os.close(fd)
+        os.unlink(path)
+    return {"value": round(2 * n * blk * rounds / wall / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{rounds} rounds of {n} x pwrite then {n} x pread of {blk} B, file in /dev/shm, {wall:.1f} s; "
+                      "Python call overhead per descriptor included"}
 
 
 def run_cpu_baseline(seconds=12.0, threads=1):
@@ -367,6 +413,10 @@ def main():
         many = min(16, os.cpu_count() or 1)
         if many > 1:
             line["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=5.0, threads=many)
+        line["cpu_baseline"]["posix_path_analogue"] = run_posix_analogue()
+        # the reference's own loopback needs libucp, which this image does not ship
+        import ctypes.util
+        line["cpu_baseline"]["libucp"] = ctypes.util.find_library("ucp") or "absent"
     print(json.dumps(line))
 
 
