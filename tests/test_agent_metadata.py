@@ -253,3 +253,15 @@ def test_partial_metadata_then_the_rest(two_agents):
     _wait(a, h)
     a.release_xfer_handle(h)
     assert np.array_equal(r2, src[4096:])
+
+
+def test_two_peers_through_the_cpp_api(oracle_plugin_dir):
+    """The same exchange through nixlAgent from C++ (tests/cpp/agent_two_peers_check.cpp, the
+    flow of the reference's examples/cpp/nixl_example.cpp), three generations of agents."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "agent_two_peers_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe, oracle_plugin_dir], capture_output=True, text=True, timeout=60)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
