@@ -53,6 +53,19 @@ def _check(rc, what):
         raise EPError(f"{what}: {_lib.kernels_error()} (status {rc})")
 
 
+class Config:
+    """The reference's normal-mode tuning record (nixl_ep_cpp.Config: SM count plus chunk sizes
+    of its NVLink and RDMA staging queues).  There are no staging queues here; only num_sms
+    keeps a meaning: num_sms / 2 is the number of channels the per-channel prefix matrix of
+    the dispatch handle is cut into (csrc/nixl_ep.cpp:630)."""
+
+    def __init__(self, num_sms, *chunk_sizes):
+        if num_sms <= 0 or num_sms % 2:
+            raise EPError("the SM count must be positive and even")
+        self.num_sms = int(num_sms)
+        self.chunk_sizes = tuple(chunk_sizes)  # accepted, unused
+
+
 class DispatchHandle(tuple):
     """The reference's dispatch handle (src_info, layout_range, num_max_dispatch_tokens_per_rank,
     hidden) (nixl_ep/buffer.py:415-420), plus the row map the dispatch kernel recorded, which
@@ -70,6 +83,26 @@ class Buffer:
     """
 
     num_sms = 20  # kept for API parity (buffer.py:57); the kernels size their own grids
+
+    num_sms = 20  # reference default (buffer.py:54); see Config
+
+    @staticmethod
+    def set_num_sms(new_num_sms):
+        """Reference: buffer.py:116-126."""
+        if new_num_sms <= 0 or new_num_sms % 2:
+            raise EPError("the SM count must be positive and even")
+        Buffer.num_sms = int(new_num_sms)
+
+    @staticmethod
+    def get_dispatch_config(num_ranks):
+        """Reference: buffer.py:221-247 (a table of queue chunk sizes per rank count, which
+        have no counterpart here)."""
+        return Config(Buffer.num_sms)
+
+    @staticmethod
+    def get_combine_config(num_ranks):
+        """Reference: buffer.py:249-275."""
+        return Config(Buffer.num_sms)
 
     def __init__(self, num_ranks, low_latency_mode=True, device="cuda:0"):
         self.num_ranks = int(num_ranks)
@@ -334,8 +367,8 @@ class Buffer:
 
     def ht_dispatch(self, x, handle=None, num_tokens_per_rank=None, num_tokens_per_rdma_rank=None,
                     is_token_in_rank=None, num_tokens_per_expert=None, topk_idx=None, topk_weights=None,
-                    expert_alignment=1, num_channels=10, previous_event=None, async_finish=False,
-                    allocate_on_comm_stream=False):
+                    expert_alignment=1, num_channels=None, previous_event=None, async_finish=False,
+                    allocate_on_comm_stream=False, config=None):
         """Reference: buffer.py:526-660, csrc/nixl_ep.cpp:615-898 (bf16 rows).
 
         x [R, T, H]; the layout tensors come from get_dispatch_layout.  Returns
@@ -361,6 +394,8 @@ class Buffer:
             return recv_x, None, None, None, None, EventOverlap(None)
         if num_tokens_per_rank is None or is_token_in_rank is None or num_tokens_per_expert is None or topk_idx is None:
             raise EPError("ht_dispatch needs either a handle or the tensors of get_dispatch_layout and topk_idx")
+        if num_channels is None:  # as the reference derives it (csrc/nixl_ep.cpp:630)
+            num_channels = (config or self.get_dispatch_config(R)).num_sms // 2
         K = topk_idx.shape[2]
         E = num_tokens_per_expert.shape[1]
         El = E // R
@@ -403,7 +438,7 @@ class Buffer:
         return recv_x, recv_topk_idx, recv_topk_weights, expert_count_list, out_handle, EventOverlap(None)
 
     def ht_combine(self, x, handle, topk_weights=None, bias=None, previous_event=None, async_finish=False,
-                   allocate_on_comm_stream=False):
+                   allocate_on_comm_stream=False, config=None):
         """Reference: buffer.py:663-714, csrc/nixl_ep.cpp:900-1028.  x [total, H] bf16 in the
         row order ht_dispatch produced.  Returns (combined_x [R, T, H], combined_topk_weights
         [R, T, K] or None, event)."""

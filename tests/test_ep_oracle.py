@@ -506,3 +506,18 @@ def test_ll_combine_logfmt_is_the_sum_of_decoded_rows():
             for k in range(K):
                 acc = (dec.astype(np.float64) * np.float64(w[r, t, k]) + acc).astype(np.float32)
             assert np.array_equal(out[r, t], eo.f32_to_bf16(acc)) or np.max(np.abs(eo.bf16_to_f32(out[r, t]) - acc)) < 1e-2
+
+
+def test_normal_mode_config_shims():
+    """Config / set_num_sms / get_*_config of the reference (buffer.py:54,116-126,221-275): only
+    the SM count keeps a meaning here (channels = num_sms / 2, csrc/nixl_ep.cpp:630)."""
+    from nixl_amd import ep
+    assert ep.Buffer.num_sms == 20 and ep.Buffer.get_dispatch_config(8).num_sms == 20
+    ep.Buffer.set_num_sms(24)
+    try:
+        assert ep.Buffer.get_combine_config(32).num_sms == 24
+        with pytest.raises(ep.EPError):
+            ep.Buffer.set_num_sms(7)
+        assert ep.Config(24, 6, 256, 6, 128).chunk_sizes == (6, 256, 6, 128)
+    finally:
+        ep.Buffer.set_num_sms(20)
