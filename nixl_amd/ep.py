@@ -59,11 +59,14 @@ class Config:
     keeps a meaning: num_sms / 2 is the number of channels the per-channel prefix matrix of
     the dispatch handle is cut into (csrc/nixl_ep.cpp:630)."""
 
-    def __init__(self, num_sms, *chunk_sizes):
+    def __init__(self, num_sms=20, num_max_nvl_chunked_send_tokens=6, num_max_nvl_chunked_recv_tokens=256,
+                 num_max_rdma_chunked_send_tokens=6, num_max_rdma_chunked_recv_tokens=256):
+        # names and defaults of csrc/nixl_ep.cpp:1502-1506
         if num_sms <= 0 or num_sms % 2:
             raise EPError("the SM count must be positive and even")
         self.num_sms = int(num_sms)
-        self.chunk_sizes = tuple(chunk_sizes)  # accepted, unused
+        self.chunk_sizes = (num_max_nvl_chunked_send_tokens, num_max_nvl_chunked_recv_tokens,
+                            num_max_rdma_chunked_send_tokens, num_max_rdma_chunked_recv_tokens)  # accepted, unused
 
 
 class DispatchHandle(tuple):
@@ -118,6 +121,23 @@ class Buffer:
         self.cpu_timeout_secs = 100  # NUM_CPU_TIMEOUT_SECS, csrc/kernels/configs.cuh
 
     # -- life cycle and sizing helpers kept for callers written against the reference ------
+    def is_available(self):
+        """Reference: csrc/nixl_ep.cpp Buffer::is_available: usable until destroy()."""
+        return self.mask_buffer is not None
+
+    def get_local_device_id(self):
+        return self.device.index or 0
+
+    # one GPU holds every rank: a single "RDMA rank" (node), reference csrc/nixl_ep.cpp:84-101
+    def get_num_rdma_ranks(self):
+        return 1
+
+    def get_rdma_rank(self):
+        return 0
+
+    def get_root_rdma_rank(self, global_):
+        return 0
+
     def destroy(self):
         """Reference: buffer.py:103-110.  Drops the device buffers this object owns."""
         self.mask_buffer = None
