@@ -17,7 +17,7 @@
 //       with wave-uniform base addresses — no search, no LDS, few registers;
 //     * any other chunk (it crosses descriptor boundaries, or it is the short last chunk)
 //       is listed by chunk index in `mixed[]`; the mixed kernel stages the descriptors the
-//       chunk touches (span[c] = {first, last}; src[j], dst[j], prefix[j] = first unit of
+//       chunk touches (span[m] = {first, last} for the m-th listed chunk; src[j], dst[j], prefix[j] = first unit of
 //       descriptor j, prefix[n] = total) in a per-wave LDS slice and walks them.
 //   Descriptors that are not 16-byte aligned in src, dst and len are cut into byte-range
 //   work items handled by a third, byte-exact kernel.
@@ -49,7 +49,7 @@ struct MixedArgs {
     const uint64_t *src; // [n]
     const uint64_t *dst; // [n]
     const uint64_t *prefix; // [n + 1], units
-    const uint2 *span; // [n_chunks], {first desc, last desc}
+    const uint2 *span; // [n_mixed], {first desc, last desc} of the m-th mixed chunk
     const uint32_t *chunks; // [n_mixed] chunk indices
     uint64_t total_units;
     uint32_t n_mixed;
@@ -172,7 +172,7 @@ copy_mixed_kernel(MixedArgs a) {
 
     for (uint32_t m = uniform(blockIdx.x * kMixedWaves + wave); m < a.n_mixed; m += n_waves) {
         const uint32_t c = uniform(a.chunks[m]);
-        const uint2 sp = a.span[c];
+        const uint2 sp = a.span[m];
         const uint32_t j0 = uniform(sp.x);
         const uint32_t j1 = uniform(sp.y);
         const uint64_t u0 = static_cast<uint64_t>(c) * kChunkUnits;
@@ -436,55 +436,61 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: request too large for 32-bit chunk index");
     const uint32_t n_chunks = static_cast<uint32_t>(n_chunks64);
 
-    std::vector<uint2> span(n_chunks);
-    std::vector<UniformRec> uni;
-    std::vector<uint32_t> mixed;
-    uni.reserve(n_chunks);
-    // Runs of consecutive uniform chunks inside one descriptor: if all runs have the same
-    // length L, one record per run is kept and the kernel derives the rest.
-    uint32_t run_len = 0, common_run = 0;
-    bool runs_equal = true;
-    size_t run_desc = ~size_t(0);
-    auto close_run = [&]() {
-        if (run_len == 0) return;
-        if (common_run == 0)
-            common_run = run_len;
-        else if (common_run != run_len)
-            runs_equal = false;
-        run_len = 0;
+    // Walk the stream by descriptor: the chunks that lie wholly inside one descriptor form a
+    // run of uniform chunks (one step for the whole run, however long); a chunk that holds a
+    // descriptor boundary, or the short last chunk, is "mixed" and remembers the first and
+    // last descriptor it touches.  If all runs have the same length L, one record per run is
+    // kept and the kernel derives the rest; otherwise every uniform chunk gets its record.
+    struct Run {
+        uint64_t src, dst;
+        uint32_t chunks;
     };
+    std::vector<Run> runs;
+    std::vector<uint32_t> mixed;
+    std::vector<uint2> span; // per mixed chunk: first and last descriptor
+    uint32_t n_uniform_chunks = 0, common_run = 0;
+    bool runs_equal = true;
     {
         size_t j = 0;
-        for (uint32_t c = 0; c < n_chunks; ++c) {
+        for (uint32_t c = 0; c < n_chunks;) {
             const uint64_t first = static_cast<uint64_t>(c) * chunk_units;
-            const uint64_t last = std::min(units, first + chunk_units) - 1;
             while (vprefix[j + 1] <= first)
                 ++j;
+            const uint64_t inside = (vprefix[j + 1] - first) / chunk_units; // whole chunks left in descriptor j
+            if (inside > 0) {
+                const uint32_t len = static_cast<uint32_t>(inside);
+                const uint64_t off = (first - vprefix[j]) * 16u;
+                runs.push_back(Run{vsrc[j] + off, vdst[j] + off, len});
+                if (common_run == 0)
+                    common_run = len;
+                else if (common_run != len)
+                    runs_equal = false;
+                n_uniform_chunks += len;
+                c += len;
+                continue;
+            }
+            const uint64_t last = std::min(units, first + chunk_units) - 1;
             size_t jl = j;
             while (vprefix[jl + 1] <= last)
                 ++jl;
-            span[c] = make_uint2(static_cast<uint32_t>(j), static_cast<uint32_t>(jl));
-            if (j == jl && last - first + 1 == chunk_units) {
-                const uint64_t off = (first - vprefix[j]) * 16u;
-                if (run_len && run_desc != j) close_run();
-                run_desc = j;
-                ++run_len;
-                uni.push_back(UniformRec{vsrc[j] + off, vdst[j] + off});
-            } else {
-                close_run();
-                mixed.push_back(c);
-            }
+            mixed.push_back(c);
+            span.push_back(make_uint2(static_cast<uint32_t>(j), static_cast<uint32_t>(jl)));
+            ++c;
         }
-        close_run();
     }
-    const uint32_t n_uniform_chunks = static_cast<uint32_t>(uni.size());
+    std::vector<UniformRec> uni;
     uint32_t chunks_per_rec = 1;
     if (runs_equal && common_run > 1) {
         chunks_per_rec = common_run;
-        size_t w = 0;
-        for (size_t i = 0; i < uni.size(); i += common_run)
-            uni[w++] = uni[i];
-        uni.resize(w);
+        uni.reserve(runs.size());
+        for (const Run &r : runs)
+            uni.push_back(UniformRec{r.src, r.dst});
+    } else {
+        uni.reserve(n_uniform_chunks);
+        const uint64_t chunk_bytes = chunk_units * 16u;
+        for (const Run &r : runs)
+            for (uint32_t k = 0; k < r.chunks; ++k)
+                uni.push_back(UniformRec{r.src + k * chunk_bytes, r.dst + k * chunk_bytes});
     }
 
     // ---- one device arena for all plan arrays --------------------------------------
@@ -495,7 +501,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     const size_t off_dst = off_src + (need_desc_arrays ? align256(nv * 8) : 0);
     const size_t off_prefix = off_dst + (need_desc_arrays ? align256(nv * 8) : 0);
     const size_t off_span = off_prefix + (need_desc_arrays ? align256((nv + 1) * 8) : 0);
-    const size_t off_mixed = off_span + (need_desc_arrays ? align256(size_t(n_chunks) * sizeof(uint2)) : 0);
+    const size_t off_mixed = off_span + (need_desc_arrays ? align256(span.size() * sizeof(uint2)) : 0);
     const size_t off_pieces = off_mixed + align256(mixed.size() * sizeof(uint32_t));
     const size_t off_items = off_pieces + align256(pieces.size() * sizeof(PieceRec));
     const size_t total = off_items + align256(items.size() * sizeof(GenericItem));
@@ -515,7 +521,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             std::memcpy(host.data() + off_src, vsrc.data(), nv * 8);
             std::memcpy(host.data() + off_dst, vdst.data(), nv * 8);
             std::memcpy(host.data() + off_prefix, vprefix.data(), (nv + 1) * 8);
-            std::memcpy(host.data() + off_span, span.data(), size_t(n_chunks) * sizeof(uint2));
+            std::memcpy(host.data() + off_span, span.data(), span.size() * sizeof(uint2));
             std::memcpy(host.data() + off_mixed, mixed.data(), mixed.size() * sizeof(uint32_t));
         }
         if (!pieces.empty()) std::memcpy(host.data() + off_pieces, pieces.data(), pieces.size() * sizeof(PieceRec));
