@@ -8,6 +8,8 @@
 // be built with the host sanitizers.
 //
 // usage: agent_two_peers_check <directory holding libplugin_MEMCPY.so>; prints "OK".
+#include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -67,6 +69,19 @@ main(int argc, char **argv) {
         REQUIRE(a.createBackend("MEMCPY", params, ba) == NIXL_SUCCESS);
         REQUIRE(b.createBackend("MEMCPY", params, bb) == NIXL_SUCCESS);
 
+        if (round == 2) {
+            // metadata of agents that have registered nothing yet loads, and is dropped again
+            // (test/gtest/unit/agent/agent.cpp:353-380)
+            nixl_blob_t bare;
+            std::string who;
+            REQUIRE(b.getLocalMD(bare) == NIXL_SUCCESS && !bare.empty());
+            REQUIRE(a.loadRemoteMD(bare, who) == NIXL_SUCCESS && who == "B");
+            REQUIRE(a.genNotif("B", "early bird") == NIXL_SUCCESS); // agent.cpp:517-542
+            nixl_notifs_t early;
+            REQUIRE(b.getNotifs(early) == NIXL_SUCCESS && early["A"] == std::vector<nixl_blob_t>{"early bird"});
+            REQUIRE(a.invalidateRemoteMD("B") == NIXL_SUCCESS);
+        }
+
         std::vector<uint8_t> src(1 << 16), dst(1 << 16, 0), extra(4096, 0);
         std::iota(src.begin(), src.end(), static_cast<uint8_t>(round));
         REQUIRE(a.registerMem(regList(src)) == NIXL_SUCCESS);
@@ -98,6 +113,8 @@ main(int argc, char **argv) {
         const std::vector<std::pair<size_t, size_t>> from = {{0, 1000}, {4096, 4096}, {60000, 5536}};
         const std::vector<std::pair<size_t, size_t>> to = {{6000, 1000}, {20000, 4096}, {0, 5536}};
         REQUIRE(a.createXferReq(NIXL_WRITE, spans(src, from), spans(dst, to), "B", req, &with_notif) == NIXL_SUCCESS);
+        nixlBackendH *used = nullptr;
+        REQUIRE(a.queryXferBackend(req, used) == NIXL_SUCCESS && used == ba); // agent.cpp:544-584
         nixl_notifs_t notifs;
         REQUIRE(b.getNotifs(notifs) == NIXL_SUCCESS && notifs.empty());
         REQUIRE(runToCompletion(a, req) == NIXL_SUCCESS);
@@ -107,8 +124,7 @@ main(int argc, char **argv) {
         REQUIRE(notifs.size() == 1 && notifs["A"] == std::vector<nixl_blob_t>{"written"});
         // a repost repeats the message; one passed to the post replaces it
         nixl_opt_args_t other;
-        other.notifMsg = std::string("bin\0ary", 7);
-        other.hasNotif = true;
+        other.notif = std::string("bin\0ary", 7); // the optional form, as agent.cpp:413 sets it
         REQUIRE(runToCompletion(a, req) == NIXL_SUCCESS);
         REQUIRE(runToCompletion(a, req, &other) == NIXL_SUCCESS);
         REQUIRE(b.getNotifs(notifs) == NIXL_SUCCESS);
@@ -158,6 +174,38 @@ main(int argc, char **argv) {
         REQUIRE(a.releaseXferReq(req) == NIXL_SUCCESS);
         REQUIRE(a.makeConnection("B") == NIXL_ERR_NOT_FOUND);
         REQUIRE(a.genNotif("B", "gone") == NIXL_ERR_NOT_FOUND);
+        // registering and deregistering a pool of regions over and over neither fails nor slows
+        // down (agent.cpp:273-336: 128 regions, 64 cycles between two timed ones, ratio <= 2;
+        // the bound here is looser because the test machine is shared)
+        if (round == 0) {
+            constexpr size_t kPool = 128;
+            std::vector<std::vector<uint8_t>> pool(kPool, std::vector<uint8_t>(256));
+            auto cycle = [&](int times) {
+                for (int r = 0; r < times; ++r) {
+                    for (auto &p : pool)
+                        REQUIRE(a.registerMem(regList(p)) == NIXL_SUCCESS);
+                    for (auto &p : pool)
+                        REQUIRE(a.deregisterMem(regList(p)) == NIXL_SUCCESS);
+                }
+            };
+            auto timed = [&]() {
+                const auto t0 = std::chrono::steady_clock::now();
+                cycle(1);
+                return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+            };
+            cycle(3);
+            double first = timed();
+            for (int i = 0; i < 2; ++i)
+                first = std::min(first, timed());
+            cycle(64);
+            double second = timed();
+            for (int i = 0; i < 2; ++i)
+                second = std::min(second, timed());
+            REQUIRE(second <= 4.0 * first && first <= 4.0 * second);
+            nixl_blob_t after;
+            REQUIRE(a.getLocalMD(after) == NIXL_SUCCESS);
+            REQUIRE(a.deregisterMem(regList(pool[0])) == NIXL_ERR_NOT_FOUND); // nothing of the pool is left
+        }
         // B still knows A and leaves it to its destructor to unload A's regions
         if (round == 1) REQUIRE(b.deregisterMem(regList(extra)) == NIXL_SUCCESS);
     }
