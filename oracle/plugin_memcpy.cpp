@@ -12,6 +12,8 @@
 // current bytes (test/unit/plugins/posix/nixl_posix_test.cpp:714-770), and a canary
 // check that bytes outside every destination range are untouched.
 //
+// Memory views (prepMemView) are tables in host memory, for tests of the agent's resolution.
+//
 // With the parameter peer_agents=1 the backend also reports supportsRemote() and
 // supportsNotif(): "remote" agents are other agents of the same process, whose registrations
 // are plain addresses here, and a notification is a push into the target engine's queue.
@@ -117,6 +119,26 @@ public:
         out = new memcpyMD(in.addr, in.len, /*of_peer=*/true);
         return NIXL_SUCCESS;
     }
+    // Memory views in host memory, in the layout the HIP backend builds on the device
+    // (include/nixl_amd_device.h: {magic, kind, count, (addr, len)...}), so that the agent's
+    // resolution of local and remote view lists can be checked on the CPU.
+    nixl_status_t prepMemView(const nixl_meta_dlist_t &descs, nixlMemViewH &mvh, const nixl_opt_b_args_t *) const override {
+        std::vector<std::pair<uint64_t, uint64_t>> entries;
+        for (const nixlMetaDesc &d : descs) {
+            if (!d.metadataP) return NIXL_ERR_INVALID_PARAM;
+            entries.emplace_back(d.addr, d.len);
+        }
+        return buildView(entries, 0, mvh);
+    }
+    nixl_status_t prepMemView(const nixl_remote_meta_dlist_t &descs, nixlMemViewH &mvh,
+                              const nixl_opt_b_args_t *) const override {
+        std::vector<std::pair<uint64_t, uint64_t>> entries;
+        for (const nixlRemoteMetaDesc &d : descs)
+            entries.emplace_back(d.metadataP ? d.addr : 0, d.metadataP ? d.len : 0); // placeholder: no registration
+        return buildView(entries, 1, mvh);
+    }
+    void releaseMemView(nixlMemViewH mvh) const override { delete[] static_cast<uint64_t *>(mvh); }
+
     nixl_status_t genNotif(const std::string &agent, const std::string &msg) const override {
         std::lock_guard<std::mutex> registry(g_registryMutex);
         const auto it = g_registry.find(agent);
@@ -182,6 +204,20 @@ public:
     }
 
 private:
+    static nixl_status_t buildView(const std::vector<std::pair<uint64_t, uint64_t>> &entries, uint32_t kind,
+                                   nixlMemViewH &mvh) {
+        if (entries.empty()) return NIXL_ERR_INVALID_PARAM;
+        auto *words = new uint64_t[2 + 2 * entries.size()];
+        words[0] = 0x5649584cull | (static_cast<uint64_t>(kind) << 32);
+        words[1] = entries.size();
+        for (size_t i = 0; i < entries.size(); ++i) {
+            words[2 + 2 * i] = entries[i].first;
+            words[3 + 2 * i] = entries[i].second;
+        }
+        mvh = words;
+        return NIXL_SUCCESS;
+    }
+
     bool known(const std::string &agent) const {
         if (agent == localAgent) return true;
         std::lock_guard<std::mutex> lock(mutex_);

@@ -265,3 +265,45 @@ def test_two_peers_through_the_cpp_api(oracle_plugin_dir):
         pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
     proc = subprocess.run([exe, oracle_plugin_dir], capture_output=True, text=True, timeout=60)
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
+def test_memory_view_lists_resolve_through_the_agent(two_agents):
+    """prepMemView on the CPU: the agent resolves a local list against its own registrations
+    and a remote list against the loaded metadata of each named peer, keeps placeholders, and
+    refuses what it cannot resolve (src/core/nixl_agent.cpp:1906-2036; the reference's unit
+    test PrepMemViewRemoteDRAM, test/gtest/unit/agent/agent.cpp:436-448).  The memcpy backend
+    builds the table in host memory in the HIP backend's layout, which is read back here."""
+    import ctypes
+    a, b = two_agents
+    mine, theirs = np.zeros(8192, np.uint8), np.zeros(4096, np.uint8)
+    _reg(a, mine)
+    _reg(b, theirs)
+
+    def table(mvh, n):
+        return list((ctypes.c_uint64 * (2 + 2 * n)).from_address(mvh))
+
+    magic = 0x5649584C
+    lv = a.prep_mem_view(_descs(a, mine, [0, 4096], [4096, 100]))
+    assert table(lv, 2) == [magic, 2, mine.ctypes.data, 4096, mine.ctypes.data + 4096, 100]
+    # the peer is unknown until its metadata is loaded
+    remote = a.get_remote_descs([(theirs.ctypes.data + 16, 64, 0, "beta"), (0, 0, 0, None),
+                                 (mine.ctypes.data, 8192, 0, "alpha")], "DRAM")
+    with pytest.raises(ag.NixlError) as e:
+        a.prep_mem_view(remote)
+    assert e.value.status == ag.NIXL_ERR_NOT_FOUND
+    a.add_remote_agent(b.get_agent_metadata())
+    rv = a.prep_mem_view(remote)
+    assert table(rv, 3) == [magic | (1 << 32), 3, theirs.ctypes.data + 16, 64, 0, 0, mine.ctypes.data, 8192]
+    a.release_mem_view(rv)
+    a.release_mem_view(lv)
+    a.release_mem_view(lv)  # a handle the agent no longer knows is ignored (logged)
+    for bad in ([(theirs.ctypes.data, 4097, 0, "beta")],          # longer than the registration
+                [(mine.ctypes.data, 64, 0, "beta")],               # alpha's memory under beta's name
+                [(0, 0, 0, None)]):                                # placeholders alone name no backend
+        with pytest.raises(ag.NixlError) as e:
+            a.prep_mem_view(a.get_remote_descs(bad, "DRAM"))
+        assert e.value.status == ag.NIXL_ERR_NOT_FOUND
+    with pytest.raises(ag.NixlError):
+        a.prep_mem_view(_descs(a, theirs, [0], [64]))  # beta's memory is not a local registration
+    # views left unreleased are freed with the agent
+    a.prep_mem_view(_descs(a, mine, [0], [64]))
