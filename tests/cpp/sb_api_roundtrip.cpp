@@ -3,7 +3,8 @@
 // 125-209; round trip "WRITE, reset the source, READ, check the pattern",
 // test/gtest/plugins/obj/obj_plugin.cpp:93-101 with the increasing-byte pattern of
 // test/gtest/plugins/memory_handler.h:42-58; handle reuse, test/unit/plugins/ucx/
-// ucx_backend_test.cpp:28-92).  The plugin is opened with the flags the reference's plugin
+// ucx_backend_test.cpp:28-92; a second engine as the target of remote transfers and
+// notifications, as that test's two-engine set-up).  The plugin is opened with the flags the reference's plugin
 // manager uses (src/core/nixl_plugin_manager.cpp:342).
 //
 // usage: sb_api_roundtrip <path to libplugin_HIP.so>; prints "OK" and exits 0 on success.
@@ -181,6 +182,95 @@ main(int argc, char **argv) {
     nixl_meta_dlist_t shorter(VRAM_SEG);
     shorter.addDesc(remote[0]);
     REQUIRE(engine->prepXfer(NIXL_WRITE, local, shorter, agent, bad) < 0 && bad == nullptr);
+
+    // A second engine under another agent name: initiator and target of one process, wired
+    // the way the agent wires two backends (connection info, public data of a registration,
+    // loadRemoteMD, connect), then a WRITE with a notification and a READ
+    // (shape of test/unit/plugins/ucx/ucx_backend_test.cpp: two engines, :383-389 data check,
+    // notification seen by the target once the transfer is complete).
+    {
+        const std::string peer = "sb-peer";
+        nixlBackendInitParams peer_params = params;
+        peer_params.localAgent = peer;
+        nixlBackendEngine *target = plugin->create_engine(&peer_params);
+        REQUIRE(target && !target->getInitErr());
+        uint8_t *tbuf = nullptr;
+        REQUIRE(hipMalloc(reinterpret_cast<void **>(&tbuf), total) == hipSuccess);
+        REQUIRE(hipMemset(tbuf, 0, total) == hipSuccess);
+        REQUIRE(hipDeviceSynchronize() == hipSuccess);
+        nixlBackendMD *t_md = nullptr, *t_at_initiator = nullptr;
+        const nixlBlobDesc t_region(reinterpret_cast<uintptr_t>(tbuf), total, 0, "");
+        REQUIRE(target->registerMem(t_region, VRAM_SEG, t_md) == NIXL_SUCCESS);
+
+        std::string t_conn, t_public;
+        REQUIRE(target->getConnInfo(t_conn) == NIXL_SUCCESS);
+        REQUIRE(target->getPublicData(t_md, t_public) == NIXL_SUCCESS && !t_public.empty());
+        // nothing of the peer is usable before its connection info is loaded
+        REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public), VRAM_SEG, peer, t_at_initiator) < 0);
+        REQUIRE(engine->loadRemoteConnInfo(peer, "HIP1:pid=1") == NIXL_ERR_NOT_SUPPORTED); // another process
+        REQUIRE(engine->loadRemoteConnInfo(peer, "garbage") < 0);
+        REQUIRE(engine->loadRemoteConnInfo(peer, t_conn) == NIXL_SUCCESS);
+        REQUIRE(engine->connect(peer) == NIXL_SUCCESS);
+        // public data that does not belong to the descriptor it arrives with is refused
+        REQUIRE(engine->loadRemoteMD(nixlBlobDesc(reinterpret_cast<uintptr_t>(tbuf), total / 2, 0, t_public), VRAM_SEG, peer,
+                                     t_at_initiator) < 0);
+        REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public.substr(1)), VRAM_SEG, peer, t_at_initiator) < 0);
+        REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public), VRAM_SEG, peer, t_at_initiator) == NIXL_SUCCESS);
+        REQUIRE(t_at_initiator && t_at_initiator != t_md);
+
+        nixl_meta_dlist_t l2(VRAM_SEG), r2(VRAM_SEG);
+        nixlMetaDesc le(reinterpret_cast<uintptr_t>(src), total, 0), re(reinterpret_cast<uintptr_t>(tbuf), total, 0);
+        le.metadataP = src_md;
+        re.metadataP = t_at_initiator;
+        l2.addDesc(le);
+        r2.addDesc(re);
+        fillIncreasing(host, 33);
+        REQUIRE(hipMemcpy(src, host.data(), total, hipMemcpyHostToDevice) == hipSuccess);
+        nixl_opt_b_args_t with_notif;
+        with_notif.notifMsg = "block landed";
+        with_notif.hasNotif = true;
+        nixlBackendReqH *w2 = nullptr;
+        REQUIRE(engine->prepXfer(NIXL_WRITE, l2, r2, peer, w2, &with_notif) == NIXL_SUCCESS && w2);
+        nixl_status_t st = engine->postXfer(NIXL_WRITE, l2, r2, peer, w2, &with_notif);
+        REQUIRE(st == NIXL_IN_PROG || st == NIXL_SUCCESS);
+        while (st == NIXL_IN_PROG)
+            st = engine->checkXfer(w2);
+        REQUIRE(st == NIXL_SUCCESS);
+        notif_list_t seen;
+        REQUIRE(target->getNotifs(seen) == NIXL_SUCCESS);
+        REQUIRE(seen.size() == 1 && seen[0].first == agent && seen[0].second == "block landed");
+        REQUIRE(hipMemcpy(back.data(), tbuf, total, hipMemcpyDeviceToHost) == hipSuccess);
+        REQUIRE(checkIncreasing(back, 33));
+        seen.clear();
+        REQUIRE(engine->getNotifs(seen) == NIXL_SUCCESS && seen.empty()); // none for the initiator
+
+        // READ from the peer, no notification
+        REQUIRE(hipMemset(src, 0, total) == hipSuccess);
+        REQUIRE(hipDeviceSynchronize() == hipSuccess);
+        nixlBackendReqH *r2h = nullptr;
+        REQUIRE(engine->prepXfer(NIXL_READ, l2, r2, peer, r2h) == NIXL_SUCCESS);
+        REQUIRE(runToCompletion(engine, NIXL_READ, l2, r2, peer, r2h) == NIXL_SUCCESS);
+        REQUIRE(hipMemcpy(back.data(), src, total, hipMemcpyDeviceToHost) == hipSuccess);
+        REQUIRE(checkIncreasing(back, 33));
+        REQUIRE(target->getNotifs(seen) == NIXL_SUCCESS && seen.empty());
+
+        // stand-alone messages, both ways and to oneself
+        REQUIRE(engine->genNotif(peer, "ping") == NIXL_SUCCESS && target->genNotif(agent, "pong") == NIXL_SUCCESS);
+        REQUIRE(engine->genNotif(agent, "self") == NIXL_SUCCESS);
+        REQUIRE(engine->genNotif("nobody", "lost") == NIXL_ERR_NOT_FOUND);
+        REQUIRE(target->getNotifs(seen) == NIXL_SUCCESS && seen.size() == 1 && seen[0].second == "ping");
+        seen.clear();
+        REQUIRE(engine->getNotifs(seen) == NIXL_SUCCESS && seen.size() == 2);
+
+        REQUIRE(engine->releaseReqH(w2) == NIXL_SUCCESS && engine->releaseReqH(r2h) == NIXL_SUCCESS);
+        REQUIRE(engine->unloadMD(t_at_initiator) == NIXL_SUCCESS); // frees the initiator's copy
+        REQUIRE(engine->disconnect(peer) == NIXL_SUCCESS);
+        REQUIRE(engine->prepXfer(NIXL_WRITE, l2, r2, peer, bad) < 0 && bad == nullptr); // no longer a peer
+        REQUIRE(target->deregisterMem(t_md) == NIXL_SUCCESS);
+        plugin->destroy_engine(target);
+        REQUIRE(engine->genNotif(peer, "too late") == NIXL_ERR_NOT_FOUND); // its queue went with it
+        REQUIRE(hipFree(tbuf) == hipSuccess);
+    }
 
     REQUIRE(engine->releaseReqH(wr) == NIXL_SUCCESS);
     REQUIRE(engine->releaseReqH(rd) == NIXL_SUCCESS);
