@@ -10,6 +10,7 @@
 //
 // HBM traffic: dispatch reads every source row once (2H) and writes it once per destination
 // rank that holds one of its experts; combine reads those rows once and writes 2H per token.
+#include <algorithm>
 #include <cstdint>
 
 #include "common.h"
@@ -47,8 +48,19 @@ block_exclusive_scan(V v, V *wave_sums, V &total) {
 }
 
 // ---- layout (kernels/layout.cu:31-138) ----------------------------------------------------
-// grid = R source ranks; LDS: E + R counters.
-__global__ void __launch_bounds__(kScanThreads)
+// grid = R source ranks x chunks of kLayoutTokens tokens, one token per thread; LDS: E + R
+// counters per workgroup, added to the (zeroed) outputs at the end.  Integer sums: the
+// result does not depend on the order of the additions.
+constexpr int kLayoutTokens = 256;
+
+__global__ void __launch_bounds__(256)
+zero_ints_kernel(int *__restrict__ a, size_t na, int *__restrict__ b, size_t nb) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < na) a[i] = 0;
+    if (i < nb) b[i] = 0;
+}
+
+__global__ void __launch_bounds__(kLayoutTokens)
 layout_kernel(const int32_t *__restrict__ topk_idx,
               int *__restrict__ per_rank,
               int *__restrict__ per_expert,
@@ -58,29 +70,59 @@ layout_kernel(const int32_t *__restrict__ topk_idx,
               int R,
               int E) {
     extern __shared__ int counters[]; // [E] experts, then [R] ranks
-    const int src = blockIdx.x, El = E / R;
+    const int chunks = (T + kLayoutTokens - 1) / kLayoutTokens;
+    const int src = blockIdx.x / chunks, El = E / R;
+    const int t = (blockIdx.x % chunks) * kLayoutTokens + threadIdx.x;
     for (int i = threadIdx.x; i < E + R; i += blockDim.x)
         counters[i] = 0;
     __syncthreads();
-    for (int t = threadIdx.x; t < T; t += blockDim.x) {
+    // whether the R flag bytes of a token can be written as one aligned 8-byte word
+    const bool word_flags = R == 8 && (reinterpret_cast<uintptr_t>(in_rank) & 7u) == 0;
+    if (t < T) {
         const int32_t *sel = topk_idx + (static_cast<size_t>(src) * T + t) * K;
         uint8_t *flags = in_rank + (static_cast<size_t>(src) * T + t) * R;
-        for (int d = 0; d < R; ++d)
-            flags[d] = 0;
-        for (int k = 0; k < K; ++k) {
-            const int e = sel[k];
-            if (e < 0 || e >= E) continue;
-            atomicAdd(&counters[e], 1);
-            flags[e / El] = 1;
+        if (R <= 64) {
+            // destination ranks of the token as a bit mask in a register
+            unsigned long long mask = 0;
+            for (int k = 0; k < K; ++k) {
+                const int e = sel[k];
+                if (e < 0 || e >= E) continue;
+                atomicAdd(&counters[e], 1);
+                mask |= 1ull << (e / El);
+            }
+            if (word_flags) {
+                unsigned long long bytes = 0;
+#pragma unroll
+                for (int d = 0; d < 8; ++d)
+                    bytes |= ((mask >> d) & 1ull) << (8 * d);
+                *reinterpret_cast<unsigned long long *>(flags) = bytes;
+            } else {
+                for (int d = 0; d < R; ++d)
+                    flags[d] = static_cast<uint8_t>((mask >> d) & 1ull);
+            }
+            while (mask) {
+                const int d = __builtin_ctzll(mask);
+                mask &= mask - 1;
+                atomicAdd(&counters[E + d], 1);
+            }
+        } else {
+            for (int d = 0; d < R; ++d)
+                flags[d] = 0;
+            for (int k = 0; k < K; ++k) {
+                const int e = sel[k];
+                if (e < 0 || e >= E) continue;
+                atomicAdd(&counters[e], 1);
+                flags[e / El] = 1;
+            }
+            for (int d = 0; d < R; ++d)
+                if (flags[d]) atomicAdd(&counters[E + d], 1);
         }
-        for (int d = 0; d < R; ++d)
-            if (flags[d]) atomicAdd(&counters[E + d], 1);
     }
     __syncthreads();
     for (int i = threadIdx.x; i < E; i += blockDim.x)
-        per_expert[static_cast<size_t>(src) * E + i] = counters[i];
+        if (counters[i]) atomicAdd(&per_expert[static_cast<size_t>(src) * E + i], counters[i]);
     for (int i = threadIdx.x; i < R; i += blockDim.x)
-        per_rank[static_cast<size_t>(src) * R + i] = counters[E + i];
+        if (counters[E + i]) atomicAdd(&per_rank[static_cast<size_t>(src) * R + i], counters[E + i]);
 }
 
 // ---- notify, part 1: per (source, destination) pair, positions inside the segment and the
@@ -608,7 +650,15 @@ nixl_amd_ep_get_dispatch_layout(const int32_t *topk_idx,
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "get_dispatch_layout: null pointer argument");
     const size_t lds = static_cast<size_t>(num_experts + num_ranks) * sizeof(int);
     if (lds > 48 * 1024) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "get_dispatch_layout: too many experts");
-    hipLaunchKernelGGL(layout_kernel, dim3(num_ranks), dim3(kScanThreads), lds, static_cast<hipStream_t>(stream), topk_idx,
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // the counts are accumulated with atomics; cleared by a kernel, not a memset, so that a
+    // caller may capture the call into a graph
+    const size_t n_rank = static_cast<size_t>(num_ranks) * num_ranks, n_expert = static_cast<size_t>(num_ranks) * num_experts;
+    hipLaunchKernelGGL(zero_ints_kernel, dim3(static_cast<unsigned>((std::max(n_rank, n_expert) + 255) / 256)), dim3(256), 0, s,
+                       num_tokens_per_rank, n_rank, num_tokens_per_expert, n_expert);
+    HIP_TRY(hipGetLastError());
+    const long long chunks = (num_tokens + kLayoutTokens - 1) / kLayoutTokens;
+    hipLaunchKernelGGL(layout_kernel, dim3(static_cast<unsigned>(num_ranks * chunks)), dim3(kLayoutTokens), lds, s, topk_idx,
                        num_tokens_per_rank, num_tokens_per_expert, is_token_in_rank, num_tokens, num_topk, num_ranks,
                        num_experts);
     HIP_TRY(hipGetLastError());
