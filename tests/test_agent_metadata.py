@@ -307,3 +307,15 @@ def test_memory_view_lists_resolve_through_the_agent(two_agents):
         a.prep_mem_view(_descs(a, theirs, [0], [64]))  # beta's memory is not a local registration
     # views left unreleased are freed with the agent
     a.prep_mem_view(_descs(a, mine, [0], [64]))
+
+
+def test_agents_used_from_several_threads(oracle_plugin_dir):
+    """tests/cpp/agent_threads_check.cpp: transfers with notifications, memory views,
+    registration and metadata calls from six threads at once; every notification arrives once."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "agent_threads_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe, oracle_plugin_dir], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
