@@ -144,7 +144,7 @@ def run_normal(dev, warmup=5, iters=20):
         "layout": t_layout,
         "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]),
                      "note": "count exchange + rows + per-row metadata; receive tensors sized for the worst case, so the "
-                             "host read-back of the counts overlaps the row kernel"},
+                             "host's wait for the counts (pinned memory) overlaps the row kernel"},
         "dispatch_cached_handle": {**t_cached, **_rate(tokens * H * 2 + rows * H * 2, t_cached["avg_us"]),
                                    "note": "layout of an earlier dispatch reused: rows only, no count exchange"},
         "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
