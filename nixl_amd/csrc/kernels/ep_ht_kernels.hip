@@ -552,22 +552,54 @@ ht_combine_kernel(uint16_t *__restrict__ combined,
 
 // ---- router -----------------------------------------------------------------------------------------
 // One wave per token; lane l holds experts l, l + 64, ...  K rounds of a wave-wide argmax
-// (larger value wins, equal values go to the lower expert index).
+// (larger value wins, equal values go to the lower expert index).  The two reductions of a
+// round (maximum of the values, then lowest index among the lanes that hold it) run on
+// the DPP data path: four steps inside the rows of 16 lanes, two row broadcasts, result in
+// lane 63.  Cross-lane permutes through LDS took three times as long.
 constexpr int kRouterMaxPerLane = 16; // E <= 1024
+
+template<int CTRL, int ROW_MASK>
+__device__ __forceinline__ int
+dpp_move(int x) {
+    // lanes whose row is masked out, or whose source lane does not exist, keep x
+    return __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xf, false);
+}
+
+// Reduction of one 32-bit value per lane over the wave; every lane of the last row (and so
+// lane 63) holds the result.  op must be idempotent (max, min).
+template<typename Op>
+__device__ __forceinline__ int
+wave_reduce_dpp(int x, Op op) {
+    x = op(x, dpp_move<0xb1, 0xf>(x));  // quad_perm [1,0,3,2]
+    x = op(x, dpp_move<0x4e, 0xf>(x));  // quad_perm [2,3,0,1]
+    x = op(x, dpp_move<0x124, 0xf>(x)); // row_ror 4
+    x = op(x, dpp_move<0x128, 0xf>(x)); // row_ror 8
+    x = op(x, dpp_move<0x142, 0xa>(x)); // row_bcast 15 into rows 1 and 3
+    x = op(x, dpp_move<0x143, 0xc>(x)); // row_bcast 31 into rows 2 and 3
+    return __builtin_amdgcn_readlane(x, kWaveSize - 1);
+}
+
+// Order-preserving map of a float onto a signed integer (negative floats reversed), so that
+// integer max is float max; -0.0 and +0.0 stay distinct neighbours, which the tie rule of the
+// values below undoes by comparing the floats themselves.
+__device__ __forceinline__ int
+float_order_key(float f) {
+    const int b = __float_as_int(f);
+    return b >= 0 ? b : b ^ 0x7fffffff;
+}
 
 // PL = experts a lane holds (a power of two >= ceil(E / 64)): the argmax rounds only walk
 // the slots that exist.
 template<int PL>
 __global__ void __launch_bounds__(256)
 router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, float *__restrict__ topk_w, int n_tokens, int E, int K) {
-    constexpr int kRouterMaxPerLane = PL; // shadows the global bound inside this kernel
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int token = blockIdx.x * (blockDim.x / kWaveSize) + threadIdx.x / kWaveSize;
-    if (token >= n_tokens) return;
-    float v[kRouterMaxPerLane];
+    if (token >= n_tokens) return; // whole waves leave together: the DPP steps below see full waves
+    float v[PL];
     unsigned taken = 0;
 #pragma unroll
-    for (int j = 0; j < kRouterMaxPerLane; ++j) {
+    for (int j = 0; j < PL; ++j) {
         const int e = j * kWaveSize + lane;
         v[j] = e < E ? logits[static_cast<size_t>(token) * E + e] : 0.f;
         if (e >= E) taken |= 1u << j;
@@ -578,26 +610,26 @@ router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, 
         float best = 0.f;
         int best_e = 0x7fffffff;
 #pragma unroll
-        for (int j = 0; j < kRouterMaxPerLane; ++j) {
+        for (int j = 0; j < PL; ++j) {
             const int e = j * kWaveSize + lane;
             if (!((taken >> j) & 1u) && (best_e == 0x7fffffff || v[j] > best)) {
                 best = v[j];
                 best_e = e;
             }
         }
-#pragma unroll
-        for (int off = kWaveSize / 2; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(best, off);
-            const int oe = __shfl_xor(best_e, off);
-            const bool mine_valid = best_e != 0x7fffffff, other_valid = oe != 0x7fffffff;
-            if (other_valid && (!mine_valid || ov > best || (ov == best && oe < best_e))) {
-                best = ov;
-                best_e = oe;
-            }
-        }
-        if ((best_e & (kWaveSize - 1)) == lane) taken |= 1u << (best_e / kWaveSize);
-        sel_v[k] = best;
-        sel_i[k] = best_e;
+        const bool have = best_e != 0x7fffffff;
+        // largest value among the lanes that still have one
+        const int key = have ? float_order_key(best) : static_cast<int>(0x80000000);
+        const int top_key = wave_reduce_dpp(key, [](int a, int b) { return a > b ? a : b; });
+        const float top = __int_as_float(top_key >= 0 ? top_key : top_key ^ 0x7fffffff);
+        // lowest expert index among the lanes that hold a value equal to it (0.0 == -0.0)
+        const int cand = (have && best == top) ? best_e : 0x7fffffff;
+        int win = wave_reduce_dpp(cand, [](int a, int b) { return a < b ? a : b; });
+        if (win == 0x7fffffff) // only NaNs are left: take them in index order
+            win = wave_reduce_dpp(have ? best_e : 0x7fffffff, [](int a, int b) { return a < b ? a : b; });
+        if ((win & (kWaveSize - 1)) == lane) taken |= 1u << (win / kWaveSize);
+        sel_v[k] = top;
+        sel_i[k] = win;
     }
     if (lane == 0) {
         const float top = sel_v[0];

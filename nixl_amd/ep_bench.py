@@ -75,6 +75,13 @@ def run_low_latency(dev, warmup=20, iters=50):
 
     t_both = _timed(both, flush, warmup, iters)
 
+    def routed():  # the router in front as well: logits -> top-k -> dispatch -> combine
+        state["routed_topk"], state["routed_w"] = buf.route(logits, K)
+        state["out"] = buf.dispatch(x, state["routed_topk"], M, E, use_fp8=True)
+        buf.combine(y, state["routed_topk"], state["routed_w"], state["out"][2])
+
+    t_routed = _timed(routed, flush, warmup, iters)
+
     tokens, pairs = R * T, int((topk >= 0).sum())
     meta = R * El * R * 8 + R * El * 4
     dispatch_bytes = tokens * H * 2 + tokens * K * 4 + pairs * (H + H // 128 * 4 + 4) + meta
@@ -87,6 +94,9 @@ def run_low_latency(dev, warmup=20, iters=50):
         "dispatch_plus_combine_us": round(both_us, 2),
         "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
         "dispatch_then_combine_one_event_pair": {**t_both, **_rate(dispatch_bytes + combine_bytes, t_both["avg_us"])},
+        "route_dispatch_combine_one_event_pair": {
+            **t_routed, **_rate(dispatch_bytes + combine_bytes + tokens * E * 4, t_routed["avg_us"]),
+            "note": "router (logits -> top-k + softmax) included; its logits add 4.2 MB"},
         "combine_logfmt": {**t_logfmt, "note": "rows passed through the LogFMT-10 codec before accumulation"},
         "router": {**t_router, "bytes": tokens * E * 4},
     }
