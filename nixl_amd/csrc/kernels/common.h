@@ -20,6 +20,40 @@ nixl_amd_fail(int code, const std::string &msg);
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
     } while (0)
 
+// Makes `device` current for the calling thread for the lifetime of the object and puts the
+// thread's previous device back afterwards: a library call must not leave the application on
+// another GPU than it was on.
+class DeviceScope {
+public:
+    explicit DeviceScope(int device) {
+        int current = -1;
+        if (hipGetDevice(&current) != hipSuccess) current = -1;
+        if (current == device) {
+            status_ = hipSuccess;
+            return;
+        }
+        status_ = hipSetDevice(device);
+        if (status_ == hipSuccess && current >= 0) previous_ = current;
+    }
+
+    ~DeviceScope() {
+        if (previous_ >= 0) (void)hipSetDevice(previous_);
+    }
+
+    DeviceScope(const DeviceScope &) = delete;
+    DeviceScope &
+    operator=(const DeviceScope &) = delete;
+
+    hipError_t
+    status() const {
+        return status_;
+    }
+
+private:
+    int previous_ = -1;
+    hipError_t status_ = hipSuccess;
+};
+
 constexpr int kWaveSize = 64;
 
 __device__ __forceinline__ uint32_t

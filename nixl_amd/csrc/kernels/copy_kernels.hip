@@ -377,7 +377,8 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
         return nixl_amd_fail(NIXL_AMD_ERR_NO_DEVICE, "plan_create: no HIP device");
     if (device < 0 || device >= ndev) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: bad device index");
-    HIP_TRY(hipSetDevice(device));
+    const DeviceScope on_device(device);
+    HIP_TRY(on_device.status());
 
     // ---- host-side lowering ------------------------------------------------------
     std::vector<uint64_t> vsrc, vdst, vprefix;
@@ -583,7 +584,8 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
 int
 nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
     if (!plan) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_launch: plan is null");
-    HIP_TRY(hipSetDevice(plan->device));
+    const DeviceScope on_device(plan->device);
+    HIP_TRY(on_device.status());
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (plan->uniform_wgs) {
         // With the die swizzle the grid is rounded up to a multiple of 8 so that every
@@ -629,7 +631,7 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
 int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan) {
     if (!plan) return NIXL_AMD_OK;
-    (void)hipSetDevice(plan->device);
+    const DeviceScope on_device(plan->device);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     hipError_t e = plan->arena ? hipFree(plan->arena) : hipSuccess;
@@ -649,7 +651,8 @@ int
 nixl_amd_copy_plan_time(nixl_amd_copy_plan_t *plan, void *stream, int iters, float *ms_per_launch) {
     if (!plan || !ms_per_launch || iters <= 0)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_time: bad argument");
-    HIP_TRY(hipSetDevice(plan->device));
+    const DeviceScope on_device(plan->device);
+    HIP_TRY(on_device.status());
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (!plan->ev0) HIP_TRY(hipEventCreate(&plan->ev0));
     if (!plan->ev1) HIP_TRY(hipEventCreate(&plan->ev1));

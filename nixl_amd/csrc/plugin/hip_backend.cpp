@@ -33,6 +33,38 @@ hipOk(hipError_t e, const char *what) {
     return false;
 }
 
+// Makes `device` current for the calling thread while the object lives and restores the
+// thread's previous device afterwards, so that a call into the backend never leaves the
+// application on another GPU than it was on.
+class DeviceScope {
+public:
+    explicit DeviceScope(int device) {
+        int current = -1;
+        if (hipGetDevice(&current) != hipSuccess) current = -1;
+        if (current == device) return;
+        status_ = hipSetDevice(device);
+        if (status_ == hipSuccess && current >= 0) previous_ = current;
+    }
+
+    ~DeviceScope() {
+        if (previous_ >= 0) (void)hipSetDevice(previous_);
+    }
+
+    DeviceScope(const DeviceScope &) = delete;
+    DeviceScope &
+    operator=(const DeviceScope &) = delete;
+
+    bool
+    ok() const {
+        if (status_ != hipSuccess) NIXL_ERROR << "HIP backend: hipSetDevice failed: " << hipGetErrorString(status_);
+        return status_ == hipSuccess;
+    }
+
+private:
+    int previous_ = -1;
+    hipError_t status_ = hipSuccess;
+};
+
 // Engines of this process by agent name: how a notification reaches another agent's queue.
 std::mutex g_registryMutex;
 std::unordered_map<std::string, const nixlHipEngine *> g_registry;
@@ -52,7 +84,7 @@ constexpr const char *kConnPrefix = "HIP1:pid=";
 } // namespace
 
 nixlHipReqH::~nixlHipReqH() {
-    (void)hipSetDevice(device);
+    const DeviceScope on_device(device);
     if (plan) (void)nixl_amd_copy_plan_destroy(plan);
     if (done) (void)hipEventDestroy(done);
 }
@@ -103,12 +135,12 @@ nixlHipEngine::~nixlHipEngine() {
     }
     reapRetired(true);
     for (const auto &[table, device] : memViews_) {
-        (void)hipSetDevice(device);
+        const DeviceScope on_device(device);
         (void)hipFree(table);
     }
     for (size_t i = 0; i < streams_.size(); ++i) {
         if (!streams_[i]) continue;
-        (void)hipSetDevice(static_cast<int>(i / streamsPerDevice_));
+        const DeviceScope on_device(static_cast<int>(i / streamsPerDevice_));
         (void)hipStreamSynchronize(streams_[i]);
         (void)hipStreamDestroy(streams_[i]);
     }
@@ -134,7 +166,7 @@ nixlHipEngine::reapRetired(bool wait) const {
     std::lock_guard<std::mutex> lock(retiredMutex_);
     size_t keep = 0;
     for (nixlHipReqH *r : retired_) {
-        (void)hipSetDevice(r->device);
+        const DeviceScope on_device(r->device);
         bool finished = true;
         if (r->posted) {
             if (wait)
@@ -277,8 +309,8 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
         return NIXL_ERR_BACKEND;
     }
-    if (!hipOk(hipSetDevice(device), "hipSetDevice") ||
-        !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
+    const DeviceScope on_device(device);
+    if (!on_device.ok() || !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
         return NIXL_ERR_BACKEND;
     req->stream = pickStream(device);
     if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
@@ -296,7 +328,8 @@ nixlHipEngine::postXfer(const nixl_xfer_op_t &,
                         const nixl_opt_b_args_t *opt_args) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req || !req->plan) return NIXL_ERR_INVALID_PARAM;
-    if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
+    const DeviceScope on_device(req->device);
+    if (!on_device.ok()) return NIXL_ERR_BACKEND;
     if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
     // the notification of an earlier post that nobody polled to completion goes out first
     deliverPending(req);
@@ -320,7 +353,8 @@ nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_ERR_INVALID_PARAM;
     if (!req->posted) return NIXL_SUCCESS; // nothing outstanding
-    if (!hipOk(hipSetDevice(req->device), "hipSetDevice")) return NIXL_ERR_BACKEND;
+    const DeviceScope on_device(req->device);
+    if (!on_device.ok()) return NIXL_ERR_BACKEND;
     const hipError_t e = hipEventQuery(req->done);
     if (e == hipSuccess) {
         // the peer learns of the transfer only after its bytes have landed
@@ -336,7 +370,7 @@ nixl_status_t
 nixlHipEngine::releaseReqH(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_SUCCESS;
-    (void)hipSetDevice(req->device);
+    const DeviceScope on_device(req->device);
     if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) {
         // A launched kernel cannot be cancelled; keep its plan alive until it has
         // drained and free it from a later call, so that this call never blocks.
@@ -538,8 +572,8 @@ nixlHipEngine::buildMemView(const std::vector<viewEntry> &entries, uint32_t kind
 
     void *table = nullptr;
     const size_t bytes = image.size() * sizeof(uint64_t);
-    if (!hipOk(hipSetDevice(device), "hipSetDevice") || !hipOk(hipMalloc(&table, bytes), "hipMalloc"))
-        return NIXL_ERR_BACKEND;
+    const DeviceScope on_device(device);
+    if (!on_device.ok() || !hipOk(hipMalloc(&table, bytes), "hipMalloc")) return NIXL_ERR_BACKEND;
     // Synchronous copy: the table is complete when the handle is handed out, whichever
     // stream the application launches its kernels on.
     if (!hipOk(hipMemcpy(table, image.data(), bytes, hipMemcpyHostToDevice), "hipMemcpy")) {
@@ -594,7 +628,7 @@ nixlHipEngine::releaseMemView(nixlMemViewH mvh) const {
         memViews_.erase(it);
     }
     // hipFree waits for the device, so a kernel still reading the table finishes first.
-    (void)hipSetDevice(device);
+    const DeviceScope on_device(device);
     (void)hipFree(mvh);
 }
 
