@@ -3,6 +3,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <unordered_map>
@@ -123,11 +124,26 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     }
     numDevices_ = n;
     streams_.assign(static_cast<size_t>(n) * streamsPerDevice_, nullptr);
-    std::lock_guard<std::mutex> lock(g_registryMutex);
-    g_registry[localAgent] = this;
+    {
+        std::lock_guard<std::mutex> lock(g_registryMutex);
+        g_registry[localAgent] = this;
+    }
+    if (init_params->enableProgTh) {
+        progressOn_ = true;
+        progressDelayUs_ = init_params->pthrDelay;
+        progress_ = std::thread(&nixlHipEngine::progressLoop, this);
+    }
 }
 
 nixlHipEngine::~nixlHipEngine() {
+    if (progress_.joinable()) {
+        {
+            std::lock_guard<std::mutex> lock(pendingMutex_);
+            stopProgress_ = true;
+        }
+        pendingCv_.notify_all();
+        progress_.join();
+    }
     {
         std::lock_guard<std::mutex> lock(g_registryMutex);
         const auto it = g_registry.find(localAgent);
@@ -333,11 +349,6 @@ nixlHipEngine::postXfer(const nixl_xfer_op_t &,
     if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
     // the notification of an earlier post that nobody polled to completion goes out first
     deliverPending(req);
-    if (opt_args && opt_args->hasNotif) {
-        req->notifPending = true;
-        req->notifTarget = remote_agent;
-        req->notifMsg = opt_args->notifMsg;
-    }
 
     if (nixl_amd_copy_plan_launch(req->plan, req->stream) != NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
@@ -345,6 +356,17 @@ nixlHipEngine::postXfer(const nixl_xfer_op_t &,
     }
     if (!hipOk(hipEventRecord(req->done, req->stream), "hipEventRecord")) return NIXL_ERR_BACKEND;
     req->posted = true;
+    if (opt_args && opt_args->hasNotif) {
+        // only now: whoever sees the flag must find the event of THIS post behind it
+        std::lock_guard<std::mutex> lock(pendingMutex_);
+        req->notifPending = true;
+        req->notifTarget = remote_agent;
+        req->notifMsg = opt_args->notifMsg;
+        if (progressOn_) {
+            watched_.push_back(req);
+            pendingCv_.notify_one();
+        }
+    }
     return NIXL_IN_PROG;
 }
 
@@ -394,10 +416,51 @@ nixlHipEngine::knowsAgent(const std::string &name) const {
 
 void
 nixlHipEngine::deliverPending(nixlHipReqH *req) const {
-    if (!req->notifPending) return;
-    req->notifPending = false;
-    if (genNotif(req->notifTarget, req->notifMsg) != NIXL_SUCCESS)
-        NIXL_WARN << "HIP backend: notification for agent '" << req->notifTarget << "' could not be delivered";
+    std::string target, msg;
+    {
+        std::lock_guard<std::mutex> lock(pendingMutex_);
+        if (!req->notifPending) return;
+        req->notifPending = false;
+        target = req->notifTarget;
+        msg = req->notifMsg;
+        const auto it = std::find(watched_.begin(), watched_.end(), req);
+        if (it != watched_.end()) watched_.erase(it);
+    }
+    if (genNotif(target, msg) != NIXL_SUCCESS)
+        NIXL_WARN << "HIP backend: notification for agent '" << target << "' could not be delivered";
+}
+
+// The progress thread: sleeps while no posted transfer carries a notification; otherwise
+// polls the events of those that do and queues each message at its target once the copy has
+// finished.  A request is only ever touched under pendingMutex_, and every path that deletes
+// one takes it off the list first (deliverPending), under the same mutex.
+void
+nixlHipEngine::progressLoop() {
+    const auto nap = std::chrono::microseconds(progressDelayUs_ ? progressDelayUs_ : 20);
+    for (;;) {
+        std::vector<std::pair<std::string, std::string>> ready;
+        {
+            std::unique_lock<std::mutex> lock(pendingMutex_);
+            pendingCv_.wait(lock, [&] { return stopProgress_ || !watched_.empty(); });
+            if (stopProgress_) return;
+            for (size_t i = 0; i < watched_.size();) {
+                nixlHipReqH *req = watched_[i];
+                const DeviceScope on_device(req->device);
+                if (hipEventQuery(req->done) == hipErrorNotReady) {
+                    ++i;
+                    continue;
+                }
+                req->notifPending = false;
+                ready.emplace_back(req->notifTarget, req->notifMsg);
+                watched_[i] = watched_.back();
+                watched_.pop_back();
+            }
+        }
+        for (const auto &[target, msg] : ready)
+            if (genNotif(target, msg) != NIXL_SUCCESS)
+                NIXL_WARN << "HIP backend: notification for agent '" << target << "' could not be delivered";
+        if (ready.empty()) std::this_thread::sleep_for(nap);
+    }
 }
 
 nixl_status_t

@@ -11,7 +11,9 @@
 #include <hip/hip_runtime_api.h>
 
 #include <atomic>
+#include <condition_variable>
 #include <mutex>
+#include <thread>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -50,7 +52,8 @@ public:
     int device = 0;
     bool posted = false;
     size_t bytes = 0;
-    // A notification that is due once the posted transfer has finished.
+    // A notification that is due once the posted transfer has finished.  Guarded by the
+    // engine's pendingMutex_, because the progress thread looks at it too.
     bool notifPending = false;
     std::string notifTarget;
     std::string notifMsg;
@@ -173,6 +176,8 @@ private:
     knowsAgent(const std::string &name) const;
     void
     deliverPending(nixlHipReqH *req) const;
+    void
+    progressLoop();
     struct viewEntry {
         uintptr_t addr;
         size_t len;
@@ -193,6 +198,17 @@ private:
     // Requests released while their kernel was still running; freed once it has finished.
     mutable std::vector<nixlHipReqH *> retired_;
     mutable std::mutex retiredMutex_;
+    // Notifications of posted transfers.  With a progress thread (enableProgTh of the init
+    // parameters, the agent's useProgThread) the requests that carry one are watched and the
+    // message is queued at the target as soon as the copy has finished; without it, when the
+    // initiator next looks at the request.
+    mutable std::mutex pendingMutex_;
+    mutable std::condition_variable pendingCv_;
+    mutable std::vector<nixlHipReqH *> watched_;
+    bool stopProgress_ = false;
+    bool progressOn_ = false;
+    uint64_t progressDelayUs_ = 0;
+    std::thread progress_;
     // Peers whose connection info was loaded (agents of this process).
     mutable std::mutex peersMutex_;
     std::vector<std::string> peers_;

@@ -558,6 +558,65 @@ def test_memory_view_tables_from_python(cuda):
         a.prep_mem_view([(x.data_ptr(), 64, 0)])
 
 
+@pytest.mark.parametrize("prog_thread", [True, False])
+def test_notification_without_initiator_polling(cuda, prog_thread):
+    """With the agent's progress thread (the Python default, reference _api.py:166) the HIP
+    backend watches posted transfers that carry a notification and queues the message at the
+    target once the copy has finished, whatever the initiator does; without the thread the
+    message waits for the initiator's next look at the request."""
+    import time
+    import torch
+    cfg = lambda: nixl_agent_config(enable_prog_thread=prog_thread, backends=())
+    a, b = nixl_agent("pt-initiator", cfg()), nixl_agent("pt-target", cfg())
+    a.create_backend("HIP")
+    b.create_backend("HIP")
+    n = 64 << 20
+    src = torch.full((n,), 7, dtype=torch.uint8, device=cuda)
+    dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
+    a.register_memory([src])
+    b.register_memory([dst])
+    torch.cuda.synchronize()
+    a.add_remote_agent(b.get_agent_metadata())
+    blk = 1 << 20
+    offs = [i * blk for i in range(n // blk)]
+    h = a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(src, offs, [blk] * len(offs)), "VRAM"),
+                          a.get_xfer_descs(_descs(dst, offs, [blk] * len(offs)), "VRAM"), "pt-target", b"no poll")
+    assert a.transfer(h) in ("PROC", "DONE")
+    if prog_thread:
+        deadline = time.monotonic() + 10
+        got = {}
+        while not got and time.monotonic() < deadline:
+            got = b.get_new_notifs()
+        assert got == {"pt-initiator": [b"no poll"]}
+        assert bool((dst == 7).all())  # the bytes were there when the message arrived
+    else:
+        torch.cuda.synchronize()
+        time.sleep(0.05)
+        assert b.get_new_notifs() == {}
+    assert a.check_xfer_state(h) == "DONE"
+    assert b.get_new_notifs() == ({} if prog_thread else {"pt-initiator": [b"no poll"]})
+    # many requests in flight at once, each with its own message; all arrive exactly once
+    hs = []
+    for i in range(16):
+        l = a.get_xfer_descs(_descs(src, [i * blk], [blk]), "VRAM")
+        r = a.get_xfer_descs(_descs(dst, [i * blk], [blk]), "VRAM")
+        hs.append(a.initialize_xfer("WRITE", l, r, "pt-target", b"req %d" % i))
+    for x in hs:
+        assert a.transfer(x) in ("PROC", "DONE")
+    for x in hs:
+        while a.check_xfer_state(x) == "PROC":
+            pass
+    seen = []
+    deadline = time.monotonic() + 10
+    while len(seen) < 16 and time.monotonic() < deadline:
+        seen += b.get_new_notifs().get("pt-initiator", [])
+    assert sorted(seen) == sorted(b"req %d" % i for i in range(16))
+    for x in hs + [h]:
+        a.release_xfer_handle(x)
+    a.close()
+    b.close()
+
+
 def test_requests_from_several_threads(cuda):
     """The reference calls prepXfer / postXfer / checkXfer / releaseReqH concurrently from
     several threads, one request each (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:
