@@ -83,6 +83,7 @@ typedef struct nixl_capi_param_iter_s *nixl_capi_param_iter_t;
 typedef struct nixl_capi_remote_dlist_s *nixl_capi_remote_dlist_t;
 typedef struct nixl_capi_mem_view_s *nixl_capi_mem_view_t;
 typedef struct nixl_capi_notif_map_s *nixl_capi_notif_map_t;
+typedef struct nixl_capi_query_resp_list_s *nixl_capi_query_resp_list_t;
 
 /* agent */
 nixl_capi_status_t nixl_capi_create_agent(const char *name, nixl_capi_agent_t *agent);
@@ -282,7 +283,7 @@ nixl_capi_invalidate_remote_md(nixl_capi_agent_t agent, const char *remote_agent
 nixl_capi_status_t
 nixl_capi_check_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_xfer_dlist_t descs);
 nixl_capi_status_t
-nixl_capi_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args);
+nixl_capi_agent_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args);
 /* extension: releases a buffer handed out by the calls above */
 nixl_capi_status_t
 nixl_capi_free_buffer(void *data);
@@ -307,6 +308,46 @@ nixl_capi_notif_map_get_notif(nixl_capi_notif_map_t map, const char *agent_name,
                               size_t *len);
 nixl_capi_status_t
 nixl_capi_notif_map_clear(nixl_capi_notif_map_t map);
+
+/* The rest of the reference wrapper's list, option and query helpers (wrapper.h:193-201,
+ * 297-355, 457), so that a caller written against it links unchanged.  xfer_dlist_trim and
+ * reg_dlist_trim build the trimmed copy and drop it, as the reference wrapper does. */
+nixl_capi_status_t nixl_capi_opt_args_get_notif_msg(nixl_capi_opt_args_t args, void **data, size_t *len);
+nixl_capi_status_t nixl_capi_opt_args_get_has_notif(nixl_capi_opt_args_t args, bool *has_notif);
+nixl_capi_status_t nixl_capi_opt_args_get_skip_desc_merge(nixl_capi_opt_args_t args, bool *skip_merge);
+nixl_capi_status_t nixl_capi_opt_args_set_ip_addr(nixl_capi_opt_args_t args, const char *ip_addr);
+nixl_capi_status_t nixl_capi_opt_args_set_port(nixl_capi_opt_args_t args, uint16_t port);
+nixl_capi_status_t nixl_capi_xfer_dlist_get_type(nixl_capi_xfer_dlist_t dlist, nixl_capi_mem_type_t *mem_type);
+nixl_capi_status_t nixl_capi_xfer_dlist_len(nixl_capi_xfer_dlist_t dlist, size_t *len);
+nixl_capi_status_t nixl_capi_xfer_dlist_is_empty(nixl_capi_xfer_dlist_t dlist, bool *is_empty);
+nixl_capi_status_t nixl_capi_xfer_dlist_trim(nixl_capi_xfer_dlist_t dlist);
+nixl_capi_status_t nixl_capi_xfer_dlist_rem_desc(nixl_capi_xfer_dlist_t dlist, int index);
+nixl_capi_status_t nixl_capi_xfer_dlist_resize(nixl_capi_xfer_dlist_t dlist, size_t new_size);
+nixl_capi_status_t nixl_capi_xfer_dlist_print(nixl_capi_xfer_dlist_t dlist);
+nixl_capi_status_t nixl_capi_reg_dlist_get_type(nixl_capi_reg_dlist_t dlist, nixl_capi_mem_type_t *mem_type);
+nixl_capi_status_t nixl_capi_reg_dlist_is_empty(nixl_capi_reg_dlist_t dlist, bool *is_empty);
+nixl_capi_status_t nixl_capi_reg_dlist_trim(nixl_capi_reg_dlist_t dlist);
+nixl_capi_status_t nixl_capi_reg_dlist_rem_desc(nixl_capi_reg_dlist_t dlist, int index);
+nixl_capi_status_t nixl_capi_reg_dlist_clear(nixl_capi_reg_dlist_t dlist);
+nixl_capi_status_t nixl_capi_reg_dlist_resize(nixl_capi_reg_dlist_t dlist, size_t new_size);
+nixl_capi_status_t nixl_capi_reg_dlist_print(nixl_capi_reg_dlist_t dlist);
+nixl_capi_status_t nixl_capi_create_query_resp_list(nixl_capi_query_resp_list_t *list);
+nixl_capi_status_t nixl_capi_destroy_query_resp_list(nixl_capi_query_resp_list_t list);
+nixl_capi_status_t nixl_capi_query_resp_list_size(nixl_capi_query_resp_list_t list, size_t *size);
+nixl_capi_status_t nixl_capi_query_resp_list_has_value(nixl_capi_query_resp_list_t list, size_t index, bool *has_value);
+nixl_capi_status_t nixl_capi_query_resp_list_get_params(nixl_capi_query_resp_list_t list, size_t index,
+                                                        nixl_capi_params_t *params);
+nixl_capi_status_t nixl_capi_query_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs,
+                                       nixl_capi_query_resp_list_t resp, nixl_capi_opt_args_t opt_args);
+/* Metadata side channels of the reference (sockets, ETCD: wrapper.h:148-163): present so that
+ * callers link; they answer NIXL_CAPI_ERROR_BACKEND (NIXL_ERR_NOT_SUPPORTED underneath). */
+nixl_capi_status_t nixl_capi_send_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_send_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs,
+                                                   nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_fetch_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_opt_args_t opt_args);
+nixl_capi_status_t nixl_capi_invalidate_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t opt_args);
+/* false: this is a working library, not the reference's link-time stub */
+bool nixl_capi_is_stub(void);
 
 #ifdef __cplusplus
 }

@@ -6,7 +6,7 @@ implementation: a missing library raises ``NativeLibraryMissing``.
 """
 import ctypes
 import os
-from ctypes import (POINTER, Structure, c_bool, c_char_p, c_float, c_int, c_int64, c_size_t,
+from ctypes import (POINTER, Structure, c_bool, c_char_p, c_float, c_int, c_int64, c_size_t, c_uint16,
                     c_uint, c_uint32, c_uint64, c_void_p)
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -204,7 +204,7 @@ _CAPI_SIGS = {
     "nixl_capi_load_remote_md": [c_void_p, c_char_p, c_size_t, POINTER(c_void_p)],
     "nixl_capi_invalidate_remote_md": [c_void_p, c_char_p],
     "nixl_capi_check_remote_md": [c_void_p, c_char_p, c_void_p],
-    "nixl_capi_make_connection": [c_void_p, c_char_p, c_void_p],
+    "nixl_capi_agent_make_connection": [c_void_p, c_char_p, c_void_p],
     "nixl_capi_free_buffer": [c_void_p],
     "nixl_capi_create_notif_map": [POINTER(c_void_p)],
     "nixl_capi_destroy_notif_map": [c_void_p],
@@ -215,6 +215,36 @@ _CAPI_SIGS = {
     "nixl_capi_notif_map_get_notifs_size": [c_void_p, c_char_p, POINTER(c_size_t)],
     "nixl_capi_notif_map_get_notif": [c_void_p, c_char_p, c_size_t, POINTER(c_void_p), POINTER(c_size_t)],
     "nixl_capi_notif_map_clear": [c_void_p],
+    "nixl_capi_opt_args_get_notif_msg": [c_void_p, POINTER(c_void_p), POINTER(c_size_t)],
+    "nixl_capi_opt_args_get_has_notif": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_opt_args_get_skip_desc_merge": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_opt_args_set_ip_addr": [c_void_p, c_char_p],
+    "nixl_capi_opt_args_set_port": [c_void_p, c_uint16],
+    "nixl_capi_xfer_dlist_get_type": [c_void_p, POINTER(c_int)],
+    "nixl_capi_xfer_dlist_len": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_xfer_dlist_is_empty": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_xfer_dlist_trim": [c_void_p],
+    "nixl_capi_xfer_dlist_rem_desc": [c_void_p, c_int],
+    "nixl_capi_xfer_dlist_resize": [c_void_p, c_size_t],
+    "nixl_capi_xfer_dlist_print": [c_void_p],
+    "nixl_capi_reg_dlist_get_type": [c_void_p, POINTER(c_int)],
+    "nixl_capi_reg_dlist_is_empty": [c_void_p, POINTER(c_bool)],
+    "nixl_capi_reg_dlist_trim": [c_void_p],
+    "nixl_capi_reg_dlist_rem_desc": [c_void_p, c_int],
+    "nixl_capi_reg_dlist_clear": [c_void_p],
+    "nixl_capi_reg_dlist_resize": [c_void_p, c_size_t],
+    "nixl_capi_reg_dlist_print": [c_void_p],
+    "nixl_capi_create_query_resp_list": [POINTER(c_void_p)],
+    "nixl_capi_destroy_query_resp_list": [c_void_p],
+    "nixl_capi_query_resp_list_size": [c_void_p, POINTER(c_size_t)],
+    "nixl_capi_query_resp_list_has_value": [c_void_p, c_size_t, POINTER(c_bool)],
+    "nixl_capi_query_resp_list_get_params": [c_void_p, c_size_t, POINTER(c_void_p)],
+    "nixl_capi_query_mem": [c_void_p, c_void_p, c_void_p, c_void_p],
+    "nixl_capi_send_local_md": [c_void_p, c_void_p],
+    "nixl_capi_send_local_partial_md": [c_void_p, c_void_p, c_void_p],
+    "nixl_capi_fetch_remote_md": [c_void_p, c_char_p, c_void_p],
+    "nixl_capi_invalidate_local_md": [c_void_p, c_void_p],
+    "nixl_capi_is_stub": [],
     "nixl_capi_release_xfer_req": [c_void_p, c_void_p],
     "nixl_capi_destroy_xfer_req": [c_void_p],
 }

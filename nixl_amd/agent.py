@@ -299,23 +299,26 @@ class nixl_agent:
                 m = ctypes.c_int()
                 self._lib.nixl_capi_mem_list_get(mems, i, ctypes.byref(m))
                 mem_names.append(self._MEM_NAMES.get(m.value, "UNKNOWN"))
-            out = {}
-            empty = ctypes.c_bool()
-            self._lib.nixl_capi_params_is_empty(params, ctypes.byref(empty))
-            if not empty.value:
-                it = ctypes.c_void_p()
-                self._lib.nixl_capi_params_create_iterator(params, ctypes.byref(it))
-                more = ctypes.c_bool(True)
-                while more.value:
-                    k, v = ctypes.c_char_p(), ctypes.c_char_p()
-                    if self._lib.nixl_capi_params_iterator_next(it, ctypes.byref(k), ctypes.byref(v), ctypes.byref(more)) != 0:
-                        break
-                    out[k.value.decode()] = v.value.decode()
-                self._lib.nixl_capi_params_destroy_iterator(it)
-            return mem_names, out
+            return mem_names, self._params_to_dict(params)
         finally:
             self._lib.nixl_capi_destroy_mem_list(mems)
             self._lib.nixl_capi_destroy_params(params)
+
+    def _params_to_dict(self, params):
+        out = {}
+        empty = ctypes.c_bool()
+        self._lib.nixl_capi_params_is_empty(params, ctypes.byref(empty))
+        if not empty.value:
+            it = ctypes.c_void_p()
+            self._lib.nixl_capi_params_create_iterator(params, ctypes.byref(it))
+            more = ctypes.c_bool(True)
+            while more.value:
+                k, v = ctypes.c_char_p(), ctypes.c_char_p()
+                if self._lib.nixl_capi_params_iterator_next(it, ctypes.byref(k), ctypes.byref(v), ctypes.byref(more)) != 0:
+                    break
+                out[k.value.decode()] = v.value.decode()
+            self._lib.nixl_capi_params_destroy_iterator(it)
+        return out
 
     def _plugin_query(self, name):
         mems, params = ctypes.c_void_p(), ctypes.c_void_p()
@@ -358,6 +361,38 @@ class nixl_agent:
             return name.value.decode()
         finally:
             self._lib.nixl_capi_destroy_backend(b)
+
+    def query_memory(self, reg_list, backend, mem_type=None):
+        """Reference: _api.py:448-485: per region, what the backend knows about it (a dict) or
+        None.  The HIP backend reports the kind of memory, its device, the size of the
+        allocation around the address and whether the region fits in it."""
+        reg = self.get_reg_descs(reg_list, mem_type)
+        if backend not in self.backends:
+            raise ValueError(f"Backend '{backend}' not found. Available backends: {list(self.backends)}")
+        resp = ctypes.c_void_p()
+        _check("create_query_resp_list", self._lib.nixl_capi_create_query_resp_list(ctypes.byref(resp)))
+        o = self._opt_args([backend])
+        try:
+            _check("query_memory", self._lib.nixl_capi_query_mem(self._h, reg._h, resp, o))
+            n = ctypes.c_size_t()
+            self._lib.nixl_capi_query_resp_list_size(resp, ctypes.byref(n))
+            out = []
+            for i in range(n.value):
+                has = ctypes.c_bool()
+                self._lib.nixl_capi_query_resp_list_has_value(resp, i, ctypes.byref(has))
+                if not has.value:
+                    out.append(None)
+                    continue
+                params = ctypes.c_void_p()
+                _check("query_resp_list_get_params", self._lib.nixl_capi_query_resp_list_get_params(resp, i, ctypes.byref(params)))
+                try:
+                    out.append(self._params_to_dict(params))
+                finally:
+                    self._lib.nixl_capi_destroy_params(params)
+            return out
+        finally:
+            self._free_opt(o)
+            self._lib.nixl_capi_destroy_query_resp_list(resp)
 
     # -- metadata and notifications between agents ------------------------------------------
     def _take_buffer(self, data, size):
@@ -406,7 +441,7 @@ class nixl_agent:
         """Reference: _api.py:471-481."""
         o = self._opt_args(backends)
         try:
-            _check("make_connection", self._lib.nixl_capi_make_connection(self._h, remote_agent.encode(), o))
+            _check("make_connection", self._lib.nixl_capi_agent_make_connection(self._h, remote_agent.encode(), o))
         finally:
             self._free_opt(o)
 

@@ -24,6 +24,9 @@ struct nixl_capi_opt_args_s {
 struct nixl_capi_xfer_dlist_s {
     nixl_xfer_dlist_t *dlist;
 };
+struct nixl_capi_query_resp_list_s {
+    std::vector<nixl_query_resp_t> responses;
+};
 struct nixl_capi_notif_map_s {
     nixl_notifs_t notifs;
 };
@@ -771,7 +774,7 @@ nixl_capi_check_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl
 }
 
 nixl_capi_status_t
-nixl_capi_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args) {
+nixl_capi_agent_make_connection(nixl_capi_agent_t agent, const char *remote_agent, nixl_capi_opt_args_t opt_args) {
     if (!agent || !remote_agent) return NIXL_CAPI_ERROR_INVALID_PARAM;
     return guarded([&] { return fold(agent->inner->makeConnection(remote_agent, opt_args ? &opt_args->args : nullptr)); });
 }
@@ -855,6 +858,224 @@ nixl_capi_notif_map_clear(nixl_capi_notif_map_t map) {
     if (!map) return NIXL_CAPI_ERROR_INVALID_PARAM;
     map->notifs.clear();
     return NIXL_CAPI_SUCCESS;
+}
+
+// ---- the remaining helpers of the reference wrapper ------------------------------------------
+
+nixl_capi_status_t
+nixl_capi_opt_args_get_notif_msg(nixl_capi_opt_args_t args, void **data, size_t *len) {
+    if (!args || !data || !len) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    const nixl_blob_t &msg = args->args.notif.has_value() ? args->args.notif.value() : args->args.notifMsg;
+    *data = nullptr;
+    *len = 0;
+    if (msg.empty()) return NIXL_CAPI_SUCCESS;
+    return copyOut(msg, data, len);
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_get_has_notif(nixl_capi_opt_args_t args, bool *has_notif) {
+    if (!args || !has_notif) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *has_notif = args->args.hasNotif || args->args.notif.has_value();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_get_skip_desc_merge(nixl_capi_opt_args_t args, bool *skip_merge) {
+    if (!args || !skip_merge) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *skip_merge = args->args.skipDescMerge;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_ip_addr(nixl_capi_opt_args_t args, const char *ip_addr) {
+    if (!args || !ip_addr) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        args->args.ipAddr = ip_addr;
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_opt_args_set_port(nixl_capi_opt_args_t args, uint16_t port) {
+    if (!args) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    args->args.port = port;
+    return NIXL_CAPI_SUCCESS;
+}
+
+extern "C++" {
+namespace {
+
+template<typename L>
+nixl_capi_status_t
+listType(L *list, nixl_capi_mem_type_t *mem_type) {
+    if (!list || !mem_type) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *mem_type = static_cast<nixl_capi_mem_type_t>(list->dlist->getType());
+    return NIXL_CAPI_SUCCESS;
+}
+
+template<typename L>
+nixl_capi_status_t
+listEmpty(L *list, bool *is_empty) {
+    if (!list || !is_empty) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *is_empty = list->dlist->isEmpty();
+    return NIXL_CAPI_SUCCESS;
+}
+
+template<typename L, typename F>
+nixl_capi_status_t
+listDo(L *list, F &&f) {
+    if (!list) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        f(*list->dlist);
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+} // namespace
+} // extern "C++"
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_get_type(nixl_capi_xfer_dlist_t dlist, nixl_capi_mem_type_t *mem_type) {
+    return listType(dlist, mem_type);
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_len(nixl_capi_xfer_dlist_t dlist, size_t *len) {
+    if (!dlist || !len) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *len = static_cast<size_t>(dlist->dlist->descCount());
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_is_empty(nixl_capi_xfer_dlist_t dlist, bool *is_empty) {
+    return listEmpty(dlist, is_empty);
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_trim(nixl_capi_xfer_dlist_t dlist) {
+    return listDo(dlist, [](nixl_xfer_dlist_t &l) { (void)l.trim(); });
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_rem_desc(nixl_capi_xfer_dlist_t dlist, int index) {
+    return listDo(dlist, [&](nixl_xfer_dlist_t &l) { l.remDesc(index); });
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_resize(nixl_capi_xfer_dlist_t dlist, size_t new_size) {
+    return listDo(dlist, [&](nixl_xfer_dlist_t &l) { l.resize(new_size); });
+}
+
+nixl_capi_status_t
+nixl_capi_xfer_dlist_print(nixl_capi_xfer_dlist_t dlist) {
+    return listDo(dlist, [](nixl_xfer_dlist_t &l) { l.print(); });
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_get_type(nixl_capi_reg_dlist_t dlist, nixl_capi_mem_type_t *mem_type) {
+    return listType(dlist, mem_type);
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_is_empty(nixl_capi_reg_dlist_t dlist, bool *is_empty) {
+    return listEmpty(dlist, is_empty);
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_trim(nixl_capi_reg_dlist_t dlist) {
+    return listDo(dlist, [](nixl_reg_dlist_t &l) { (void)l.trim(); });
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_rem_desc(nixl_capi_reg_dlist_t dlist, int index) {
+    return listDo(dlist, [&](nixl_reg_dlist_t &l) { l.remDesc(index); });
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_clear(nixl_capi_reg_dlist_t dlist) {
+    return listDo(dlist, [](nixl_reg_dlist_t &l) { l.clear(); });
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_resize(nixl_capi_reg_dlist_t dlist, size_t new_size) {
+    return listDo(dlist, [&](nixl_reg_dlist_t &l) { l.resize(new_size); });
+}
+
+nixl_capi_status_t
+nixl_capi_reg_dlist_print(nixl_capi_reg_dlist_t dlist) {
+    return listDo(dlist, [](nixl_reg_dlist_t &l) { l.print(); });
+}
+
+nixl_capi_status_t
+nixl_capi_create_query_resp_list(nixl_capi_query_resp_list_t *list) {
+    if (!list) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        *list = new nixl_capi_query_resp_list_s;
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_destroy_query_resp_list(nixl_capi_query_resp_list_t list) {
+    if (!list) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    delete list;
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_query_resp_list_size(nixl_capi_query_resp_list_t list, size_t *size) {
+    if (!list || !size) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *size = list->responses.size();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_query_resp_list_has_value(nixl_capi_query_resp_list_t list, size_t index, bool *has_value) {
+    if (!list || !has_value || index >= list->responses.size()) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    *has_value = list->responses[index].has_value();
+    return NIXL_CAPI_SUCCESS;
+}
+
+nixl_capi_status_t
+nixl_capi_query_resp_list_get_params(nixl_capi_query_resp_list_t list, size_t index, nixl_capi_params_t *params) {
+    if (!list || !params || index >= list->responses.size() || !list->responses[index].has_value())
+        return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] {
+        *params = new nixl_capi_params_s{list->responses[index].value()};
+        return NIXL_CAPI_SUCCESS;
+    });
+}
+
+nixl_capi_status_t
+nixl_capi_query_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, nixl_capi_query_resp_list_t resp,
+                    nixl_capi_opt_args_t opt_args) {
+    if (!agent || !descs || !resp) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->queryMem(*descs->dlist, resp->responses, opt_args ? &opt_args->args : nullptr)); });
+}
+
+nixl_capi_status_t
+nixl_capi_send_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t) {
+    return agent ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+}
+
+nixl_capi_status_t
+nixl_capi_send_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, nixl_capi_opt_args_t) {
+    return agent && descs ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+}
+
+nixl_capi_status_t
+nixl_capi_fetch_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_opt_args_t) {
+    return agent && remote_name ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+}
+
+nixl_capi_status_t
+nixl_capi_invalidate_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t) {
+    return agent ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+}
+
+bool
+nixl_capi_is_stub(void) {
+    return false;
 }
 
 } // extern "C"

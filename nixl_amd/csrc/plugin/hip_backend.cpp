@@ -568,6 +568,37 @@ nixlHipEngine::getNotifs(notif_list_t &notif_list) {
 }
 
 nixl_status_t
+nixlHipEngine::queryMem(const nixl_reg_dlist_t &descs, std::vector<nixl_query_resp_t> &resp) const {
+    resp.clear();
+    resp.reserve(static_cast<size_t>(descs.descCount()));
+    for (const nixlBlobDesc &d : descs) {
+        hipPointerAttribute_t attr{};
+        const void *ptr = reinterpret_cast<const void *>(d.addr);
+        if (d.addr == 0 || hipPointerGetAttributes(&attr, ptr) != hipSuccess ||
+            (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeHost)) {
+            (void)hipGetLastError(); // a failed query leaves a sticky error behind
+            resp.emplace_back(std::nullopt);
+            continue;
+        }
+        nixl_b_params_t info;
+        info["type"] = attr.type == hipMemoryTypeDevice ? "device" : "pinned host";
+        info["device"] = std::to_string(attr.device);
+        void *base = nullptr;
+        size_t size = 0;
+        if (hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t *>(&base), &size,
+                                  reinterpret_cast<hipDeviceptr_t>(const_cast<void *>(ptr))) == hipSuccess) {
+            const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+            info["allocation_bytes"] = std::to_string(size);
+            info["fits"] = (d.addr >= b && d.len <= size && d.addr - b <= size - d.len) ? "1" : "0";
+        } else {
+            (void)hipGetLastError();
+        }
+        resp.emplace_back(std::move(info));
+    }
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
 nixlHipEngine::estimateXferCost(const nixl_xfer_op_t &,
                                 const nixl_meta_dlist_t &local,
                                 const nixl_meta_dlist_t &,

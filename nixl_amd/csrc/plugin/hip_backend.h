@@ -156,6 +156,12 @@ public:
     void
     releaseMemView(nixlMemViewH mvh) const override;
 
+    // Per descriptor: what the HIP runtime knows of the address range, or no value if it
+    // does not know it (the reference's storage backends answer "does it exist" the same way,
+    // src/plugins/posix/posix_backend.cpp queryMem).
+    nixl_status_t
+    queryMem(const nixl_reg_dlist_t &descs, std::vector<nixl_query_resp_t> &resp) const override;
+
     nixl_status_t
     estimateXferCost(const nixl_xfer_op_t &operation,
                      const nixl_meta_dlist_t &local,

@@ -319,3 +319,46 @@ def test_agents_used_from_several_threads(oracle_plugin_dir):
         pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
     proc = subprocess.run([exe, oracle_plugin_dir], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
+def test_list_and_option_helpers_of_the_c_wrapper(two_agents):
+    """The descriptor-list, option and stub helpers of the reference's C wrapper
+    (src/bindings/rust/wrapper.h:193-201,297-326,457) behave as their names say; the metadata
+    side channels that need sockets or ETCD answer with an error instead of being absent."""
+    import ctypes
+    from nixl_amd import _lib
+    lib = _lib.agent_lib()
+    a, _ = two_agents
+    buf = np.zeros(4096, np.uint8)
+    x = a.get_xfer_descs(np.array([[buf.ctypes.data, 64, 0], [buf.ctypes.data + 64, 64, 0]], dtype=np.uint64), "DRAM")
+    n, empty, mem = ctypes.c_size_t(), ctypes.c_bool(), ctypes.c_int()
+    assert lib.nixl_capi_xfer_dlist_len(x._h, ctypes.byref(n)) == 0 and n.value == 2
+    assert lib.nixl_capi_xfer_dlist_get_type(x._h, ctypes.byref(mem)) == 0 and mem.value == 0
+    assert lib.nixl_capi_xfer_dlist_rem_desc(x._h, 0) == 0
+    assert lib.nixl_capi_xfer_dlist_rem_desc(x._h, 5) != 0  # out of range: an error, not a crash
+    assert lib.nixl_capi_xfer_dlist_len(x._h, ctypes.byref(n)) == 0 and n.value == 1
+    assert lib.nixl_capi_xfer_dlist_resize(x._h, 3) == 0 and lib.nixl_capi_xfer_dlist_trim(x._h) == 0
+    assert lib.nixl_capi_xfer_dlist_len(x._h, ctypes.byref(n)) == 0 and n.value == 3
+    assert lib.nixl_capi_xfer_dlist_is_empty(x._h, ctypes.byref(empty)) == 0 and not empty.value
+    r = ag.nixl_reg_dlist(np.array([[buf.ctypes.data, 4096, 0]], dtype=np.uint64), 0)
+    assert lib.nixl_capi_reg_dlist_get_type(r._h, ctypes.byref(mem)) == 0 and mem.value == 0
+    assert lib.nixl_capi_reg_dlist_clear(r._h) == 0
+    assert lib.nixl_capi_reg_dlist_is_empty(r._h, ctypes.byref(empty)) == 0 and empty.value
+    o = ctypes.c_void_p()
+    assert lib.nixl_capi_create_opt_args(ctypes.byref(o)) == 0
+    flag, data, size = ctypes.c_bool(True), ctypes.c_void_p(), ctypes.c_size_t()
+    assert lib.nixl_capi_opt_args_get_has_notif(o, ctypes.byref(flag)) == 0 and not flag.value
+    assert lib.nixl_capi_opt_args_get_notif_msg(o, ctypes.byref(data), ctypes.byref(size)) == 0 and not data.value
+    assert lib.nixl_capi_opt_args_set_notif_msg(o, b"m\x00sg", 4) == 0 and lib.nixl_capi_opt_args_set_has_notif(o, True) == 0
+    assert lib.nixl_capi_opt_args_get_notif_msg(o, ctypes.byref(data), ctypes.byref(size)) == 0
+    assert ctypes.string_at(data, size.value) == b"m\x00sg"
+    lib.nixl_capi_free_buffer(data)
+    assert lib.nixl_capi_opt_args_get_has_notif(o, ctypes.byref(flag)) == 0 and flag.value
+    assert lib.nixl_capi_opt_args_set_skip_desc_merge(o, True) == 0
+    assert lib.nixl_capi_opt_args_get_skip_desc_merge(o, ctypes.byref(flag)) == 0 and flag.value
+    assert lib.nixl_capi_opt_args_set_ip_addr(o, b"127.0.0.1") == 0 and lib.nixl_capi_opt_args_set_port(o, 5555) == 0
+    for call in (lambda: lib.nixl_capi_send_local_md(a._h, o), lambda: lib.nixl_capi_fetch_remote_md(a._h, b"beta", o),
+                 lambda: lib.nixl_capi_invalidate_local_md(a._h, o), lambda: lib.nixl_capi_send_local_partial_md(a._h, r._h, o)):
+        assert call() != 0 and a.last_status() == ag.NIXL_ERR_NOT_SUPPORTED
+    lib.nixl_capi_destroy_opt_args(o)
+    assert lib.nixl_capi_is_stub() == 0

@@ -617,6 +617,24 @@ def test_notification_without_initiator_polling(cuda, prog_thread):
     b.close()
 
 
+def test_query_memory(hip_agent, cuda):
+    """query_memory (reference _api.py:448-485): the HIP backend says what the runtime knows of
+    each region, and nothing for an address it does not know."""
+    import torch
+    t = torch.zeros(1 << 20, dtype=torch.uint8, device=cuda)
+    pinned = torch.zeros(4096, dtype=torch.uint8, pin_memory=True)
+    host = np.zeros(4096, np.uint8)
+    got = hip_agent.query_memory(np.array([[t.data_ptr() + 4096, 8192, 0], [t.data_ptr(), 1 << 30, 0],
+                                           [host.ctypes.data, 4096, 0]], dtype=np.uint64), "HIP", "VRAM")
+    assert got[0]["type"] == "device" and got[0]["device"] == "0" and got[0]["fits"] == "1"
+    assert int(got[0]["allocation_bytes"]) >= 1 << 20
+    assert got[1]["fits"] == "0" and got[2] is None
+    got = hip_agent.query_memory(np.array([[pinned.data_ptr(), 4096, 0]], dtype=np.uint64), "HIP", "DRAM")
+    assert got[0]["type"] == "pinned host"
+    with pytest.raises(ValueError):
+        hip_agent.query_memory([t], "UCX")
+
+
 def test_requests_from_several_threads(cuda):
     """The reference calls prepXfer / postXfer / checkXfer / releaseReqH concurrently from
     several threads, one request each (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:
