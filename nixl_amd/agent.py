@@ -495,6 +495,55 @@ class nixl_agent:
         finally:
             self._free_opt(o)
 
+    # -- metadata side channels of the reference (sockets, ETCD): not offered ------------------
+    def _no_side_channel(self, what):
+        raise NixlError(f"{what}: no metadata side channel here; pass get_agent_metadata() to add_remote_agent() by hand",
+                        -1, NIXL_ERR_NOT_SUPPORTED)
+
+    def send_local_metadata(self, ip_addr="", port=0):
+        """Reference: _api.py:909-920."""
+        self._no_side_channel("send_local_metadata")
+
+    def send_partial_agent_metadata(self, descs, inc_conn_info=False, backends=(), ip_addr="", port=0, label=""):
+        """Reference: _api.py:922-951."""
+        self._no_side_channel("send_partial_agent_metadata")
+
+    def fetch_remote_metadata(self, remote_agent, ip_addr="", port=0, label=""):
+        """Reference: _api.py:953-966."""
+        self._no_side_channel("fetch_remote_metadata")
+
+    def invalidate_local_metadata(self, ip_addr="", port=0):
+        """Reference: _api.py:968-977."""
+        self._no_side_channel("invalidate_local_metadata")
+
+    # -- descriptor lists as bytes -------------------------------------------------------------
+    _DESCS_MAGIC = b"NXDL1"
+
+    def get_serialized_descs(self, descs):
+        """Reference: _api.py:1201-1210 (which pickles the list).  Here a flat record that is
+        safe to read back from an untrusted peer: magic, kind, memory type, count, then
+        (addr, len, devId) triples; a registration list is serialised without its blobs."""
+        if isinstance(descs, nixl_xfer_dlist):
+            kind = 1
+        elif isinstance(descs, nixl_reg_dlist):
+            kind = 2
+        else:
+            raise TypeError("get_serialized_descs takes a nixl_xfer_dlist or a nixl_reg_dlist")
+        tri = np.ascontiguousarray(descs.triples, dtype=np.uint64).reshape(-1, 3)
+        return self._DESCS_MAGIC + bytes([kind, descs.mem]) + np.uint64(tri.shape[0]).tobytes() + tri.tobytes()
+
+    def deserialize_descs(self, serialized_descs):
+        """Reference: _api.py:1212-1221."""
+        b = bytes(serialized_descs)
+        m = len(self._DESCS_MAGIC)
+        if len(b) < m + 10 or b[:m] != self._DESCS_MAGIC or b[m] not in (1, 2) or b[m + 1] not in _MEM.values():
+            raise ValueError("not a serialized descriptor list")
+        n = int(np.frombuffer(b, np.uint64, 1, m + 2)[0])
+        if len(b) != m + 10 + 24 * n:
+            raise ValueError("serialized descriptor list has the wrong length")
+        tri = np.frombuffer(b, np.uint64, 3 * n, m + 10).reshape(n, 3).copy()
+        return (nixl_xfer_dlist if b[m] == 1 else nixl_reg_dlist)(tri, b[m + 1])
+
     def prep_mem_view(self, dlist, *, backends=None):
         """Reference: _api.py:728-759.  A local (nixl_xfer_dlist) or remote
         (nixl_remote_dlist) list becomes a table that device code indexes; returns the handle

@@ -362,3 +362,29 @@ def test_list_and_option_helpers_of_the_c_wrapper(two_agents):
         assert call() != 0 and a.last_status() == ag.NIXL_ERR_NOT_SUPPORTED
     lib.nixl_capi_destroy_opt_args(o)
     assert lib.nixl_capi_is_stub() == 0
+
+
+def test_descriptor_lists_as_bytes_and_absent_side_channels(two_agents):
+    """get_serialized_descs / deserialize_descs (reference _api.py:1201-1221; the reference
+    pickles, this build writes a flat record) and the socket / ETCD metadata calls, which say
+    that they are not offered."""
+    a, b = two_agents
+    buf = np.zeros(8192, np.uint8)
+    _reg(b, buf)
+    _reg(a, buf)
+    x = _descs(a, buf, [0, 4096], [100, 200])
+    wire = a.get_serialized_descs(x)
+    y = b.deserialize_descs(wire)
+    assert isinstance(y, ag.nixl_xfer_dlist) and y.mem == x.mem and np.array_equal(y.triples, x.triples)
+    h = b.prep_xfer_dlist("NIXL_INIT_AGENT", y)  # usable as a list
+    h.release()
+    r = ag.nixl_reg_dlist(np.array([[buf.ctypes.data, 8192, 0]], dtype=np.uint64), 0)
+    assert isinstance(a.deserialize_descs(a.get_serialized_descs(r)), ag.nixl_reg_dlist)
+    for bad in (b"", wire[:-1], b"XXXXX" + wire[5:], wire + b"\x00", wire[:5] + bytes([9]) + wire[6:]):
+        with pytest.raises(ValueError):
+            a.deserialize_descs(bad)
+    for call in (a.send_local_metadata, lambda: a.fetch_remote_metadata("beta"), a.invalidate_local_metadata,
+                 lambda: a.send_partial_agent_metadata(r)):
+        with pytest.raises(ag.NixlError) as e:
+            call()
+        assert e.value.status == ag.NIXL_ERR_NOT_SUPPORTED
