@@ -126,6 +126,15 @@ public:
     invalidateRemoteMD(const std::string &remote_agent);
     nixl_status_t
     checkRemoteMD(const std::string remote_name, const nixl_xfer_dlist_t &descs) const;
+    // The side channels themselves: declared so that callers link; NIXL_ERR_NOT_SUPPORTED.
+    nixl_status_t
+    sendLocalMD(const nixl_opt_args_t *extra_params = nullptr) const;
+    nixl_status_t
+    sendLocalPartialMD(const nixl_reg_dlist_t &descs, const nixl_opt_args_t *extra_params = nullptr) const;
+    nixl_status_t
+    fetchRemoteMD(const std::string remote_name, const nixl_opt_args_t *extra_params = nullptr);
+    nixl_status_t
+    invalidateLocalMD(const nixl_opt_args_t *extra_params = nullptr) const;
 };
 
 #endif // NIXL_AMD_AGENT_API_H

@@ -1482,3 +1482,26 @@ nixlAgent::checkRemoteMD(const std::string remote_name, const nixl_xfer_dlist_t 
     }
     return NIXL_ERR_NOT_FOUND;
 }
+
+// ---- metadata side channels of the reference (listener thread, sockets, ETCD;
+// src/core/nixl_agent.cpp:1838-1860, src/core/nixl_listener.cpp): not part of this build ----
+
+nixl_status_t
+nixlAgent::sendLocalMD(const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::sendLocalPartialMD(const nixl_reg_dlist_t &, const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::fetchRemoteMD(const std::string, const nixl_opt_args_t *) {
+    return NIXL_ERR_NOT_SUPPORTED;
+}
+
+nixl_status_t
+nixlAgent::invalidateLocalMD(const nixl_opt_args_t *) const {
+    return NIXL_ERR_NOT_SUPPORTED;
+}

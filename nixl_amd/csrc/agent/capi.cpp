@@ -1054,23 +1054,25 @@ nixl_capi_query_mem(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, nixl_c
 }
 
 nixl_capi_status_t
-nixl_capi_send_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t) {
-    return agent ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+nixl_capi_send_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t opt_args) {
+    return agent ? fold(agent->inner->sendLocalMD(opt_args ? &opt_args->args : nullptr)) : NIXL_CAPI_ERROR_INVALID_PARAM;
 }
 
 nixl_capi_status_t
-nixl_capi_send_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, nixl_capi_opt_args_t) {
-    return agent && descs ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+nixl_capi_send_local_partial_md(nixl_capi_agent_t agent, nixl_capi_reg_dlist_t descs, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !descs) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return fold(agent->inner->sendLocalPartialMD(*descs->dlist, opt_args ? &opt_args->args : nullptr));
 }
 
 nixl_capi_status_t
-nixl_capi_fetch_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_opt_args_t) {
-    return agent && remote_name ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+nixl_capi_fetch_remote_md(nixl_capi_agent_t agent, const char *remote_name, nixl_capi_opt_args_t opt_args) {
+    if (!agent || !remote_name) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    return guarded([&] { return fold(agent->inner->fetchRemoteMD(remote_name, opt_args ? &opt_args->args : nullptr)); });
 }
 
 nixl_capi_status_t
-nixl_capi_invalidate_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t) {
-    return agent ? fold(NIXL_ERR_NOT_SUPPORTED) : NIXL_CAPI_ERROR_INVALID_PARAM;
+nixl_capi_invalidate_local_md(nixl_capi_agent_t agent, nixl_capi_opt_args_t opt_args) {
+    return agent ? fold(agent->inner->invalidateLocalMD(opt_args ? &opt_args->args : nullptr)) : NIXL_CAPI_ERROR_INVALID_PARAM;
 }
 
 bool
