@@ -443,6 +443,9 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
 // the same bytes were isolated 32-byte stores and cost five times as long.
 constexpr int kHtMetaThreads = 256;
 
+// VEC: selections moved four at a time and the (rank, token) pair in one store; the host
+// picks it when K is a multiple of 4 and every pointer is 16-byte aligned.
+template <bool VEC>
 __global__ void __launch_bounds__(kHtMetaThreads)
 ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
                float *__restrict__ recv_topk_weights,
@@ -464,7 +467,23 @@ ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
     const long long row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
     if (row < row_offset[dst] || row >= row_offset[dst + 1]) return;
     const int El = d.E / d.R;
-    if (recv_topk_idx)
+    if (VEC && recv_topk_idx) {
+        // four selections a step: 16-byte loads and stores (tok*K and row*K are multiples of 4)
+        const int lo = dst * El, hi = lo + El;
+        for (int k = 0; k < d.K; k += 4) {
+            const int4 sel = *reinterpret_cast<const int4 *>(topk_idx + tok * d.K + k);
+            const bool l0 = sel.x >= lo && sel.x < hi, l1 = sel.y >= lo && sel.y < hi;
+            const bool l2 = sel.z >= lo && sel.z < hi, l3 = sel.w >= lo && sel.w < hi;
+            *reinterpret_cast<int4 *>(recv_topk_idx + row * d.K + k) =
+                make_int4(l0 ? sel.x - lo : -1, l1 ? sel.y - lo : -1, l2 ? sel.z - lo : -1, l3 ? sel.w - lo : -1);
+            if (recv_topk_weights) {
+                float4 w = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (topk_weights) w = *reinterpret_cast<const float4 *>(topk_weights + tok * d.K + k);
+                *reinterpret_cast<float4 *>(recv_topk_weights + row * d.K + k) =
+                    make_float4(l0 ? w.x : 0.f, l1 ? w.y : 0.f, l2 ? w.z : 0.f, l3 ? w.w : 0.f);
+            }
+        }
+    } else if (recv_topk_idx)
         for (int k = 0; k < d.K; ++k) {
             const int sel = topk_idx[tok * d.K + k];
             const bool local = sel >= dst * El && sel < (dst + 1) * El;
@@ -472,8 +491,12 @@ ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
             if (recv_topk_weights) recv_topk_weights[row * d.K + k] = local && topk_weights ? topk_weights[tok * d.K + k] : 0.f;
         }
     if (recv_src_meta) {
-        recv_src_meta[row * 2] = r;
-        recv_src_meta[row * 2 + 1] = t;
+        if (VEC) {
+            *reinterpret_cast<int2 *>(recv_src_meta + row * 2) = make_int2(r, t);
+        } else {
+            recv_src_meta[row * 2] = r;
+            recv_src_meta[row * 2 + 1] = t;
+        }
     }
 }
 
@@ -778,7 +801,11 @@ nixl_amd_ep_ht_dispatch(void *recv_x,
         const long long blocks = static_cast<long long>(num_ranks) * num_ranks * ((num_tokens + kHtMetaThreads - 1) / kHtMetaThreads);
         if (blocks >= (1ll << 31)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many ranks and tokens");
         const dim3 grid(static_cast<unsigned>(blocks));
-        hipLaunchKernelGGL(ht_meta_kernel, grid, dim3(kHtMetaThreads), 0, s, recv_topk_idx, recv_topk_weights, recv_src_meta,
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(recv_topk_idx) | reinterpret_cast<uintptr_t>(recv_topk_weights) |
+                               reinterpret_cast<uintptr_t>(recv_src_meta) | reinterpret_cast<uintptr_t>(topk_idx) |
+                               reinterpret_cast<uintptr_t>(topk_weights);
+        const auto kernel = (num_topk % 4 == 0 && bits % 16 == 0) ? ht_meta_kernel<true> : ht_meta_kernel<false>;
+        hipLaunchKernelGGL(kernel, grid, dim3(kHtMetaThreads), 0, s, recv_topk_idx, recv_topk_weights, recv_src_meta,
                            topk_idx, topk_weights, is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
                            reinterpret_cast<const long long *>(recv_row_offset), d);
     }
