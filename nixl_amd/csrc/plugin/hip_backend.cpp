@@ -183,15 +183,10 @@ nixlHipEngine::reapRetired(bool wait) const {
     size_t keep = 0;
     for (nixlHipReqH *r : retired_) {
         const DeviceScope on_device(r->device);
-        bool finished = true;
-        if (r->posted) {
-            if (wait)
-                (void)hipEventSynchronize(r->done);
-            else
-                finished = (hipEventQuery(r->done) != hipErrorNotReady);
-        }
-        if (finished) {
-            deliverPending(r);
+        hipError_t state = hipSuccess;
+        if (r->posted) state = wait ? hipEventSynchronize(r->done) : hipEventQuery(r->done);
+        if (state != hipErrorNotReady) {
+            deliverPending(r, state == hipSuccess);
             delete r;
         } else
             retired_[keep++] = r;
@@ -346,9 +341,12 @@ nixlHipEngine::postXfer(const nixl_xfer_op_t &,
     if (!req || !req->plan) return NIXL_ERR_INVALID_PARAM;
     const DeviceScope on_device(req->device);
     if (!on_device.ok()) return NIXL_ERR_BACKEND;
-    if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
-    // the notification of an earlier post that nobody polled to completion goes out first
-    deliverPending(req);
+    if (req->posted) {
+        const hipError_t earlier = hipEventQuery(req->done);
+        if (earlier == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
+        // the notification of an earlier post that nobody polled to completion goes out first
+        deliverPending(req, earlier == hipSuccess);
+    }
 
     if (nixl_amd_copy_plan_launch(req->plan, req->stream) != NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
@@ -380,10 +378,11 @@ nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
     const hipError_t e = hipEventQuery(req->done);
     if (e == hipSuccess) {
         // the peer learns of the transfer only after its bytes have landed
-        deliverPending(req);
+        deliverPending(req, true);
         return NIXL_SUCCESS;
     }
     if (e == hipErrorNotReady) return NIXL_IN_PROG;
+    deliverPending(req, false);
     NIXL_ERROR << "HIP backend: transfer failed: " << hipGetErrorString(e);
     return NIXL_ERR_BACKEND;
 }
@@ -393,14 +392,15 @@ nixlHipEngine::releaseReqH(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_SUCCESS;
     const DeviceScope on_device(req->device);
-    if (req->posted && hipEventQuery(req->done) == hipErrorNotReady) {
+    const hipError_t state = req->posted ? hipEventQuery(req->done) : hipSuccess;
+    if (state == hipErrorNotReady) {
         // A launched kernel cannot be cancelled; keep its plan alive until it has
         // drained and free it from a later call, so that this call never blocks.
         std::lock_guard<std::mutex> lock(retiredMutex_);
         retired_.push_back(req);
         return NIXL_SUCCESS;
     }
-    if (req->posted) deliverPending(req);
+    deliverPending(req, state == hipSuccess);
     delete req;
     return NIXL_SUCCESS;
 }
@@ -414,8 +414,11 @@ nixlHipEngine::knowsAgent(const std::string &name) const {
     return std::find(peers_.begin(), peers_.end(), name) != peers_.end();
 }
 
+// Takes the request off the progress thread's list and, if its copy completed, queues its
+// message at the target.  The message of a copy that failed is dropped: the peer must not
+// read bytes that never arrived.
 void
-nixlHipEngine::deliverPending(nixlHipReqH *req) const {
+nixlHipEngine::deliverPending(nixlHipReqH *req, bool completed) const {
     std::string target, msg;
     {
         std::lock_guard<std::mutex> lock(pendingMutex_);
@@ -425,6 +428,10 @@ nixlHipEngine::deliverPending(nixlHipReqH *req) const {
         msg = req->notifMsg;
         const auto it = std::find(watched_.begin(), watched_.end(), req);
         if (it != watched_.end()) watched_.erase(it);
+    }
+    if (!completed) {
+        NIXL_ERROR << "HIP backend: transfer failed, notification for agent '" << target << "' dropped";
+        return;
     }
     if (genNotif(target, msg) != NIXL_SUCCESS)
         NIXL_WARN << "HIP backend: notification for agent '" << target << "' could not be delivered";
@@ -446,12 +453,17 @@ nixlHipEngine::progressLoop() {
             for (size_t i = 0; i < watched_.size();) {
                 nixlHipReqH *req = watched_[i];
                 const DeviceScope on_device(req->device);
-                if (hipEventQuery(req->done) == hipErrorNotReady) {
+                const hipError_t state = hipEventQuery(req->done);
+                if (state == hipErrorNotReady) {
                     ++i;
                     continue;
                 }
                 req->notifPending = false;
-                ready.emplace_back(req->notifTarget, req->notifMsg);
+                if (state == hipSuccess)
+                    ready.emplace_back(req->notifTarget, req->notifMsg);
+                else
+                    NIXL_ERROR << "HIP backend: transfer failed, notification for agent '" << req->notifTarget
+                               << "' dropped";
                 watched_[i] = watched_.back();
                 watched_.pop_back();
             }

@@ -181,7 +181,7 @@ private:
     bool
     knowsAgent(const std::string &name) const;
     void
-    deliverPending(nixlHipReqH *req) const;
+    deliverPending(nixlHipReqH *req, bool completed) const;
     void
     progressLoop();
     struct viewEntry {
