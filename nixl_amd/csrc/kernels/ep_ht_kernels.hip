@@ -318,18 +318,36 @@ ht_prefix_kernel(const int *__restrict__ channel_prefix,
                  int alignment) {
     __shared__ int wave_sums[kScanThreads / kWaveSize];
     const int tid = threadIdx.x;
+    // Loads go out eight at a time before anything depends on them: issued one by one, the
+    // round trips of this single workgroup add up to most of the kernel's time.
+    constexpr int kBatch = 8;
     for (int e = tid; e < E; e += kScanThreads) {
         int n = 0;
-        for (int r = 0; r < R; ++r)
-            n += per_expert[static_cast<size_t>(r) * E + e];
+        for (int r0 = 0; r0 < R; r0 += kBatch) {
+            int v[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                v[j] = r0 + j < R ? per_expert[static_cast<size_t>(r0 + j) * E + e] : 0;
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                n += v[j];
+        }
         recv_expert_count[e] = (n + alignment - 1) / alignment * alignment;
     }
     // R <= kScanThreads: thread d owns destination d
     int total = 0;
     if (tid < R) {
-        for (int r = 0; r < R; ++r) {
-            total += channel_prefix[(static_cast<size_t>(r) * R + tid) * C + (C - 1)];
-            recv_rank_prefix[tid * R + r] = total;
+        for (int r0 = 0; r0 < R; r0 += kBatch) {
+            int v[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                v[j] = r0 + j < R ? channel_prefix[(static_cast<size_t>(r0 + j) * R + tid) * C + (C - 1)] : 0;
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                if (r0 + j < R) {
+                    total += v[j];
+                    recv_rank_prefix[tid * R + r0 + j] = total;
+                }
         }
         if (recv_counter) recv_counter[tid] = total;
     }
