@@ -447,6 +447,26 @@ def test_config3_small_descriptor_stress_full_size(hip_agent, cuda):
         h.release()
 
 
+def test_descriptors_longer_than_4_gib(cuda):
+    """Two descriptors whose lengths do not fit in 32 bits: one 16-byte aligned (streamed in
+    1 KiB chunks, chunk offsets beyond 2^32) and one that starts and ends on odd bytes (cut
+    into byte-range items).  Canary bytes around both destinations."""
+    import torch
+    big = (4 << 30) + (3 << 20)
+    odd = (4 << 30) + 12345
+    src = torch.empty((big + odd + 64 + 7) // 8 * 8, dtype=torch.uint8, device=cuda)
+    src.view(torch.int64).random_()
+    dst = torch.full((big + odd + 4096,), 0x5A, dtype=torch.uint8, device=cuda)
+    d0, d1 = 1024, 1024 + big + 1031  # the second destination starts on an odd byte
+    s0, s1 = 0, big + 7
+    plan = _plan([(src.data_ptr() + s0, dst.data_ptr() + d0, big), (src.data_ptr() + s1, dst.data_ptr() + d1, odd)])
+    _run_plan(torch, plan)
+    assert _lib.kernels().nixl_amd_copy_plan_destroy(plan) == 0
+    assert torch.equal(dst[d0:d0 + big], src[s0:s0 + big])
+    assert torch.equal(dst[d1:d1 + odd], src[s1:s1 + odd])
+    assert bool((dst[:d0] == 0x5A).all()) and bool((dst[d0 + big:d1] == 0x5A).all()) and bool((dst[d1 + odd:] == 0x5A).all())
+
+
 def test_golden_descriptor_list(cuda):
     """Committed vector (tests/golden/kv_descs.npz): mixed aligned / unaligned / empty
     descriptors, destination pre-filled with a canary byte."""
