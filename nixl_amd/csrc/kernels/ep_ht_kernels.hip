@@ -458,7 +458,7 @@ ht_dispatch_kernel(uint16_t *__restrict__ recv_x,
 // token.  grid = R * R * ceil(T / 256): (source, destination) pairs major, one token per
 // thread.  Consecutive tokens that go to the destination occupy consecutive rows,
 // so a wave writes a contiguous stretch of each array; written from the row kernel above,
-// the same bytes were isolated 32-byte stores and cost five times as long.
+// the same bytes were isolated 32-byte stores and cost several times as long.
 constexpr int kHtMetaThreads = 256;
 
 // VEC: selections moved four at a time and the (rank, token) pair in one store; the host
