@@ -207,6 +207,48 @@ nixl_amd_ep_ht_dispatch(void *recv_x,
                         void *stream);
 
 /*
+ * Normal-mode dispatch of rows of any element type, with optional per-token scales: the
+ * (x, x_scales) form of ht::dispatch, which the reference uses for fp8 rows
+ * (csrc/nixl_ep.cpp:701-711 argument checks, :840-857 launch; kernels/nixl_ep_ht.cu:729 reads
+ * scale i of a token at token * scale_token_stride + i * scale_hidden_stride, :1198-1209
+ * writes recv_x_scales densely as [total][num_scales]).
+ *   x, recv_x          rows of `hidden` elements of `elem_bytes` (1, 2 or 4) bytes; a row is a
+ *                      multiple of 16 bytes and at most 16 KiB
+ *   x_scales           32-bit words (fp32, or packed UE8M0 as int32), addressed as
+ *                      rank * scale_rank_stride + token * scale_token_stride +
+ *                      i * scale_hidden_stride (strides in words, so that a transposed
+ *                      tensor can be passed as it is); NULL with num_scales 0 for no scales
+ *   recv_x_scales      [total][num_scales] words, row order as recv_x
+ * Everything else as nixl_amd_ep_ht_dispatch, which is this call with elem_bytes 2 and no
+ * scales.
+ */
+int
+nixl_amd_ep_ht_dispatch_scaled(void *recv_x,
+                               void *recv_x_scales,
+                               int32_t *recv_topk_idx,
+                               float *recv_topk_weights,
+                               int32_t *recv_src_meta,
+                               const void *x,
+                               const void *x_scales,
+                               const int32_t *topk_idx,
+                               const float *topk_weights,
+                               const uint8_t *is_token_in_rank,
+                               const int *recv_gbl_rank_prefix_sum,
+                               const int *send_head,
+                               const int64_t *recv_row_offset,
+                               int num_tokens,
+                               int hidden,
+                               int elem_bytes,
+                               int num_scales,
+                               int64_t scale_rank_stride,
+                               int64_t scale_token_stride,
+                               int64_t scale_hidden_stride,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               void *stream);
+
+/*
  * Normal-mode combine.  Replaces ht::combine with one reduction stage
  * (kernels/api.cuh:176-203; combine_token, kernels/nixl_ep_ht.cu:1682-1737):
  * combined_x[r][t] = bf16( float(bias_0) + float(bias_1) + sum over destination ranks that

@@ -83,6 +83,7 @@ _EP_SIGS = {
     "nixl_amd_ep_get_dispatch_layout": [c_void_p] * 4 + [c_int] * 4 + [c_void_p],
     "nixl_amd_ep_ht_notify_dispatch": [c_void_p] * 8 + [c_int] * 5 + [c_void_p],
     "nixl_amd_ep_ht_dispatch": [c_void_p] * 11 + [c_int] * 5 + [c_void_p],
+    "nixl_amd_ep_ht_dispatch_scaled": [c_void_p] * 13 + [c_int] * 4 + [c_int64] * 3 + [c_int] * 3 + [c_void_p],
     "nixl_amd_ep_ht_combine": [c_void_p] * 10 + [c_int] * 4 + [c_void_p],
     "nixl_amd_ep_router_topk": [c_void_p] * 3 + [c_int] * 3 + [c_void_p],
     "nixl_amd_ep_f32_to_e4m3": [c_void_p, c_void_p, c_size_t, c_void_p],

@@ -518,6 +518,97 @@ ht_meta_kernel(int32_t *__restrict__ recv_topk_idx,
     }
 }
 
+// Per-token scales that travel with the rows (kernels/nixl_ep_ht.cu:729 reads them at
+// token * scale_token_stride + i * scale_hidden_stride, :1198-1209 writes them densely per
+// received row).  grid = R * R * ceil(T / 64): the first wave resolves the rows of 64
+// consecutive tokens of one (source, destination) pair into LDS; the workgroup then moves
+// their scales through an LDS tile of 64 tokens x 64 scales.  The tile is filled along
+// whichever index is contiguous in the source (tokens, for the transposed storage the
+// reference's callers pass; scales otherwise) and drained along the scales, so that a wave
+// reads and writes consecutive addresses either way (consecutive tokens that go to the
+// destination occupy consecutive rows).  Scales are moved as 32-bit words whatever they
+// hold (fp32 or packed UE8M0).
+constexpr int kHtScaleTokens = 64;
+constexpr int kHtScaleTile = 64;
+constexpr int kHtScaleThreads = 256;
+
+__global__ void __launch_bounds__(kHtScaleThreads)
+ht_row_scales_kernel(uint32_t *__restrict__ recv_scales,
+                     const uint32_t *__restrict__ scales,
+                     const uint8_t *__restrict__ in_rank,
+                     const int *__restrict__ prefix,
+                     const int *__restrict__ send_head,
+                     const long long *__restrict__ row_offset,
+                     HtDims d,
+                     int S,
+                     long long rank_stride,
+                     long long token_stride,
+                     long long scale_stride,
+                     int wide) {
+    __shared__ long long rows[kHtScaleTokens];
+    __shared__ uint32_t tile[kHtScaleTokens][kHtScaleTile + 1]; // odd pitch: no bank conflicts either way
+    const int blocks_per_pair = (d.T + kHtScaleTokens - 1) / kHtScaleTokens;
+    const int pair = blockIdx.x / blocks_per_pair;
+    const int r = pair / d.R, dst = pair % d.R;
+    const int t0 = (blockIdx.x % blocks_per_pair) * kHtScaleTokens;
+    const int tid = threadIdx.x;
+    if (tid < kHtScaleTokens) {
+        const int t = t0 + tid;
+        long long row = -1;
+        if (t < d.T && in_rank[(static_cast<size_t>(r) * d.T + t) * d.R + dst]) {
+            row = recv_row(prefix, send_head, row_offset, d, r, t, dst);
+            if (row < row_offset[dst] || row >= row_offset[dst + 1]) row = -1;
+        }
+        rows[tid] = row;
+    }
+    __syncthreads();
+    const uint32_t *__restrict__ src = scales + static_cast<long long>(r) * rank_stride;
+    const bool tokens_contiguous = token_stride < scale_stride;
+    for (int g0 = 0; g0 < S; g0 += kHtScaleTile) {
+        const int gs = min(kHtScaleTile, S - g0);
+        // every load of the tile is issued before the first value is used: one load, one
+        // LDS write at a time, the round trips of the 16 steps add up
+        constexpr int kSteps = kHtScaleTokens * kHtScaleTile / kHtScaleThreads;
+        uint32_t v[kSteps];
+        int at[kSteps];
+#pragma unroll
+        for (int k = 0; k < kSteps; ++k) {
+            const int i = tid + k * kHtScaleThreads;
+            const int j = tokens_contiguous ? i % kHtScaleTokens : i / gs;
+            const int g = tokens_contiguous ? i / kHtScaleTokens : i - j * gs;
+            at[k] = -1;
+            v[k] = 0;
+            if (i < kHtScaleTokens * gs && rows[j] >= 0) {
+                at[k] = j * (kHtScaleTile + 1) + g;
+                v[k] = src[static_cast<long long>(t0 + j) * token_stride + static_cast<long long>(g0 + g) * scale_stride];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kSteps; ++k)
+            if (at[k] >= 0) (&tile[0][0])[at[k]] = v[k];
+        __syncthreads();
+        if (wide) {
+            // four scales a store: the isolated 4-byte stores of the narrow form run at a
+            // fraction of the rate
+            const int quads = gs / 4;
+            for (int i = tid; i < kHtScaleTokens * quads; i += kHtScaleThreads) {
+                const int j = i / quads, q = (i - j * quads) * 4;
+                const long long row = rows[j];
+                if (row >= 0)
+                    *reinterpret_cast<uint4 *>(recv_scales + row * S + g0 + q) =
+                        make_uint4(tile[j][q], tile[j][q + 1], tile[j][q + 2], tile[j][q + 3]);
+            }
+        } else {
+            for (int i = tid; i < kHtScaleTokens * gs; i += kHtScaleThreads) {
+                const int j = i / gs, g = i - j * gs;
+                const long long row = rows[j];
+                if (row >= 0) recv_scales[row * S + g0 + g] = tile[j][g];
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // ---- combine (combine_token, kernels/nixl_ep_ht.cu:1682-1737) -----------------------------------
 __global__ void __launch_bounds__(1024)
 ht_combine_kernel(uint16_t *__restrict__ combined,
@@ -781,6 +872,87 @@ nixl_amd_ep_ht_notify_dispatch(const uint8_t *is_token_in_rank,
 }
 
 int
+nixl_amd_ep_ht_dispatch_scaled(void *recv_x,
+                               void *recv_x_scales,
+                               int32_t *recv_topk_idx,
+                               float *recv_topk_weights,
+                               int32_t *recv_src_meta,
+                               const void *x,
+                               const void *x_scales,
+                               const int32_t *topk_idx,
+                               const float *topk_weights,
+                               const uint8_t *is_token_in_rank,
+                               const int *recv_gbl_rank_prefix_sum,
+                               const int *send_head,
+                               const int64_t *recv_row_offset,
+                               int num_tokens,
+                               int hidden,
+                               int elem_bytes,
+                               int num_scales,
+                               int64_t scale_rank_stride,
+                               int64_t scale_token_stride,
+                               int64_t scale_hidden_stride,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               void *stream) {
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: elem_bytes must be 1, 2 or 4");
+    if (hidden <= 0) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: hidden must be positive");
+    if ((static_cast<long long>(hidden) * elem_bytes) % 16 != 0)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: a row must be a multiple of 16 bytes");
+    // the row kernels count a row in 2-byte elements, whatever it holds
+    const long long row_halves = static_cast<long long>(hidden) * elem_bytes / 2;
+    if (row_halves > 8192) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: a row may hold at most 16 KiB");
+    const int rc = check_ht("ht_dispatch", num_tokens, static_cast<int>(row_halves), num_topk, num_ranks, num_experts);
+    if (rc) return rc;
+    if (!recv_x || !x || !is_token_in_rank || !recv_gbl_rank_prefix_sum || !send_head || !recv_row_offset)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: null pointer argument");
+    if (recv_topk_idx && !topk_idx) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: recv_topk_idx without topk_idx");
+    if (num_scales < 0 || num_scales > 4096) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: num_scales must be in [0, 4096]");
+    if ((x_scales != nullptr) != (recv_x_scales != nullptr) || (x_scales && num_scales == 0))
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: x_scales, recv_x_scales and num_scales go together");
+    if (x_scales && (scale_rank_stride < 0 || scale_token_stride < 0 || scale_hidden_stride < 0))
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: negative scale stride");
+    const HtDims d{num_ranks, num_tokens, static_cast<int>(row_halves), num_topk, num_experts};
+    const int lanes = round_up_wave(d.H / 8);
+    const int parts = (lanes + kHtDispatchLanes - 1) / kHtDispatchLanes;
+    if (static_cast<long long>(num_ranks) * num_tokens * parts >= (1ll << 31))
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many tokens");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens * parts), dim3(kHtDispatchLanes),
+                       static_cast<size_t>(num_ranks) * 12, s, static_cast<uint16_t *>(recv_x),
+                       static_cast<const uint16_t *>(x), is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                       reinterpret_cast<const long long *>(recv_row_offset), d, parts);
+    HIP_TRY(hipGetLastError());
+    if (x_scales) {
+        const long long blocks = static_cast<long long>(num_ranks) * num_ranks * ((num_tokens + kHtScaleTokens - 1) / kHtScaleTokens);
+        if (blocks >= (1ll << 31)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many ranks and tokens");
+        hipLaunchKernelGGL(ht_row_scales_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kHtScaleThreads), 0, s,
+                           static_cast<uint32_t *>(recv_x_scales), static_cast<const uint32_t *>(x_scales), is_token_in_rank,
+                           recv_gbl_rank_prefix_sum, send_head, reinterpret_cast<const long long *>(recv_row_offset), d,
+                           num_scales, static_cast<long long>(scale_rank_stride), static_cast<long long>(scale_token_stride),
+                           static_cast<long long>(scale_hidden_stride),
+                           (num_scales % 4 == 0 && reinterpret_cast<uintptr_t>(recv_x_scales) % 16 == 0) ? 1 : 0);
+        HIP_TRY(hipGetLastError());
+    }
+    if (recv_topk_idx || recv_src_meta) {
+        const long long blocks = static_cast<long long>(num_ranks) * num_ranks * ((num_tokens + kHtMetaThreads - 1) / kHtMetaThreads);
+        if (blocks >= (1ll << 31)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many ranks and tokens");
+        const dim3 grid(static_cast<unsigned>(blocks));
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(recv_topk_idx) | reinterpret_cast<uintptr_t>(recv_topk_weights) |
+                               reinterpret_cast<uintptr_t>(recv_src_meta) | reinterpret_cast<uintptr_t>(topk_idx) |
+                               reinterpret_cast<uintptr_t>(topk_weights);
+        const auto kernel = (num_topk % 4 == 0 && bits % 16 == 0) ? ht_meta_kernel<true> : ht_meta_kernel<false>;
+        hipLaunchKernelGGL(kernel, grid, dim3(kHtMetaThreads), 0, s, recv_topk_idx, recv_topk_weights, recv_src_meta,
+                           topk_idx, topk_weights, is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
+                           reinterpret_cast<const long long *>(recv_row_offset), d);
+    }
+    HIP_TRY(hipGetLastError());
+    return NIXL_AMD_OK;
+}
+
+int
 nixl_amd_ep_ht_dispatch(void *recv_x,
                         int32_t *recv_topk_idx,
                         float *recv_topk_weights,
@@ -798,37 +970,9 @@ nixl_amd_ep_ht_dispatch(void *recv_x,
                         int num_ranks,
                         int num_experts,
                         void *stream) {
-    const int rc = check_ht("ht_dispatch", num_tokens, hidden, num_topk, num_ranks, num_experts);
-    if (rc) return rc;
-    if (hidden == 0) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: hidden must be positive");
-    if (!recv_x || !x || !is_token_in_rank || !recv_gbl_rank_prefix_sum || !send_head || !recv_row_offset)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: null pointer argument");
-    if (recv_topk_idx && !topk_idx) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ht_dispatch: recv_topk_idx without topk_idx");
-    const HtDims d{num_ranks, num_tokens, hidden, num_topk, num_experts};
-    const int lanes = round_up_wave(hidden / 8);
-    const int parts = (lanes + kHtDispatchLanes - 1) / kHtDispatchLanes;
-    if (static_cast<long long>(num_ranks) * num_tokens * parts >= (1ll << 31))
-        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many tokens");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(ht_dispatch_kernel, dim3(static_cast<unsigned>(num_ranks) * num_tokens * parts), dim3(kHtDispatchLanes),
-                       static_cast<size_t>(num_ranks) * 12, s, static_cast<uint16_t *>(recv_x),
-                       static_cast<const uint16_t *>(x), is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
-                       reinterpret_cast<const long long *>(recv_row_offset), d, parts);
-    HIP_TRY(hipGetLastError());
-    if (recv_topk_idx || recv_src_meta) {
-        const long long blocks = static_cast<long long>(num_ranks) * num_ranks * ((num_tokens + kHtMetaThreads - 1) / kHtMetaThreads);
-        if (blocks >= (1ll << 31)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ht_dispatch: too many ranks and tokens");
-        const dim3 grid(static_cast<unsigned>(blocks));
-        const uintptr_t bits = reinterpret_cast<uintptr_t>(recv_topk_idx) | reinterpret_cast<uintptr_t>(recv_topk_weights) |
-                               reinterpret_cast<uintptr_t>(recv_src_meta) | reinterpret_cast<uintptr_t>(topk_idx) |
-                               reinterpret_cast<uintptr_t>(topk_weights);
-        const auto kernel = (num_topk % 4 == 0 && bits % 16 == 0) ? ht_meta_kernel<true> : ht_meta_kernel<false>;
-        hipLaunchKernelGGL(kernel, grid, dim3(kHtMetaThreads), 0, s, recv_topk_idx, recv_topk_weights, recv_src_meta,
-                           topk_idx, topk_weights, is_token_in_rank, recv_gbl_rank_prefix_sum, send_head,
-                           reinterpret_cast<const long long *>(recv_row_offset), d);
-    }
-    HIP_TRY(hipGetLastError());
-    return NIXL_AMD_OK;
+    return nixl_amd_ep_ht_dispatch_scaled(recv_x, nullptr, recv_topk_idx, recv_topk_weights, recv_src_meta, x, nullptr, topk_idx,
+                                          topk_weights, is_token_in_rank, recv_gbl_rank_prefix_sum, send_head, recv_row_offset,
+                                          num_tokens, hidden, 2, 0, 0, 0, 0, num_topk, num_ranks, num_experts, stream);
 }
 
 int

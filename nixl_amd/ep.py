@@ -85,8 +85,6 @@ class Buffer:
     every rank, and no RDMA buffer sizing because no staging buffers exist.
     """
 
-    num_sms = 20  # kept for API parity (buffer.py:57); the kernels size their own grids
-
     num_sms = 20  # reference default (buffer.py:54); see Config
 
     @staticmethod
@@ -389,34 +387,62 @@ class Buffer:
                     is_token_in_rank=None, num_tokens_per_expert=None, topk_idx=None, topk_weights=None,
                     expert_alignment=1, num_channels=None, previous_event=None, async_finish=False,
                     allocate_on_comm_stream=False, config=None):
-        """Reference: buffer.py:526-660, csrc/nixl_ep.cpp:615-898 (bf16 rows).
+        """Reference: buffer.py:526-660, csrc/nixl_ep.cpp:615-898.
 
-        x [R, T, H]; the layout tensors come from get_dispatch_layout.  Returns
-        (recv_x, recv_topk_idx, recv_topk_weights, num_recv_tokens_per_expert_list, handle,
-        event).  recv_* hold every destination rank's rows back to back; destination d owns
-        rows recv_row_offset[d] : recv_row_offset[d + 1] (handle field)."""
+        x [R, T, H] bfloat16, or a tuple (x, x_scales) of fp8 rows [R, T, H] and their
+        per-token scales [R, T, S] (float32, or int32 for packed UE8M0; any strides, e.g. the
+        transposed layout the reference's test passes); the layout tensors come from
+        get_dispatch_layout and topk_idx / topk_weights are optional.  Returns (recv_x or
+        (recv_x, recv_x_scales), recv_topk_idx, recv_topk_weights,
+        num_recv_tokens_per_expert_list, handle, event).  recv_* hold every destination rank's
+        rows back to back; destination d owns rows recv_row_offset[d] : recv_row_offset[d + 1]
+        (handle field)."""
         if self.low_latency_mode:
             raise EPError("ht_dispatch() requires high-throughput mode (low_latency_mode=False)")
-        if x.dim() != 3 or not x.is_contiguous() or x.dtype != torch.bfloat16:
-            raise EPError("x must be a contiguous [R, T, H] bfloat16 tensor")
+        x, x_scales = x if isinstance(x, tuple) else (x, None)
+        if x.dim() != 3 or not x.is_contiguous():
+            raise EPError("x must be a contiguous [R, T, H] tensor")
+        if x_scales is None and x.dtype != torch.bfloat16:
+            raise EPError("x must be bfloat16 unless it comes with scales, as (x, x_scales)")
         R, T, H = x.shape
         dev = x.device
+        if (H * x.element_size()) % 16:
+            raise EPError("a row of x must be a multiple of 16 bytes")  # csrc/nixl_ep.cpp:660
+        S = 0
+        if x_scales is not None:
+            # csrc/nixl_ep.cpp:703-711
+            if x_scales.dtype not in (torch.float32, torch.int32) or x_scales.dim() != 3 or tuple(x_scales.shape[:2]) != (R, T):
+                raise EPError("x_scales must be a float32 or int32 tensor of shape [R, T, num_scales]")
+            S = x_scales.shape[2]
+
+        def rows_kernel(recv_x, recv_scales, recv_idx, recv_w, recv_meta, idx, w, in_rank, prefix, send_head, row_offset, K, E):
+            strides = x_scales.stride() if x_scales is not None else (0, 0, 0)
+            _check(self._k.nixl_amd_ep_ht_dispatch_scaled(
+                _ptr(recv_x), _ptr(recv_scales), _ptr(recv_idx), _ptr(recv_w), _ptr(recv_meta), _ptr(x), _ptr(x_scales),
+                _ptr(idx), _ptr(w), _ptr(in_rank), _ptr(prefix), _ptr(send_head), _ptr(row_offset), T, H,
+                x.element_size(), S, strides[0], strides[1], strides[2], K, R, E, _stream()), "ht_dispatch")
+
+        def with_scales(recv_x, recv_scales):
+            return (recv_x, recv_scales) if x_scales is not None else recv_x
+
         if handle is not None:
             # Cached mode (buffer.py:560-597): the layout of an earlier dispatch is reused, so
             # there is no count exchange and no host synchronisation; only rows travel.
             in_rank, prefix, _chan, recv_src_meta, send_head, row_offset = handle
             if tuple(in_rank.shape) != (R, T, R):
                 raise EPError("handle does not belong to a dispatch of this shape")
-            recv_x = torch.empty((recv_src_meta.shape[0], H), dtype=torch.bfloat16, device=dev)
-            _check(self._k.nixl_amd_ep_ht_dispatch(_ptr(recv_x), None, None, None, _ptr(x), None, None, _ptr(in_rank),
-                                                   _ptr(prefix), _ptr(send_head), _ptr(row_offset), T, H, 0, R, R,
-                                                   _stream()), "ht_dispatch")
-            return recv_x, None, None, None, None, EventOverlap(None)
-        if num_tokens_per_rank is None or is_token_in_rank is None or num_tokens_per_expert is None or topk_idx is None:
-            raise EPError("ht_dispatch needs either a handle or the tensors of get_dispatch_layout and topk_idx")
+            n_rows = recv_src_meta.shape[0]
+            recv_x = torch.empty((n_rows, H), dtype=x.dtype, device=dev)
+            recv_scales = torch.empty((n_rows, S), dtype=x_scales.dtype, device=dev) if x_scales is not None else None
+            rows_kernel(recv_x, recv_scales, None, None, None, None, None, in_rank, prefix, send_head, row_offset, 0, R)
+            return with_scales(recv_x, recv_scales), None, None, None, None, EventOverlap(None)
+        if num_tokens_per_rank is None or is_token_in_rank is None or num_tokens_per_expert is None:
+            raise EPError("ht_dispatch needs either a handle or the tensors of get_dispatch_layout")
+        if (topk_idx is None) != (topk_weights is None):
+            raise EPError("topk_idx and topk_weights go together")  # csrc/nixl_ep.cpp:686
         if num_channels is None:  # as the reference derives it (csrc/nixl_ep.cpp:630)
             num_channels = (config or self.get_dispatch_config(R)).num_sms // 2
-        K = topk_idx.shape[2]
+        K = topk_idx.shape[2] if topk_idx is not None else 0
         E = num_tokens_per_expert.shape[1]
         El = E // R
         prefix = torch.empty((R, R), dtype=torch.int32, device=dev)
@@ -439,23 +465,26 @@ class Buffer:
         # queued right behind the count kernels, the GPU never idles through the host round
         # trip, and the host only waits for the counts to cut the views.
         capacity = R * T * R
-        ahead = capacity * (H * 2 + K * 8 + 8) <= self.ht_recv_worst_case_limit
+        ahead = capacity * (H * x.element_size() + S * 4 + K * 8 + 8) <= self.ht_recv_worst_case_limit
         rows = capacity if ahead else self._wait_counts(mapped, R)
-        recv_x = torch.empty((rows, H), dtype=torch.bfloat16, device=dev)
-        recv_topk_idx = torch.empty((rows, K), dtype=torch.int32, device=dev)
-        recv_topk_weights = torch.empty((rows, K), dtype=torch.float32, device=dev)
+        recv_x = torch.empty((rows, H), dtype=x.dtype, device=dev)
+        recv_scales = torch.empty((rows, S), dtype=x_scales.dtype, device=dev) if x_scales is not None else None
+        recv_topk_idx = torch.empty((rows, K), dtype=torch.int32, device=dev) if K else None
+        recv_topk_weights = torch.empty((rows, K), dtype=torch.float32, device=dev) if K else None
         recv_src_meta = torch.empty((rows, 2), dtype=torch.int32, device=dev)
-        _check(self._k.nixl_amd_ep_ht_dispatch(_ptr(recv_x), _ptr(recv_topk_idx), _ptr(recv_topk_weights),
-                                               _ptr(recv_src_meta), _ptr(x), _ptr(topk_idx), _ptr(topk_weights),
-                                               _ptr(is_token_in_rank), _ptr(prefix), _ptr(send_head), _ptr(row_offset),
-                                               T, H, K, R, E, _stream()), "ht_dispatch")
+        rows_kernel(recv_x, recv_scales, recv_topk_idx, recv_topk_weights, recv_src_meta, topk_idx, topk_weights,
+                    is_token_in_rank, prefix, send_head, row_offset, K, E)
         if ahead:
             total = self._wait_counts(mapped, R)
-            recv_x, recv_topk_idx = recv_x[:total], recv_topk_idx[:total]
-            recv_topk_weights, recv_src_meta = recv_topk_weights[:total], recv_src_meta[:total]
+            recv_x, recv_src_meta = recv_x[:total], recv_src_meta[:total]
+            if recv_scales is not None:
+                recv_scales = recv_scales[:total]
+            if K:
+                recv_topk_idx, recv_topk_weights = recv_topk_idx[:total], recv_topk_weights[:total]
         expert_count_list = mapped[R:].reshape(R, El).tolist()
         out_handle = (is_token_in_rank, prefix, chan, recv_src_meta, send_head, row_offset)
-        return recv_x, recv_topk_idx, recv_topk_weights, expert_count_list, out_handle, EventOverlap(None)
+        return (with_scales(recv_x, recv_scales), recv_topk_idx, recv_topk_weights, expert_count_list, out_handle,
+                EventOverlap(None))
 
     def ht_combine(self, x, handle, topk_weights=None, bias=None, previous_event=None, async_finish=False,
                    allocate_on_comm_stream=False, config=None):

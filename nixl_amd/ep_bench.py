@@ -143,7 +143,20 @@ def run_normal(dev, warmup=5, iters=20):
     coef = (recv_w * (recv_idx >= 0)).sum(1, keepdim=True)
     y = (recv_x.float() * coef).to(torch.bfloat16)
     t_combine = _timed(lambda: buf.ht_combine(y, handle, topk_weights=recv_w), flush, warmup, iters)
+    # fp8 rows with their per-128-channel scales, the (x, x_scales) form; scales stored
+    # transposed as the reference's test passes them (tests/test_ht.py:78-79)
+    S = H // 128
+    x8 = torch.randint(0, 256, (R, T, H), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    sc = torch.rand((R, T, S), device=dev).transpose(1, 2).contiguous().transpose(1, 2)
+
+    def dispatch_fp8():
+        per_rank, _, per_expert, in_rank, _ = state["layout"]
+        buf.ht_dispatch((x8, sc), num_tokens_per_rank=per_rank, is_token_in_rank=in_rank,
+                        num_tokens_per_expert=per_expert, topk_idx=topk, topk_weights=w, num_channels=C)
+
+    t_fp8 = _timed(dispatch_fp8, flush, warmup, iters)
     tokens = R * T
+    fp8_bytes = (tokens + rows) * (H + S * 4) + tokens * K * 8 + rows * (K * 8 + 8) + tokens * K * 4 + tokens * R
     dispatch_bytes = tokens * H * 2 + rows * H * 2 + tokens * K * 8 + rows * (K * 8 + 8) + tokens * K * 4 + tokens * R
     combine_bytes = rows * H * 2 + rows * K * 4 + tokens * H * 2 + tokens * K * 4
     counts = np.array(per_expert_list).reshape(-1)
@@ -158,6 +171,8 @@ def run_normal(dev, warmup=5, iters=20):
         "dispatch_cached_handle": {**t_cached, **_rate(tokens * H * 2 + rows * H * 2, t_cached["avg_us"]),
                                    "note": "layout of an earlier dispatch reused: rows only, no count exchange"},
         "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
+        "dispatch_fp8_rows_with_scales": {**t_fp8, **_rate(fp8_bytes, t_fp8["avg_us"]),
+                                          "note": "rows of 7168 fp8 bytes plus 56 fp32 scales per token"},
     }
 
 

@@ -443,6 +443,66 @@ def test_ht_pipeline_matches_oracle(cuda, shape):
         assert np.array_equal(comb_w.cpu().numpy(), want_w)
 
 
+@pytest.mark.parametrize("scale_dtype", [np.float32, np.int32])
+def test_ht_dispatch_fp8_rows_with_scales(cuda, scale_dtype):
+    """The (x, x_scales) form of normal-mode dispatch.  The reference's test passes fp8 rows
+    with scales whose storage is transposed (tests/test_ht.py:78-79) and expects each received
+    row's scales to be its source token's (:215-231: per_token_cast_back of the pair, then check_data).  Rows are
+    checked as bytes against the oracle's row move, scales against a gather by the oracle's
+    source rank and token, for the first dispatch, without top-k, and with a cached handle."""
+    R, T, H, K, E, C = 4, 333, 512, 4, 16, 4
+    S = H // 128
+    _, topk, w = make_world(5, R, T, H, K, E)
+    rng = np.random.default_rng(9)
+    x8 = rng.integers(0, 256, (R, T, H), dtype=np.uint8)
+    sc = (rng.standard_normal((R, T, S)) * 100).astype(scale_dtype)
+    x8d = torch.from_numpy(x8).to(cuda).view(torch.float8_e4m3fn)
+    sc_d = torch.from_numpy(sc).to(cuda).transpose(1, 2).contiguous().transpose(1, 2)
+    assert sc_d.stride() == (T * S, 1, T)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    buf = Buffer(R, low_latency_mode=False, device=cuda)
+    per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(td, E)
+    (recv_x, recv_sc), recv_idx, recv_w, _, handle, _ = buf.ht_dispatch(
+        (x8d, sc_d), num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert,
+        topk_idx=td, topk_weights=wd, num_channels=C)
+    torch.cuda.synchronize()
+    lay = [eo.dispatch_layout(topk[r], R, E) for r in range(R)]
+    o_in_rank = np.stack([l[2] for l in lay])
+    o_prefix, _, _ = eo.ht_notify(o_in_rank, np.stack([l[1] for l in lay]), C, 1)
+    o = eo.ht_dispatch(x8.view(np.uint16), topk, w, o_in_rank, o_prefix, E)
+    want_sc = sc[o["recv_src_rank"], o["recv_src_token"]]
+    assert recv_x.dtype == torch.float8_e4m3fn and tuple(recv_x.shape) == (o["recv_x"].shape[0], H)
+    assert np.array_equal(recv_x.view(torch.uint8).cpu().numpy(), o["recv_x"].view(np.uint8))
+    assert recv_sc.is_contiguous() and np.array_equal(recv_sc.cpu().numpy(), want_sc)
+    assert np.array_equal(recv_idx.cpu().numpy(), o["recv_topk_idx"])
+    assert np.array_equal(recv_w.cpu().numpy(), o["recv_topk_weights"])
+    # without top-k (tests/test_ht.py:176-199 runs both): rows, scales and the handle only
+    (nx, nsc), n_idx, n_w, _, n_handle, _ = buf.ht_dispatch(
+        (x8d, sc_d), num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert,
+        num_channels=C)
+    torch.cuda.synchronize()
+    assert n_idx is None and n_w is None and torch.equal(n_handle[3], handle[3])
+    assert torch.equal(nx.view(torch.uint8), recv_x.view(torch.uint8)) and torch.equal(nsc, recv_sc)
+    # cached handle, other data, scales stored row-major this time
+    x8b = rng.integers(0, 256, (R, T, H), dtype=np.uint8)
+    scb = (rng.standard_normal((R, T, S)) * 100).astype(scale_dtype)
+    (cx, csc), c_idx, _, _, _, _ = buf.ht_dispatch(
+        (torch.from_numpy(x8b).to(cuda).view(torch.float8_e4m3fn), torch.from_numpy(scb).to(cuda)), handle=handle)
+    torch.cuda.synchronize()
+    o2 = eo.ht_dispatch(x8b.view(np.uint16), topk, w, o_in_rank, o_prefix, E)
+    assert c_idx is None
+    assert np.array_equal(cx.view(torch.uint8).cpu().numpy(), o2["recv_x"].view(np.uint8))
+    assert np.array_equal(csc.cpu().numpy(), scb[o2["recv_src_rank"], o2["recv_src_token"]])
+    # argument checks of csrc/nixl_ep.cpp:660,686,703-707
+    with pytest.raises(EPError):
+        buf.ht_dispatch((x8d, sc_d[:, :-1]), handle=handle)
+    with pytest.raises(EPError):
+        buf.ht_dispatch(x8d, handle=handle)  # fp8 rows need their scales
+    with pytest.raises(EPError):
+        buf.ht_dispatch((x8d, sc_d), num_tokens_per_rank=per_rank, is_token_in_rank=in_rank,
+                        num_tokens_per_expert=per_expert, topk_idx=td, num_channels=C)
+
+
 def test_ht_dispatch_sized_ahead_equals_sized_exactly(cuda):
     """Normal-mode dispatch either sizes its receive tensors for the worst case and launches
     before the counts reach the host, or (past a byte limit) waits for the counts as the
