@@ -8,11 +8,14 @@ _api.py:999-1092).  Only the single-agent loopback subset exists; there is no me
 exchange or notification path.
 """
 import ctypes
+import logging
 import os
 
 import numpy as np
 
 from . import _lib
+
+logger = logging.getLogger("nixl_amd")
 
 NIXL_INIT_AGENT = ""
 
@@ -221,12 +224,19 @@ class nixl_xfer_handle:
 class nixl_agent:
     """Reference: nixl_agent, src/api/python/_api.py:189-296."""
 
-    def __init__(self, agent_name, nixl_conf=None, plugin_dirs=()):
+    def __init__(self, agent_name, nixl_conf=None, instantiate_all=False, plugin_dirs=()):
+        """Reference: _api.py:200-282.  Without a configuration the defaults of
+        nixl_agent_config apply (the HIP backend here, where the reference names UCX);
+        instantiate_all creates a backend for every plugin found instead; plugin_dirs (not in
+        the reference) adds directories to the plugin search path."""
         if not agent_name:
             raise ValueError("agent name must not be empty")  # as the reference bindings do
         self._lib = _lib.agent_lib()
         self.name = agent_name
-        conf = nixl_conf or nixl_agent_config(backends=())
+        if nixl_conf and instantiate_all:
+            instantiate_all = False
+            logger.warning("Ignoring instantiate_all based on the provided config in agent creation.")
+        conf = nixl_conf or nixl_agent_config()
         dirs = [_lib.PLUGIN_DIR] + list(plugin_dirs)
         prev = os.environ.get("NIXL_PLUGIN_DIR")
         if prev:
@@ -240,7 +250,14 @@ class nixl_agent:
         self.backends = {}
         self.notifs = {}  # what update_notifs / check_remote_xfer_done have not handed out yet
         self.nixl_ops = {"WRITE": 1, "READ": 0}
-        for b in conf.backends:
+        self.plugin_list = self.get_plugin_list()
+        if not self.plugin_list:
+            self.close()
+            raise RuntimeError("No plugins available for NIXL, cannot start transfers!")
+        for b in (self.plugin_list if instantiate_all else conf.backends):
+            if b not in self.plugin_list:
+                logger.warning("Skipping backend registration %s due to the missing plugin.", b)
+                continue
             self.create_backend(b)
 
     def close(self):

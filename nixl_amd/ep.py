@@ -178,6 +178,22 @@ class Buffer:
         """Reference alias, buffer.py:163-172."""
         return Buffer.get_low_latency_buffer_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts)
 
+    @staticmethod
+    def is_sm90_compiled():
+        """Reference: buffer.py:112-114 (whether Hopper-only code paths were built)."""
+        return False
+
+    def get_local_buffer_tensor(self, dtype, size=None, offset=0, use_rdma_buffer=False):
+        """Reference: buffer.py:188-209, a typed view of the rank's staging buffer.  There is
+        no staging buffer here (rows are written straight to their final place), so there is
+        nothing to view."""
+        raise EPError("get_local_buffer_tensor: this Buffer has no staging buffer")
+
+    def set_tcp_store_group(self, tcp_store_group):
+        """Reference: buffer.py:789-797 (a store for metadata exchange between processes);
+        all ranks share this process, so the store is only remembered."""
+        self._tcp_store_group = tcp_store_group
+
     def get_next_combine_buffer(self, handle):
         """Reference: buffer.py:743-764.  A bf16 tensor shaped like the packed_recv_x of the
         dispatch that produced `handle`; experts may write their outputs into it and call
@@ -385,8 +401,8 @@ class Buffer:
 
     def ht_dispatch(self, x, handle=None, num_tokens_per_rank=None, num_tokens_per_rdma_rank=None,
                     is_token_in_rank=None, num_tokens_per_expert=None, topk_idx=None, topk_weights=None,
-                    expert_alignment=1, num_channels=None, previous_event=None, async_finish=False,
-                    allocate_on_comm_stream=False, config=None):
+                    expert_alignment=1, config=None, previous_event=None, async_finish=False,
+                    allocate_on_comm_stream=False, num_channels=None):
         """Reference: buffer.py:526-660, csrc/nixl_ep.cpp:615-898.
 
         x [R, T, H] bfloat16, or a tuple (x, x_scales) of fp8 rows [R, T, H] and their
@@ -486,8 +502,8 @@ class Buffer:
         return (with_scales(recv_x, recv_scales), recv_topk_idx, recv_topk_weights, expert_count_list, out_handle,
                 EventOverlap(None))
 
-    def ht_combine(self, x, handle, topk_weights=None, bias=None, previous_event=None, async_finish=False,
-                   allocate_on_comm_stream=False, config=None):
+    def ht_combine(self, x, handle, topk_weights=None, bias=None, config=None, previous_event=None,
+                   async_finish=False, allocate_on_comm_stream=False):
         """Reference: buffer.py:663-714, csrc/nixl_ep.cpp:900-1028.  x [total, H] bf16 in the
         row order ht_dispatch produced.  Returns (combined_x [R, T, H], combined_topk_weights
         [R, T, K] or None, event)."""

@@ -432,6 +432,40 @@ def test_low_latency_buffer_size_hint_follows_the_reference_layout():
     assert small == (2 * max(64 * d, 64 * c) + 2 * max(64 * d, 64 * c) + 2 * 128 + 128) // 128 * 128
 
 
+def test_buffer_exposes_the_reference_method_names():
+    """Every public method of the reference's Buffer (examples/device/ep/nixl_ep/buffer.py:
+    43-886) exists here under the same name, so that code written against it finds them."""
+    from nixl_amd.ep import Buffer
+    names = ["destroy", "is_sm90_compiled", "set_num_sms", "capture", "get_low_latency_buffer_size_hint",
+             "get_rdma_size_hint", "get_comm_stream", "get_local_buffer_tensor", "get_dispatch_config",
+             "get_combine_config", "get_dispatch_layout", "low_latency_dispatch", "dispatch",
+             "low_latency_combine", "combine", "ht_dispatch", "ht_combine", "update_mask_buffer",
+             "query_mask_buffer", "clean_mask_buffer", "get_next_combine_buffer", "update_memory_buffers",
+             "set_tcp_store_group", "connect_ranks", "disconnect_ranks", "barrier"]
+    missing = [n for n in names if not callable(getattr(Buffer, n, None))]
+    assert not missing, missing
+    assert Buffer.is_sm90_compiled() is False
+    # ... and takes its arguments in the reference's order (buffer.py:278-284, 329-341, 443-454,
+    # 526-540, 663-672), so that positional calls mean the same; extensions come after them
+    import inspect
+    order = {
+        "get_dispatch_layout": ["topk_idx", "num_experts", "previous_event", "async_finish", "allocate_on_comm_stream"],
+        "low_latency_dispatch": ["x", "topk_idx", "num_max_dispatch_tokens_per_rank", "num_experts",
+                                 "cumulative_local_expert_recv_stats", "dispatch_wait_recv_cost_stats", "use_fp8",
+                                 "round_scale", "use_ue8m0", "async_finish", "return_recv_hook"],
+        "low_latency_combine": ["x", "topk_idx", "topk_weights", "handle", "use_logfmt", "zero_copy", "async_finish",
+                                "return_recv_hook", "out", "combine_wait_recv_cost_stats"],
+        "ht_dispatch": ["x", "handle", "num_tokens_per_rank", "num_tokens_per_rdma_rank", "is_token_in_rank",
+                        "num_tokens_per_expert", "topk_idx", "topk_weights", "expert_alignment", "config",
+                        "previous_event", "async_finish", "allocate_on_comm_stream"],
+        "ht_combine": ["x", "handle", "topk_weights", "bias", "config", "previous_event", "async_finish",
+                       "allocate_on_comm_stream"],
+    }
+    for name, want in order.items():
+        got = [p for p in inspect.signature(getattr(Buffer, name)).parameters if p != "self"]
+        assert got[:len(want)] == want, (name, got)
+
+
 def _logfmt_reference_f64(vals):
     """LogFMT-10 round trip of one 128-channel group in float64 from its definition
     (examples/device/ep/csrc/kernels/nixl_ep_ll.cu:459-616): returns (decoded, step) or

@@ -293,3 +293,58 @@ def test_api_behaviour_of_the_reference_python_tests(cpu_agent, oracle_plugin_di
     cont = torch.arange(8).reshape(2, 4)
     assert a.get_reg_descs(torch.transpose(cont, 0, 1)) is None and a.get_xfer_descs(torch.transpose(cont, 0, 1)) is None
     assert a.get_xfer_descs(cont, "DRAM").descCount() == 1  # a single tensor, not only a list
+
+
+def test_python_agent_follows_the_reference_signatures(oracle_plugin_dir, caplog):
+    """Every public method of the reference's nixl_agent (src/api/python/_api.py:189-1160) is
+    here with the same leading arguments in the same order, and the constructor behaves as
+    _api.py:200-264: a configured backend without a plugin is skipped with a warning,
+    instantiate_all creates every backend found, instantiate_all next to a configuration is
+    ignored."""
+    import inspect
+    import logging
+    from nixl_amd.agent import nixl_agent, nixl_agent_config
+    reference = {
+        "get_plugin_list": [], "get_plugin_mem_types": ["backend"], "get_plugin_params": ["backend"],
+        "get_backend_mem_types": ["backend"], "get_backend_params": ["backend"],
+        "create_backend": ["backend", "initParams"], "register_memory": ["reg_list", "mem_type", "backends"],
+        "deregister_memory": ["dereg_list", "backends"], "query_memory": ["reg_list", "backend", "mem_type"],
+        "make_connection": ["remote_agent", "backends"],
+        "prep_xfer_dlist": ["agent_name", "xfer_list", "mem_type", "backends"], "estimate_xfer_cost": ["req_handle"],
+        "make_prepped_xfer": ["operation", "local_xfer_side", "local_indices", "remote_xfer_side", "remote_indices",
+                              "notif_msg", "backends", "skip_desc_merge"],
+        "initialize_xfer": ["operation", "local_descs", "remote_descs", "remote_agent", "notif_msg", "backends"],
+        "transfer": ["handle", "notif_msg"], "check_xfer_state": ["handle"], "get_xfer_telemetry": ["handle"],
+        "query_xfer_backend": ["handle"], "release_xfer_handle": ["handle"], "release_dlist_handle": ["handle"],
+        "prep_mem_view": ["dlist"], "release_mem_view": ["mvh"], "get_new_notifs": ["backends"],
+        "update_notifs": ["backends"],
+        "check_remote_xfer_done": ["remote_agent_name", "lookup_tag", "backends", "tag_is_prefix"],
+        "send_notif": ["remote_agent_name", "notif_msg", "backend"], "get_agent_metadata": [],
+        "get_partial_agent_metadata": ["descs", "inc_conn_info", "backends"], "add_remote_agent": ["metadata"],
+        "remove_remote_agent": ["agent"], "send_local_metadata": ["ip_addr", "port"],
+        "send_partial_agent_metadata": ["descs", "inc_conn_info", "backends", "ip_addr", "port", "label"],
+        "fetch_remote_metadata": ["remote_agent", "ip_addr", "port", "label"],
+        "invalidate_local_metadata": ["ip_addr", "port"], "check_remote_metadata": ["agent", "descs"],
+        "get_xfer_descs": ["descs", "mem_type"], "get_remote_descs": ["descs", "mem_type"],
+        "get_reg_descs": ["descs", "mem_type"], "get_serialized_descs": ["descs"],
+        "deserialize_descs": ["serialized_descs"],
+    }
+    for name, want in reference.items():
+        fn = getattr(nixl_agent, name, None)
+        assert callable(fn), name
+        got = [p for p in inspect.signature(fn).parameters if p != "self"]
+        assert got[:len(want)] == want, (name, got)
+    ctor = [p for p in inspect.signature(nixl_agent.__init__).parameters if p != "self"]
+    assert ctor[:3] == ["agent_name", "nixl_conf", "instantiate_all"]
+
+    with caplog.at_level(logging.WARNING, logger="nixl_amd"):
+        a = nixl_agent("ctor-a", nixl_agent_config(backends=("NOSUCH", "MEMCPY")), plugin_dirs=[oracle_plugin_dir])
+    assert list(a.backends) == ["MEMCPY"]
+    assert any("Skipping backend registration NOSUCH" in r.getMessage() for r in caplog.records)
+    a.close()
+    caplog.clear()
+    with caplog.at_level(logging.WARNING, logger="nixl_amd"):
+        b = nixl_agent("ctor-b", nixl_agent_config(backends=("MEMCPY",)), True, plugin_dirs=[oracle_plugin_dir])
+    assert list(b.backends) == ["MEMCPY"]  # the configuration wins
+    assert any("Ignoring instantiate_all" in r.getMessage() for r in caplog.records)
+    b.close()
