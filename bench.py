@@ -36,6 +36,13 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 MEASURED_TRAFFIC_BYTES = {(1024, 8192, 32768): 4311669989}
 
 
+def _kv_layout():
+    """Llama-3.1-8B with 16 tokens per block in bf16: 32 layers x {K, V}, 32 KiB per sub-block
+    (nixl_amd/kvshape.py restates the reference's KV-size model)."""
+    from nixl_amd import kvshape
+    return kvshape.paged_kv_layout(kvshape.model("LLAMA3.1_8B"), 16, "bfloat16")
+
+
 def _kv_descs(base, layers, pool_blocks, blk, block_ids):
     """One descriptor per (block, layer, K|V) in a pool laid out [layer][K|V][block][blk]."""
     block_ids = np.asarray(block_ids, dtype=np.uint64)
@@ -54,8 +61,9 @@ def run_kv(args):
     from nixl_amd import nixl_agent, nixl_agent_config
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    layers, pool_blocks, n_sel, blk = 32, args.pool_blocks, args.blocks, args.block_bytes
-    lk = layers * 2
+    kv = _kv_layout()
+    layers, pool_blocks, n_sel, blk = kv.layers, args.pool_blocks, args.blocks, args.block_bytes
+    lk = layers * kv.sub_blocks_per_layer
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     src_pool = torch.empty((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
@@ -294,8 +302,9 @@ def run_cpu_baseline(seconds=12.0, threads=1):
     selected blocks (4096 descriptors of 32 KiB per request), single thread."""
     from nixl_amd import nixl_agent, nixl_agent_config
     plugin_dir = os.path.join(ROOT, "oracle", "_build")
-    layers, pool_blocks, n_sel, blk = 32, 512, 64, 32768
-    lk = layers * 2
+    kv = _kv_layout()
+    layers, pool_blocks, n_sel, blk = kv.layers, 512, 64, kv.bytes_per_sub_block
+    lk = layers * kv.sub_blocks_per_layer
     rng = np.random.default_rng(7)
     src_pool = rng.integers(0, 256, lk * pool_blocks * blk, dtype=np.uint8)
     dst_pool = np.zeros(lk * pool_blocks * blk, dtype=np.uint8)
@@ -347,7 +356,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=1024, help="KV blocks moved per request")
     ap.add_argument("--pool-blocks", type=int, default=8192)
-    ap.add_argument("--block-bytes", type=int, default=32768, help="bytes per (layer, K|V) sub-block")
+    ap.add_argument("--block-bytes", type=int, default=0,
+                    help="bytes per (layer, K|V) sub-block; 0: what the model gives (32768)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ep", action="store_true")
     ap.add_argument("--no-small", action="store_true", help="skip the small-descriptor stress")
@@ -364,6 +374,8 @@ def main():
     import __graft_entry__ as entry
     entry._ensure_built()
 
+    if not args.block_bytes:
+        args.block_bytes = _kv_layout().bytes_per_sub_block
     if args.calibrate_copy:
         run_calibration_copy()
     kv = run_kv(args)
