@@ -385,6 +385,26 @@ class Buffer:
         return idx, w
 
     # -- normal (high-throughput) mode ---------------------------------------------------------
+    # The reference runs normal-mode work on a communication stream: it makes that stream wait
+    # for `previous_event` (or for the caller's stream), and hands back an event instead of
+    # joining the streams when `async_finish` is set (csrc/nixl_ep.cpp:558-571,596-611).  Here
+    # the work runs on the caller's current stream, so only the two events remain.
+    @staticmethod
+    def _after(previous_event, async_finish, allocate_on_comm_stream):
+        if allocate_on_comm_stream and not (previous_event is not None and async_finish):
+            raise EPError("allocate_on_comm_stream needs previous_event and async_finish")  # csrc/nixl_ep.cpp:562
+        event = getattr(previous_event, "event", None)
+        if event is not None:
+            torch.cuda.current_stream().wait_event(event)
+
+    @staticmethod
+    def _done(async_finish):
+        if not async_finish:
+            return EventOverlap(None)
+        event = torch.cuda.Event()
+        event.record()
+        return EventOverlap(event)
+
     def get_dispatch_layout(self, topk_idx, num_experts, previous_event=None, async_finish=False,
                             allocate_on_comm_stream=False):
         """Reference: buffer.py:278-326, csrc/nixl_ep.cpp:551-613.  topk_idx [R, T, K].
@@ -392,12 +412,13 @@ class Buffer:
         num_tokens_per_expert [R, E], is_token_in_rank [R, T, R] bool, event)."""
         R, T, K = topk_idx.shape
         dev = topk_idx.device
+        self._after(previous_event, async_finish, allocate_on_comm_stream)
         per_rank = torch.empty((R, R), dtype=torch.int32, device=dev)
         per_expert = torch.empty((R, num_experts), dtype=torch.int32, device=dev)
         in_rank = torch.empty((R, T, R), dtype=torch.bool, device=dev)
         _check(self._k.nixl_amd_ep_get_dispatch_layout(_ptr(topk_idx), _ptr(per_rank), _ptr(per_expert), _ptr(in_rank),
                                                        T, K, R, num_experts, _stream()), "get_dispatch_layout")
-        return per_rank, None, per_expert, in_rank, EventOverlap(None)
+        return per_rank, None, per_expert, in_rank, self._done(async_finish)
 
     def ht_dispatch(self, x, handle=None, num_tokens_per_rank=None, num_tokens_per_rdma_rank=None,
                     is_token_in_rank=None, num_tokens_per_expert=None, topk_idx=None, topk_weights=None,
@@ -441,6 +462,8 @@ class Buffer:
         def with_scales(recv_x, recv_scales):
             return (recv_x, recv_scales) if x_scales is not None else recv_x
 
+        self._after(previous_event, async_finish, allocate_on_comm_stream)
+
         if handle is not None:
             # Cached mode (buffer.py:560-597): the layout of an earlier dispatch is reused, so
             # there is no count exchange and no host synchronisation; only rows travel.
@@ -451,7 +474,7 @@ class Buffer:
             recv_x = torch.empty((n_rows, H), dtype=x.dtype, device=dev)
             recv_scales = torch.empty((n_rows, S), dtype=x_scales.dtype, device=dev) if x_scales is not None else None
             rows_kernel(recv_x, recv_scales, None, None, None, None, None, in_rank, prefix, send_head, row_offset, 0, R)
-            return with_scales(recv_x, recv_scales), None, None, None, None, EventOverlap(None)
+            return with_scales(recv_x, recv_scales), None, None, None, None, self._done(async_finish)
         if num_tokens_per_rank is None or is_token_in_rank is None or num_tokens_per_expert is None:
             raise EPError("ht_dispatch needs either a handle or the tensors of get_dispatch_layout")
         if (topk_idx is None) != (topk_weights is None):
@@ -500,7 +523,7 @@ class Buffer:
         expert_count_list = mapped[R:].reshape(R, El).tolist()
         out_handle = (is_token_in_rank, prefix, chan, recv_src_meta, send_head, row_offset)
         return (with_scales(recv_x, recv_scales), recv_topk_idx, recv_topk_weights, expert_count_list, out_handle,
-                EventOverlap(None))
+                self._done(async_finish))
 
     def ht_combine(self, x, handle, topk_weights=None, bias=None, config=None, previous_event=None,
                    async_finish=False, allocate_on_comm_stream=False):
@@ -515,9 +538,10 @@ class Buffer:
         dev = x.device
         bias_0, bias_1 = (bias if isinstance(bias, (tuple, list)) else (bias, None))
         K = topk_weights.shape[1] if topk_weights is not None else 0
+        self._after(previous_event, async_finish, allocate_on_comm_stream)
         combined = torch.empty((R, T, H), dtype=torch.bfloat16, device=dev)
         combined_w = torch.empty((R, T, K), dtype=torch.float32, device=dev) if K else None
         _check(self._k.nixl_amd_ep_ht_combine(_ptr(combined), _ptr(combined_w), _ptr(x), _ptr(topk_weights),
                                               _ptr(bias_0), _ptr(bias_1), _ptr(in_rank), _ptr(prefix), _ptr(send_head),
                                               _ptr(row_offset), T, H, max(K, 1), R, _stream()), "ht_combine")
-        return combined, combined_w, EventOverlap(None)
+        return combined, combined_w, self._done(async_finish)

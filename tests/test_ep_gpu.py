@@ -503,6 +503,57 @@ def test_ht_dispatch_fp8_rows_with_scales(cuda, scale_dtype):
                         num_tokens_per_expert=per_expert, topk_idx=td, num_channels=C)
 
 
+def test_ht_calls_honour_previous_event_and_async_finish(cuda):
+    """previous_event / async_finish as the reference defines them (csrc/nixl_ep.cpp:558-571,
+    596-611; its test passes buffer.capture() and waits on the returned event,
+    tests/test_ht.py:204-214): the work waits for the event it is given, and with
+    async_finish the returned event covers it.  The input is produced on a side stream behind
+    a long fill, so a dispatch that ignored the event would read it too early."""
+    R, T, H, K, E, C = 4, 257, 512, 4, 16, 4
+    x, topk, w = make_world(13, R, T, H, K, E)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    buf = Buffer(R, low_latency_mode=False, device=cuda)
+    want_x = x.to(cuda)
+    xd = torch.zeros_like(want_x)
+    ballast = torch.empty(1 << 30, dtype=torch.uint8, device=cuda)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=cuda)
+    with torch.cuda.stream(side):
+        for _ in range(8):
+            ballast.fill_(1)  # a few milliseconds of work ahead of the copy
+        xd.copy_(want_x)
+        produced = Buffer.capture()  # an EventOverlap on the side stream
+    per_rank, _, per_expert, in_rank, ev0 = buf.get_dispatch_layout(td, E, previous_event=produced, async_finish=True)
+    assert ev0.event is not None
+    recv_x, recv_idx, recv_w, _, handle, ev1 = buf.ht_dispatch(
+        xd, num_tokens_per_rank=per_rank, is_token_in_rank=in_rank, num_tokens_per_expert=per_expert, topk_idx=td,
+        topk_weights=wd, previous_event=produced, async_finish=True, num_channels=C)
+    assert ev1.event is not None
+    # a consumer on another stream orders itself behind the dispatch through the returned event
+    with torch.cuda.stream(side):
+        ev1.current_stream_wait()
+        seen = recv_x.clone()
+        after = Buffer.capture()
+    comb, _, ev2 = buf.ht_combine(seen, handle, topk_weights=recv_w, previous_event=after, async_finish=True)
+    ev2.event.synchronize()
+    torch.cuda.synchronize()
+    lay = [eo.dispatch_layout(topk[r], R, E) for r in range(R)]
+    o_in_rank = np.stack([l[2] for l in lay])
+    o_prefix, _, _ = eo.ht_notify(o_in_rank, np.stack([l[1] for l in lay]), C, 1)
+    o = eo.ht_dispatch(bits16(x).reshape(R, T, H), topk, w, o_in_rank, o_prefix, E)
+    assert np.array_equal(bits16(seen).reshape(-1, H), o["recv_x"])
+    want, _ = eo.ht_combine(o["recv_x"], o["recv_topk_weights"], o_in_rank, o_prefix, o["send_head"], o["row_offset"],
+                            None, None)
+    assert np.array_equal(bits16(comb).reshape(R, T, H), want)
+    # csrc/nixl_ep.cpp:562,718,938
+    with pytest.raises(EPError):
+        buf.get_dispatch_layout(td, E, allocate_on_comm_stream=True)
+    with pytest.raises(EPError):
+        buf.ht_combine(seen, handle, allocate_on_comm_stream=True, async_finish=True)
+    sync_out = buf.ht_combine(seen, handle)
+    assert sync_out[2].event is None
+
+
 def test_ht_dispatch_sized_ahead_equals_sized_exactly(cuda):
     """Normal-mode dispatch either sizes its receive tensors for the worst case and launches
     before the counts reach the host, or (past a byte limit) waits for the counts as the
