@@ -286,6 +286,8 @@ class Buffer:
         event, hook) with handle = (src_info, layout_range, num_max_dispatch_tokens_per_rank,
         hidden).  `num_tokens_per_rank` ([R] int32 device tensor) is an extension for ragged
         worlds: rank r only owns the first num_tokens_per_rank[r] rows of x[r].
+        dispatch_wait_recv_cost_stats (cycles spent waiting for each source rank's data,
+        nixl_ep_ll.cu:349-350) is left as it is: nothing here waits for another rank.
         """
         if not self.low_latency_mode:
             raise EPError("dispatch() requires low-latency mode (low_latency_mode=True)")
