@@ -87,6 +87,11 @@ inline constexpr uint16_t default_comm_port = 8888;
 // Agent name of a placeholder entry in a remote memory-view list
 // (src/api/cpp/nixl_types.h:305, src/infra/nixl_descriptors.cpp:30).
 extern const std::string nixl_null_agent;
+// Label under which the reference's metadata side channel stores an agent's metadata
+// (src/api/cpp/nixl_types.h:139, value from src/core/nixl_md_manager.cpp:37); kept for callers
+// that name it.  The reference also declares default_partial_metadata_label (:145) but defines
+// it nowhere, so it is not repeated here.
+extern const std::string default_metadata_label;
 
 namespace nixlEnumStrings {
 

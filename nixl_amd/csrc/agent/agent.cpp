@@ -254,6 +254,7 @@ nixlMemSection::populate(const nixl_xfer_dlist_t &query,
 // =====================================================================================
 
 const std::string nixl_null_agent = "NULL_AGENT";
+const std::string default_metadata_label = "metadata";
 
 nixlAgentData::~nixlAgentData() {
     for (const auto &[view, engine] : mvhToEngine)
