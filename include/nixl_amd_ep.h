@@ -89,6 +89,41 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                         void *stream);
 
 /*
+ * Low-latency dispatch that allocates nothing.  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory: code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc.  Arguments and results are those of
+ * nixl_amd_ep_ll_dispatch without `workspace`: the scratch is a fixed array of
+ * NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the
+ * process ends.  A shape whose nixl_amd_ep_ll_workspace_bytes exceeds that size is refused with
+ * NIXL_AMD_ERR_TOO_LARGE before anything is launched.  All calls on one GPU share the array:
+ * two calls may not overlap on one GPU (different streams, or threads), or they race.  The
+ * call itself issues no hipMalloc, hipFree, memset or other allocating routine.
+ */
+#define NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES (4u << 20)
+int
+nixl_amd_ep_ll_dispatch_static(void *packed_recv_x,
+                               void *packed_recv_x_scales,
+                               int *packed_recv_src_info,
+                               int64_t *packed_recv_layout_range,
+                               int *packed_recv_count,
+                               const int *mask_buffer,
+                               int *cumulative_local_expert_recv_stats,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const int *num_tokens_per_rank,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_fp8,
+                               int round_scale,
+                               int use_ue8m0,
+                               int *row_map,
+                               void *stream);
+
+/*
  * Low-latency combine for all ranks.  Replaces ep_kernels::combine (kernels/api.cuh:226-238;
  * kernel kernels/nixl_ep_ll.cu:618-1017): combined_x[r][t] = bf16( sum over k, in top-k
  * order, of float(x[row(r,t,k)]) * topk_weights[r][t][k] ) with fused multiply-adds in

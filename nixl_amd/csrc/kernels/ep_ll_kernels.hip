@@ -31,6 +31,7 @@
 // (kernels/nixl_ep_ll.cu:959-1012).  Traffic per token: read K * 2H, write 2H.
 #include <algorithm>
 #include <cstdint>
+#include <mutex>
 
 #include "common.h"
 #include "ep_common.h"
@@ -507,6 +508,39 @@ int g_combine_lanes = 1024;
 
 } // namespace
 
+// Scratch of the entry point that allocates nothing (nixl_amd_ep_ll_dispatch_static): the
+// dispatch workspace lives in this array instead of in memory the caller brings.  Every GPU
+// the library runs on holds its own copy, at its own address, until the process ends.  The
+// array's name is only a host-side handle for hipGetSymbolAddress; host code passes kernels
+// the per-device address kept in g_scratch_ptr and never the name itself.
+constexpr size_t kStaticScratchBytes = NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch`; resolved once per device.
+int
+static_scratch(void **out) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch_static: device id out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return nixl_amd_fail(NIXL_AMD_ERR_HIP, "ll_dispatch_static: the scratch array has no device address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return NIXL_AMD_OK;
+}
+
+} // namespace
+
 extern "C" {
 
 int
@@ -628,6 +662,47 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                        static_cast<size_t>(d.R) * sizeof(int), s, sa);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_ll_dispatch_static(void *packed_recv_x,
+                               void *packed_recv_x_scales,
+                               int *packed_recv_src_info,
+                               int64_t *packed_recv_layout_range,
+                               int *packed_recv_count,
+                               const int *mask_buffer,
+                               int *cumulative_local_expert_recv_stats,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const int *num_tokens_per_rank,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_fp8,
+                               int round_scale,
+                               int use_ue8m0,
+                               int *row_map,
+                               void *stream) {
+    const size_t need = nixl_amd_ep_ll_workspace_bytes(num_ranks, num_experts, num_tokens, num_topk, hidden);
+    if (need > kStaticScratchBytes)
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE,
+                             "ll_dispatch_static: this shape needs " + std::to_string(need) +
+                                 " bytes of scratch, the built-in array holds " + std::to_string(kStaticScratchBytes) +
+                                 "; use nixl_amd_ep_ll_dispatch with a workspace of the caller's");
+    void *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+    // Every word of the workspace that a kernel reads is written earlier in the same call
+    // (counts and positions by the layout kernel, rows and scales by the dispatch kernel), so
+    // what the previous call left behind needs no clearing.
+    return nixl_amd_ep_ll_dispatch(packed_recv_x, packed_recv_x_scales, packed_recv_src_info, packed_recv_layout_range,
+                                   packed_recv_count, mask_buffer, cumulative_local_expert_recv_stats, x, topk_idx,
+                                   num_tokens_per_rank, num_tokens, hidden, num_max_dispatch_tokens_per_rank, num_topk,
+                                   num_ranks, num_experts, use_fp8, round_scale, use_ue8m0, row_map, ws, kStaticScratchBytes,
+                                   stream);
 }
 
 int
