@@ -43,12 +43,14 @@ def _kv_layout():
     return kvshape.paged_kv_layout(kvshape.model("LLAMA3.1_8B"), 16, "bfloat16")
 
 
-def _kv_descs(base, layers, pool_blocks, blk, block_ids):
-    """One descriptor per (block, layer, K|V) in a pool laid out [layer][K|V][block][blk]."""
+def _kv_descs(base, layers, pool_blocks, blk, block_ids, order):
+    """One descriptor per (block, layer, K|V) in a pool laid out [layer][K|V][block][blk], listed
+    layer by layer ("layer": the order in which per-layer registrations are walked) or block by
+    block ("block": all 64 sub-blocks of one block id together)."""
     block_ids = np.asarray(block_ids, dtype=np.uint64)
     lk = np.arange(layers * 2, dtype=np.uint64)
-    addr = (np.uint64(base) + lk[None, :] * np.uint64(pool_blocks * blk) + block_ids[:, None] * np.uint64(blk))
-    return addr.reshape(-1)
+    addr = (np.uint64(base) + lk[:, None] * np.uint64(pool_blocks * blk) + block_ids[None, :] * np.uint64(blk))
+    return (addr if order == "layer" else addr.T).reshape(-1)
 
 
 def _triples(addrs, blk):
@@ -83,8 +85,8 @@ def run_kv(args):
     sel = rng.choice(pool_blocks, n_sel, replace=False)
     dst_ids = rng.permutation(pool_blocks)[:n_sel]
     n_desc = n_sel * lk
-    src_addrs = _kv_descs(src_pool.data_ptr(), layers, pool_blocks, blk, sel)
-    dst_addrs = _kv_descs(dst_pool.data_ptr(), layers, pool_blocks, blk, dst_ids)
+    src_addrs = _kv_descs(src_pool.data_ptr(), layers, pool_blocks, blk, sel, args.order)
+    dst_addrs = _kv_descs(dst_pool.data_ptr(), layers, pool_blocks, blk, dst_ids, args.order)
     stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
 
     t0 = time.perf_counter()
@@ -316,8 +318,8 @@ def run_cpu_baseline(seconds=12.0, threads=1):
     sel = rng.choice(pool_blocks, n_sel, replace=False)
     dst_ids = rng.permutation(pool_blocks)[:n_sel]
     n_desc = n_sel * lk
-    src_addrs = _kv_descs(src_pool.ctypes.data, layers, pool_blocks, blk, sel)
-    dst_addrs = _kv_descs(dst_pool.ctypes.data, layers, pool_blocks, blk, dst_ids)
+    src_addrs = _kv_descs(src_pool.ctypes.data, layers, pool_blocks, blk, sel, "layer")
+    dst_addrs = _kv_descs(dst_pool.ctypes.data, layers, pool_blocks, blk, dst_ids, "layer")
     stg_addrs = np.uint64(staging.ctypes.data) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
     h_src = agent.prep_xfer_dlist("", _triples(src_addrs, blk), "DRAM")
     h_stg_r = agent.prep_xfer_dlist("cpu", _triples(stg_addrs, blk), "DRAM")
@@ -358,6 +360,8 @@ def main():
     ap.add_argument("--pool-blocks", type=int, default=8192)
     ap.add_argument("--block-bytes", type=int, default=0,
                     help="bytes per (layer, K|V) sub-block; 0: what the model gives (32768)")
+    ap.add_argument("--order", choices=("layer", "block"), default="layer",
+                    help="descriptor list order: layer by layer, or block by block")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ep", action="store_true")
     ap.add_argument("--no-small", action="store_true", help="skip the small-descriptor stress")

@@ -48,7 +48,10 @@ typedef struct nixl_amd_copy_desc {
 /* Launch-shape knobs.  Zero in any field selects the built-in default. */
 typedef struct nixl_amd_copy_tuning {
     int units_per_lane; /* 16-byte units one lane moves per chunk: 1, 2, 4, 8 or 16 */
-    int nontemporal; /* 1 = non-temporal loads/stores, 2 = plain; 0 = default */
+    int nontemporal; /* cache policy: 1 = non-temporal loads and stores, 2 = plain, 3 = plain loads and
+                      * streaming device-scope stores, 4 = non-temporal loads and streaming
+                      * device-scope stores; 0 = 4 if the destinations of consecutive
+                      * descriptors adjoin or advance by a constant step, else 3 */
     int max_workgroups; /* grid cap of the mixed and byte-path kernels; waves loop beyond it */
     int waves_per_workgroup; /* uniform-chunk kernel: 1, 2, 4, 8 or 16 */
     int xcd_swizzle; /* 1 = each accelerator die walks a contiguous slice of the chunk list, 2 = off */

@@ -76,21 +76,37 @@ using v4u = __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned;
 using gv4_ptr = __attribute__((address_space(1))) v4u *;
 using gv4_cptr = const __attribute__((address_space(1))) v4u *;
 
-template<bool NT>
+// Cache policy of a plan's loads and stores (tuning field `nontemporal`), measured on MI355X
+// with 16 KiB blocks (TB/s of traffic; sequential = consecutive descriptors adjoin):
+//                                     seq->seq  random->seq  seq->random  random->random
+//   1  nt loads,    nt stores           6.66       6.28         5.76          5.12
+//   2  plain loads, plain stores        6.44       5.30         5.80          5.12
+//   3  plain loads, sc1 nt stores       6.65       6.07         5.90          5.31
+//   4  nt loads,    sc1 nt stores       6.71       6.35         5.80          5.15
+// "sc1 nt" is a streaming store with device scope.  A plan whose destinations adjoin or
+// advance by a constant step takes 4, any other plan 3.
+constexpr int kPolNtNt = 1, kPolPlain = 2, kPolPlainSc1Nt = 3, kPolNtSc1Nt = 4;
+
+template<int POL>
 __device__ __forceinline__ v4u
 load16(uint64_t addr) {
     gv4_cptr g = (gv4_cptr)(addr);
-    return NT ? __builtin_nontemporal_load(g) : *g;
+    if constexpr (POL == kPolNtNt || POL == kPolNtSc1Nt)
+        return __builtin_nontemporal_load(g);
+    else
+        return *g;
 }
 
-template<bool NT>
+template<int POL>
 __device__ __forceinline__ void
 store16(uint64_t addr, const v4u &v) {
     gv4_ptr g = (gv4_ptr)(addr);
-    if constexpr (NT)
+    if constexpr (POL == kPolNtNt)
         __builtin_nontemporal_store(v, g);
-    else
+    else if constexpr (POL == kPolPlain)
         *g = v;
+    else
+        asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(g), "v"(v) : "memory");
 }
 
 // Workgroups are handed to the 8 dies round-robin.  With the swizzle on, die x works
@@ -107,14 +123,14 @@ logical_workgroup(uint32_t n_wgs, bool swizzle) {
 // consecutive chunks of one descriptor (1 when the runs of such chunks differ in length;
 // with equal-length descriptors, e.g. KV blocks, one record per descriptor), so that the
 // record array stays small next to the payload.
-template<int UPL, bool NT, int WAVES>
+template<int UPL, int POL, int WAVES>
 __global__ void __launch_bounds__(kWaveSize *WAVES)
-copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, int swizzle, uint32_t chunks_per_rec) {
+copy_uniform_kernel(const UniformRec *recs, uint32_t first_chunk, uint32_t n_chunks, uint32_t n_wgs, int swizzle, uint32_t chunks_per_rec) {
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t wave = threadIdx.x / kWaveSize;
     const uint32_t wg = logical_workgroup(n_wgs, swizzle != 0);
-    const uint32_t c = uniform(wg * WAVES + wave);
-    if (wg >= n_wgs || c >= n_chunks) return;
+    if (wg >= n_wgs || wg * WAVES + wave >= n_chunks) return;
+    const uint32_t c = uniform(first_chunk + wg * WAVES + wave); // n_chunks, n_wgs: of this launch
     const uint32_t r = c / chunks_per_rec;
     const uint64_t off = static_cast<uint64_t>(c % chunks_per_rec) * (kWaveSize * UPL * 16u) + lane * 16u;
     const uint64_t s = uniform64(recs[r].src) + off;
@@ -122,10 +138,10 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, i
     v4u v[UPL];
 #pragma unroll
     for (int k = 0; k < UPL; ++k)
-        v[k] = load16<NT>(s + k * (kWaveSize * 16u));
+        v[k] = load16<POL>(s + k * (kWaveSize * 16u));
 #pragma unroll
     for (int k = 0; k < UPL; ++k)
-        store16<NT>(d + k * (kWaveSize * 16u), v[k]);
+        store16<POL>(d + k * (kWaveSize * 16u), v[k]);
 }
 
 // One wavefront per piece: the descriptor's own {src, dst, units} record, up to
@@ -135,9 +151,9 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t n_chunks, uint32_t n_wgs, i
 constexpr int kPieceLoads = 4;
 constexpr uint32_t kPieceUnits = kWaveSize * kPieceLoads; // 4 KiB
 
-template<bool NT, int LOADS, int WAVES>
+template<int POL, int LOADS, int WAVES>
 __global__ void __launch_bounds__(kWaveSize *WAVES)
-copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) {
+copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) { // recs, n_recs: of this launch
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
     const uint32_t p = uniform(blockIdx.x * WAVES + threadIdx.x / kWaveSize);
     if (p >= n_recs) return;
@@ -150,15 +166,15 @@ copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) {
 #pragma unroll
     for (int k = 0; k < LOADS; ++k) {
         const uint32_t u = min(k * kWaveSize + lane, units - 1);
-        v[k] = load16<NT>(rec.src + u * 16ull);
+        v[k] = load16<POL>(rec.src + u * 16ull);
     }
 #pragma unroll
     for (int k = 0; k < LOADS; ++k)
-        if (k * kWaveSize + lane < units) store16<NT>(d + k * (kWaveSize * 16u), v[k]);
+        if (k * kWaveSize + lane < units) store16<POL>(d + k * (kWaveSize * 16u), v[k]);
 }
 
 // One wavefront per chunk that crosses descriptor boundaries or is short.
-template<int UPL, bool NT>
+template<int UPL, int POL>
 __global__ void __launch_bounds__(kMixedThreads)
 copy_mixed_kernel(MixedArgs a) {
     constexpr uint32_t kChunkUnits = kWaveSize * UPL;
@@ -214,10 +230,10 @@ copy_mixed_kernel(MixedArgs a) {
             }
 #pragma unroll
             for (int k = 0; k < UPL; ++k)
-                if (sa[k]) v[k] = load16<NT>(sa[k]);
+                if (sa[k]) v[k] = load16<POL>(sa[k]);
 #pragma unroll
             for (int k = 0; k < UPL; ++k)
-                if (da[k]) store16<NT>(da[k], v[k]);
+                if (da[k]) store16<POL>(da[k], v[k]);
             __builtin_amdgcn_wave_barrier();
         } else {
             // More than 64 tiny descriptors in one chunk: bisect the global prefix array.
@@ -232,7 +248,7 @@ copy_mixed_kernel(MixedArgs a) {
                         hi = mid - 1;
                 }
                 const uint64_t off = (u - a.prefix[lo]) * 16u;
-                store16<NT>(a.dst[lo] + off, load16<NT>(a.src[lo] + off));
+                store16<POL>(a.dst[lo] + off, load16<POL>(a.src[lo] + off));
             }
         }
     }
@@ -279,40 +295,80 @@ copy_generic_kernel(const GenericItem *items, uint32_t n_items) {
     }
 }
 
-template<int UPL, bool NT>
+// Largest grid of one launch: HIP refuses grids of 2^32 or more threads, i.e. 2^22 workgroups of
+// 16 waves; a plan with more work than that goes out as several launches.
+constexpr uint32_t kMaxGrid = 1u << 21;
+
+struct UniformLaunch {
+    const UniformRec *recs;
+    uint32_t first_chunk, n_chunks, n_wgs, chunks_per_rec;
+    int swizzle;
+    dim3 grid;
+    hipStream_t stream;
+};
+
+template<int UPL, int POL>
 void
-launch_uniform(int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz, uint32_t cpr) {
+launch_uniform(int waves, const UniformLaunch &u) {
+#define NIXL_AMD_UNIFORM(WV)                                                                              \
+    hipLaunchKernelGGL((copy_uniform_kernel<UPL, POL, WV>), u.grid, dim3(kWaveSize * WV), 0, u.stream, u.recs, \
+                       u.first_chunk, u.n_chunks, u.n_wgs, u.swizzle, u.chunks_per_rec)
     switch (waves) {
-    case 1: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 1>), grid, dim3(64), 0, s, recs, n, n_wgs, swz, cpr); break;
-    case 2: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 2>), grid, dim3(128), 0, s, recs, n, n_wgs, swz, cpr); break;
-    case 4: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 4>), grid, dim3(256), 0, s, recs, n, n_wgs, swz, cpr); break;
-    case 8: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 8>), grid, dim3(512), 0, s, recs, n, n_wgs, swz, cpr); break;
-    default: hipLaunchKernelGGL((copy_uniform_kernel<UPL, NT, 16>), grid, dim3(1024), 0, s, recs, n, n_wgs, swz, cpr); break;
+    case 1: NIXL_AMD_UNIFORM(1); break;
+    case 2: NIXL_AMD_UNIFORM(2); break;
+    case 4: NIXL_AMD_UNIFORM(4); break;
+    case 8: NIXL_AMD_UNIFORM(8); break;
+    default: NIXL_AMD_UNIFORM(16); break;
     }
+#undef NIXL_AMD_UNIFORM
 }
 
-template<bool NT>
+template<int POL>
 void
-launch_uniform_upl(int upl, int waves, dim3 grid, hipStream_t s, const UniformRec *recs, uint32_t n, uint32_t n_wgs, int swz, uint32_t cpr) {
+launch_uniform_upl(int upl, int waves, const UniformLaunch &u) {
     switch (upl) {
-    case 1: launch_uniform<1, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
-    case 2: launch_uniform<2, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
-    case 4: launch_uniform<4, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
-    case 8: launch_uniform<8, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
-    default: launch_uniform<16, NT>(waves, grid, s, recs, n, n_wgs, swz, cpr); break;
+    case 1: launch_uniform<1, POL>(waves, u); break;
+    case 2: launch_uniform<2, POL>(waves, u); break;
+    case 4: launch_uniform<4, POL>(waves, u); break;
+    case 8: launch_uniform<8, POL>(waves, u); break;
+    default: launch_uniform<16, POL>(waves, u); break;
     }
 }
 
-template<bool NT>
+template<int POL>
 void
 launch_mixed_upl(int upl, dim3 grid, hipStream_t s, const MixedArgs &a) {
     const dim3 block(kMixedThreads);
     switch (upl) {
-    case 1: hipLaunchKernelGGL((copy_mixed_kernel<1, NT>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((copy_mixed_kernel<2, NT>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((copy_mixed_kernel<4, NT>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((copy_mixed_kernel<8, NT>), grid, block, 0, s, a); break;
-    default: hipLaunchKernelGGL((copy_mixed_kernel<16, NT>), grid, block, 0, s, a); break;
+    case 1: hipLaunchKernelGGL((copy_mixed_kernel<1, POL>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((copy_mixed_kernel<2, POL>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((copy_mixed_kernel<4, POL>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((copy_mixed_kernel<8, POL>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((copy_mixed_kernel<16, POL>), grid, block, 0, s, a); break;
+    }
+}
+
+template<int POL>
+void
+launch_pieces(uint32_t w, dim3 grid, hipStream_t s, const PieceRec *recs, uint32_t n) {
+    const dim3 block(kWaveSize * w);
+    if (w == 1)
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 1>), grid, block, 0, s, recs, n);
+    else if (w == 2)
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 2>), grid, block, 0, s, recs, n);
+    else
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 4>), grid, block, 0, s, recs, n);
+}
+
+// Calls f.template operator()<POL>() for the plan's policy.
+template<typename F>
+void
+with_policy(int policy, F &&f) {
+    switch (policy) {
+    case kPolNtNt: f.template operator()<kPolNtNt>(); break;
+    case kPolPlain: f.template operator()<kPolPlain>(); break;
+    case kPolPlainSc1Nt: f.template operator()<kPolPlainSc1Nt>(); break;
+    default: f.template operator()<kPolNtSc1Nt>(); break;
     }
 }
 
@@ -321,7 +377,7 @@ launch_mixed_upl(int upl, dim3 grid, hipStream_t s, const MixedArgs &a) {
 struct nixl_amd_copy_plan {
     int device = 0;
     int upl = 1;
-    bool nt = true;
+    int policy = kPolNtSc1Nt;
     int waves = 1;
     int swizzle = 0;
     uint32_t max_wgs = 0;
@@ -357,8 +413,9 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     if (n >= (1ull << 32)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: more than 2^32-1 descriptors");
 
     // Defaults from a sweep on MI355X: the smallest chunk (one 128-bit load and store per
-    // lane, one wave per workgroup) with non-temporal accesses gave the highest HBM rate.
-    int upl = 1, nt = 1, waves = 1, swizzle = 0;
+    // lane, one wave per workgroup) gave the highest HBM rate; the cache policy follows the
+    // destination pattern (below).
+    int upl = 1, nt = 0, waves = 1, swizzle = 0;
     uint32_t max_wgs = 0;
     if (tuning) {
         if (tuning->units_per_lane) upl = tuning->units_per_lane;
@@ -369,7 +426,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     }
     if (upl != 1 && upl != 2 && upl != 4 && upl != 8 && upl != 16)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 1, 2, 4, 8 or 16");
-    if (nt != 1 && nt != 2) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0, 1 or 2");
+    if (nt < 0 || nt > 4) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0 to 4");
     if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: waves_per_workgroup must be 1, 2, 4, 8 or 16");
 
@@ -510,7 +567,25 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     auto *plan = new nixl_amd_copy_plan();
     plan->device = device;
     plan->upl = upl;
-    plan->nt = (nt == 1);
+    if (nt == 0) {
+        // Destinations that adjoin (a gather into staging, one long copy) or advance by a
+        // constant step (the same block of every layer of a pool) take non-temporal loads;
+        // destinations without such a pattern (a scatter over a pool) take plain loads.
+        uint64_t pairs = 0, regular = 0, prev_dst = 0, prev_end = 0, prev_step = 0;
+        for (size_t i = 0; i < n; ++i) {
+            if (descs[i].len == 0) continue;
+            if (prev_end) {
+                const uint64_t step = descs[i].dst - prev_dst;
+                ++pairs;
+                regular += (descs[i].dst == prev_end || step == prev_step);
+                prev_step = step;
+            }
+            prev_dst = descs[i].dst;
+            prev_end = descs[i].dst + descs[i].len;
+        }
+        nt = (pairs == 0 || 2 * regular >= pairs) ? kPolNtSc1Nt : kPolPlainSc1Nt;
+    }
+    plan->policy = nt;
     plan->waves = waves;
     plan->swizzle = swizzle;
     plan->max_wgs = max_wgs;
@@ -560,6 +635,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     auto wgs_for = [&](uint32_t n_waves, uint32_t waves_per_wg, bool cap) {
         uint32_t w = (n_waves + waves_per_wg - 1) / waves_per_wg;
         if (cap && plan->max_wgs && w > plan->max_wgs) w = plan->max_wgs;
+        if (cap && w > kMaxGrid) w = kMaxGrid; // those kernels loop over their work items
         return w;
     };
     plan->uniform_wgs = wgs_for(plan->n_uniform, static_cast<uint32_t>(waves), false);
@@ -588,36 +664,37 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
     HIP_TRY(on_device.status());
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (plan->uniform_wgs) {
-        // With the die swizzle the grid is rounded up to a multiple of 8 so that every
-        // die owns an equally long slice; surplus workgroups exit at once.
-        uint32_t grid = plan->uniform_wgs;
-        if (plan->swizzle) grid = ((grid + kNumXcd - 1) / kNumXcd) * kNumXcd;
-        if (plan->nt)
-            launch_uniform_upl<true>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
-                                     plan->uniform_wgs, plan->swizzle, plan->chunks_per_rec);
-        else
-            launch_uniform_upl<false>(plan->upl, plan->waves, dim3(grid), s, plan->uniform_recs, plan->n_uniform,
-                                      plan->uniform_wgs, plan->swizzle, plan->chunks_per_rec);
-        HIP_TRY(hipGetLastError());
+        // One launch per kMaxGrid workgroups.  With the die swizzle each launch's grid is
+        // rounded up to a multiple of 8 so that every die owns an equally long slice; surplus
+        // workgroups exit at once.
+        const uint32_t waves = static_cast<uint32_t>(plan->waves);
+        for (uint64_t wg64 = 0; wg64 < plan->uniform_wgs; wg64 += kMaxGrid) {
+            const uint32_t wg0 = static_cast<uint32_t>(wg64);
+            UniformLaunch u{};
+            u.recs = plan->uniform_recs;
+            u.first_chunk = wg0 * waves;
+            u.n_chunks = plan->n_uniform - u.first_chunk;
+            u.n_wgs = std::min(kMaxGrid, plan->uniform_wgs - wg0);
+            u.chunks_per_rec = plan->chunks_per_rec;
+            u.swizzle = plan->swizzle;
+            u.grid = dim3(plan->swizzle ? ((u.n_wgs + kNumXcd - 1) / kNumXcd) * kNumXcd : u.n_wgs);
+            u.stream = s;
+            with_policy(plan->policy, [&]<int POL>() { launch_uniform_upl<POL>(plan->upl, plan->waves, u); });
+            HIP_TRY(hipGetLastError());
+        }
     }
     if (plan->n_pieces) {
         const uint32_t w = static_cast<uint32_t>(plan->waves > 4 ? 4 : plan->waves);
-        const dim3 grid((plan->n_pieces + w - 1) / w), block(kWaveSize * w);
-#define NIXL_AMD_PIECE(NTV, WV) \
-    hipLaunchKernelGGL((copy_piece_kernel<NTV, kPieceLoads, WV>), grid, block, 0, s, plan->piece_recs, plan->n_pieces)
-        if (plan->nt) {
-            if (w == 1) NIXL_AMD_PIECE(true, 1); else if (w == 2) NIXL_AMD_PIECE(true, 2); else NIXL_AMD_PIECE(true, 4);
-        } else {
-            if (w == 1) NIXL_AMD_PIECE(false, 1); else if (w == 2) NIXL_AMD_PIECE(false, 2); else NIXL_AMD_PIECE(false, 4);
+        const uint32_t per_launch = kMaxGrid * w;
+        for (uint32_t p0 = 0; p0 < plan->n_pieces; p0 += per_launch) {
+            const uint32_t n = std::min(per_launch, plan->n_pieces - p0);
+            with_policy(plan->policy,
+                        [&]<int POL>() { launch_pieces<POL>(w, dim3((n + w - 1) / w), s, plan->piece_recs + p0, n); });
+            HIP_TRY(hipGetLastError());
         }
-#undef NIXL_AMD_PIECE
-        HIP_TRY(hipGetLastError());
     }
     if (plan->mixed_wgs) {
-        if (plan->nt)
-            launch_mixed_upl<true>(plan->upl, dim3(plan->mixed_wgs), s, plan->mixed_args);
-        else
-            launch_mixed_upl<false>(plan->upl, dim3(plan->mixed_wgs), s, plan->mixed_args);
+        with_policy(plan->policy, [&]<int POL>() { launch_mixed_upl<POL>(plan->upl, dim3(plan->mixed_wgs), s, plan->mixed_args); });
         HIP_TRY(hipGetLastError());
     }
     if (plan->generic_wgs) {

@@ -58,7 +58,7 @@ def _disjoint_layout(rng, lens, align, region):
 
 
 @pytest.mark.parametrize("upl", [1, 2, 4, 8, 16])
-@pytest.mark.parametrize("nt", [1, 2])
+@pytest.mark.parametrize("nt", [1, 2, 3, 4])
 def test_aligned_descriptors_match_oracle(cuda, upl, nt):
     import torch
     rng = np.random.default_rng(upl * 10 + nt)
