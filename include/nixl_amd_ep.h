@@ -34,9 +34,9 @@ extern "C" {
 int
 nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes);
 
-/* Bytes of scratch the low-latency dispatch needs (per-(rank, expert) send counts,
- * per-(token, k) rows, per-token scales); the scratch must be 4-byte aligned.  Reference:
- * `workspace` of ep_kernels::dispatch, kernels/nixl_ep_ll.cu:423-426. */
+/* Bytes of scratch the low-latency dispatch needs (one 64-bit word of selection bits per
+ * (expert, rank, 64 tokens), a flag per 64 tokens, per-token scales, a 256-byte header); the
+ * scratch must be 16-byte aligned.  Reference: `workspace` of ep_kernels::dispatch, kernels/nixl_ep_ll.cu:423-426. */
 size_t
 nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk, int hidden);
 
@@ -46,7 +46,11 @@ nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, i
  * csrc/nixl_ep.cpp:1030-1143).
  *   x                      [R][T][H] bf16
  *   topk_idx               [R][T][K] int32, -1 = no selection; the K entries of one token
- *                          must be distinct (as a top-k selection is)
+ *                          must be distinct (as a top-k selection is).  The reference gives a
+ *                          repeated expert a row of its own (kernels/nixl_ep_ll.cu:186-190); here
+ *                          the repeats share one row, and the call reports it:
+ *                          nixl_amd_ep_ll_dispatch_status then returns
+ *                          NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT
  *   num_tokens_per_rank    [R] int32 tokens present on each rank (<= T), or NULL = T
  *   mask_buffer            [R][R] int32 or NULL; tokens travel a -> b only if neither
  *                          mask[a][b] nor mask[b][a] is set (kernels/nixl_ep_ll.cu:197,266,319)
@@ -89,6 +93,52 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                         void *stream);
 
 /*
+ * Routing and low-latency dispatch in one call: nixl_amd_ep_ll_dispatch with the top-k
+ * selection done first, by the kernel that prepares the dispatch (no launch of its own).
+ * The reference's callers bring their own top-k (tests/elastic/elastic.py:153-158); this is
+ * the north-star's "dispatch does top-k routing".
+ *   logits        [R][T][E] float, in
+ *   topk_idx      [R][T][K] int32, out: the K largest logits of each token, descending, ties
+ *                 to the lower expert index (what nixl_amd_ep_router_topk returns)
+ *   topk_weights  [R][T][K] float, out: softmax over those K logits
+ * num_experts <= 1024.  Everything else as nixl_amd_ep_ll_dispatch.
+ */
+int
+nixl_amd_ep_ll_route_dispatch(void *packed_recv_x,
+                              void *packed_recv_x_scales,
+                              int *packed_recv_src_info,
+                              int64_t *packed_recv_layout_range,
+                              int *packed_recv_count,
+                              const int *mask_buffer,
+                              int *cumulative_local_expert_recv_stats,
+                              const void *x,
+                              const float *logits,
+                              int32_t *topk_idx,
+                              float *topk_weights,
+                              const int *num_tokens_per_rank,
+                              int num_tokens,
+                              int hidden,
+                              int num_max_dispatch_tokens_per_rank,
+                              int num_topk,
+                              int num_ranks,
+                              int num_experts,
+                              int use_fp8,
+                              int round_scale,
+                              int use_ue8m0,
+                              int *row_map,
+                              void *workspace,
+                              size_t workspace_bytes,
+                              void *stream);
+
+/* Status of the last dispatch that used `workspace`, read back after waiting for `stream`:
+ * 0, or NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT if some token's top-k named an expert twice (the
+ * reference would have delivered that token to the expert twice; here it arrives once).  No
+ * reference counterpart: the reference has no such restriction. */
+#define NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT 1
+int
+nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status);
+
+/*
  * Low-latency dispatch that allocates nothing.  No counterpart in the reference; it is for
  * callers that cannot allocate device memory: code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc.  Arguments and results are those of
@@ -99,7 +149,7 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
  * two calls may not overlap on one GPU (different streams, or threads), or they race.  The
  * call itself issues no hipMalloc, hipFree, memset or other allocating routine.
  */
-#define NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES (4u << 20)
+#define NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES (2u << 20)
 int
 nixl_amd_ep_ll_dispatch_static(void *packed_recv_x,
                                void *packed_recv_x_scales,

@@ -79,6 +79,8 @@ def kernels_error():
 
 _EP_SIGS = {
     "nixl_amd_ep_ll_dispatch": [c_void_p] * 10 + [c_int] * 9 + [c_void_p, c_void_p, c_size_t, c_void_p],
+    "nixl_amd_ep_ll_route_dispatch": [c_void_p] * 12 + [c_int] * 9 + [c_void_p, c_void_p, c_size_t, c_void_p],
+    "nixl_amd_ep_ll_dispatch_status": [c_void_p, c_void_p, POINTER(c_int)],
     "nixl_amd_ep_ll_dispatch_static": [c_void_p] * 10 + [c_int] * 9 + [c_void_p, c_void_p],
     "nixl_amd_ep_ll_combine": [c_void_p] * 9 + [c_int] * 7 + [c_void_p],
     "nixl_amd_ep_get_dispatch_layout": [c_void_p] * 4 + [c_int] * 4 + [c_void_p],

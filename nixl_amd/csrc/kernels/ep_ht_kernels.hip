@@ -690,36 +690,6 @@ ht_combine_kernel(uint16_t *__restrict__ combined,
 // lane 63.  Cross-lane permutes through LDS took three times as long.
 constexpr int kRouterMaxPerLane = 16; // E <= 1024
 
-template<int CTRL, int ROW_MASK>
-__device__ __forceinline__ int
-dpp_move(int x) {
-    // lanes whose row is masked out, or whose source lane does not exist, keep x
-    return __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xf, false);
-}
-
-// Reduction of one 32-bit value per lane over the wave; every lane of the last row (and so
-// lane 63) holds the result.  op must be idempotent (max, min).
-template<typename Op>
-__device__ __forceinline__ int
-wave_reduce_dpp(int x, Op op) {
-    x = op(x, dpp_move<0xb1, 0xf>(x));  // quad_perm [1,0,3,2]
-    x = op(x, dpp_move<0x4e, 0xf>(x));  // quad_perm [2,3,0,1]
-    x = op(x, dpp_move<0x124, 0xf>(x)); // row_ror 4
-    x = op(x, dpp_move<0x128, 0xf>(x)); // row_ror 8
-    x = op(x, dpp_move<0x142, 0xa>(x)); // row_bcast 15 into rows 1 and 3
-    x = op(x, dpp_move<0x143, 0xc>(x)); // row_bcast 31 into rows 2 and 3
-    return __builtin_amdgcn_readlane(x, kWaveSize - 1);
-}
-
-// Order-preserving map of a float onto a signed integer (negative floats reversed), so that
-// integer max is float max; -0.0 and +0.0 stay distinct neighbours, which the tie rule of the
-// values below undoes by comparing the floats themselves.
-__device__ __forceinline__ int
-float_order_key(float f) {
-    const int b = __float_as_int(f);
-    return b >= 0 ? b : b ^ 0x7fffffff;
-}
-
 // PL = experts a lane holds (a power of two >= ceil(E / 64)): the argmax rounds only walk
 // the slots that exist.
 template<int PL>
@@ -738,31 +708,8 @@ router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, 
     }
     float sel_v[16];
     int sel_i[16];
-    for (int k = 0; k < K; ++k) {
-        float best = 0.f;
-        int best_e = 0x7fffffff;
-#pragma unroll
-        for (int j = 0; j < PL; ++j) {
-            const int e = j * kWaveSize + lane;
-            if (!((taken >> j) & 1u) && (best_e == 0x7fffffff || v[j] > best)) {
-                best = v[j];
-                best_e = e;
-            }
-        }
-        const bool have = best_e != 0x7fffffff;
-        // largest value among the lanes that still have one
-        const int key = have ? float_order_key(best) : static_cast<int>(0x80000000);
-        const int top_key = wave_reduce_dpp(key, [](int a, int b) { return a > b ? a : b; });
-        const float top = __int_as_float(top_key >= 0 ? top_key : top_key ^ 0x7fffffff);
-        // lowest expert index among the lanes that hold a value equal to it (0.0 == -0.0)
-        const int cand = (have && best == top) ? best_e : 0x7fffffff;
-        int win = wave_reduce_dpp(cand, [](int a, int b) { return a < b ? a : b; });
-        if (win == 0x7fffffff) // only NaNs are left: take them in index order
-            win = wave_reduce_dpp(have ? best_e : 0x7fffffff, [](int a, int b) { return a < b ? a : b; });
-        if ((win & (kWaveSize - 1)) == lane) taken |= 1u << (win / kWaveSize);
-        sel_v[k] = top;
-        sel_i[k] = win;
-    }
+    for (int k = 0; k < K; ++k)
+        router_round<PL>(v, taken, lane, sel_v[k], sel_i[k]);
     if (lane == 0) {
         const float top = sel_v[0];
         float ex[16], sum = 0.f;

@@ -6,20 +6,22 @@
 // per-expert contiguous output; kernels/nixl_ep_ll.cu:134-393) is done here in two
 // launches that touch the payload once, because every "remote" slot is an address in the
 // same HBM:
-//   1. ll_layout_kernel    one workgroup per source rank builds, in LDS, one bitmask of
-//                          tokens per expert and derives count[r][e] and the position of
-//                          every (token, k) inside its (r, e) segment;
-//   2. ll_dispatch_kernel  one workgroup per token reads its bf16 row once, quantises it in
-//                          registers and writes it straight to its K final rows of
-//                          packed_recv_x (row = e * N + sum of the lower source ranks'
-//                          counts for e + position), plus src_info and the token's H/128
-//                          scales (once, contiguous);
-//   3. ll_scales_kernel    workgroups per expert scan the per-rank counts into layout_range,
-//                          recv_count and the statistics, and copy each received row's
-//                          scales into the column-major scales array with coalesced stores
-//                          (writing them from step 2 would be one isolated 4-byte store per
-//                          scale).
-// Steps 1 and 3 move a few megabytes; step 2 moves the payload.
+//   1. ll_bits_kernel      one workgroup per 64 consecutive tokens of a rank builds, in LDS,
+//                          one 64-bit word per expert (bit j: token j of the group selected the
+//                          expert) and writes it to bits[e][rank][group]: every word has one
+//                          writer, so nothing is cleared beforehand and nothing is atomic in
+//                          global memory.  With logits instead of top-k indices the same
+//                          kernel does the routing first (a wave per token, four tokens per
+//                          wave) and writes the indices and weights out as well.
+//   2. ll_dispatch_kernel  one workgroup per token reads its bf16 row once and, while the row
+//                          travels, counts for each of its K experts the bits in front of its
+//                          own (tokens of lower ranks, then lower tokens of its rank): that is
+//                          its row inside the expert.  It quantises the row in registers and
+//                          writes it straight to its K final rows of packed_recv_x, plus
+//                          src_info and the scales in their column-major place.  Workgroup e
+//                          also turns expert e's bits into layout_range, recv_count and the
+//                          statistics.
+// Step 1 moves 0.3 MB; step 2 moves the payload.
 // The order this produces is the canonical one among those the reference's atomics allow:
 // segments by source rank ascending, tokens ascending inside a segment.
 //
@@ -39,10 +41,12 @@
 
 namespace {
 
-constexpr int kLayoutThreads = 1024; // one (token, k) per thread at 128 tokens x top-8
-constexpr int kScaleThreads = 256;
-constexpr int kLayoutLdsBytes = 32768;
+constexpr int kBitsThreads = 256; // index path: two (token, k) entries per thread at top-8
+constexpr int kRouteThreads = 1024; // routing path: 16 waves, four tokens each
+constexpr int kGroupTokens = 64; // tokens per word of the selection bits
 constexpr int kMaxTopk = 16; // reference limit, kernels/nixl_ep_ll.cu:412,421
+constexpr int kRouterMaxPerLane = 16; // E <= 1024 when routing
+constexpr size_t kWorkspaceHeader = 256; // [0]: status of the last dispatch on this workspace
 
 struct LlDims {
     int R, T, H, K, E, El, M, N;
@@ -53,81 +57,176 @@ pair_blocked(const int *mask, int R, int a, int b) {
     return mask != nullptr && (mask[a * R + b] != 0 || mask[b * R + a] != 0);
 }
 
-// ---- 1. counts and positions ------------------------------------------------------------
+__device__ __forceinline__ int
+wave_sum(int v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+        v += __shfl_xor(v, off);
+    return v;
+}
 
-// grid = R workgroups.  send_count [R][E]; pos [R][T][K] (position inside the (r, e)
-// segment, -1 for no selection / out-of-range expert / blocked rank pair / absent token).
-__global__ void __launch_bounds__(kLayoutThreads)
-ll_layout_kernel(const int32_t *__restrict__ topk_idx,
-                 const int *__restrict__ num_tokens_per_rank,
-                 const int *__restrict__ mask,
-                 int *__restrict__ send_count,
-                 int *__restrict__ pos,
-                 LlDims d,
-                 int experts_per_pass) {
-    extern __shared__ unsigned long long bits[]; // [experts_per_pass][W]
-    const int r = blockIdx.x;
-    const int tid = threadIdx.x;
-    const int W = (d.T + 63) / 64;
-    const int nt = num_tokens_per_rank ? min(num_tokens_per_rank[r], d.T) : d.T;
-    const int32_t *idx = topk_idx + static_cast<size_t>(r) * d.T * d.K;
-    int *my_pos = pos + static_cast<size_t>(r) * d.T * d.K;
+// ---- 1. selection bits (and routing) -------------------------------------------------------------
 
-    for (int p = nt * d.K + tid; p < d.T * d.K; p += kLayoutThreads)
-        my_pos[p] = -1;
+struct BitsArgs {
+    unsigned long long *bits; // [E][R][Wr]
+    int *group_status; // [R][Wr]: 1 if a token of the group names an expert twice
+    int32_t *topk_idx; // [R][T][K]; written when routing, read otherwise
+    float *topk_weights; // [R][T][K], routing only
+    const float *logits; // [R][T][E], routing only
+    const int *num_tokens_per_rank;
+    const int *mask;
+    LlDims d;
+    int Wr; // words (groups of 64 tokens) per rank
+};
 
-    for (int e0 = 0; e0 < d.E; e0 += experts_per_pass) {
-        const int ne = min(experts_per_pass, d.E - e0);
-        for (int i = tid; i < ne * W; i += kLayoutThreads)
-            bits[i] = 0ull;
-        __syncthreads();
-        for (int p = tid; p < nt * d.K; p += kLayoutThreads) {
-            const int e = idx[p];
-            if (e >= e0 && e < e0 + ne) {
-                const int t = p / d.K;
-                atomicOr(&bits[(e - e0) * W + (t >> 6)], 1ull << (t & 63));
+// grid = R * Wr workgroups; dynamic LDS: E words.
+template<bool ROUTE, int PL>
+__global__ void __launch_bounds__(ROUTE ? kRouteThreads : kBitsThreads)
+ll_bits_kernel(BitsArgs a) {
+    extern __shared__ unsigned long long words[]; // [E]
+    __shared__ int dup;
+    __shared__ int sel_i[ROUTE ? kGroupTokens : 1][kMaxTopk];
+    __shared__ float sel_v[ROUTE ? kGroupTokens : 1][kMaxTopk];
+    const LlDims d = a.d;
+    const int tid = threadIdx.x, n_threads = blockDim.x;
+    const int r = blockIdx.x / a.Wr, t0 = (blockIdx.x % a.Wr) * kGroupTokens;
+    const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
+    for (int e = tid; e < d.E; e += n_threads)
+        words[e] = 0ull;
+    if (tid == 0) dup = 0;
+
+    if constexpr (ROUTE) {
+        // K rounds of a wave-wide argmax per token; lane l holds experts l, l + 64, ...
+        const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize, n_waves = n_threads / kWaveSize;
+        for (int j = wave; j < kGroupTokens && t0 + j < d.T; j += n_waves) {
+            const float *row = a.logits + (static_cast<size_t>(r) * d.T + t0 + j) * d.E;
+            float v[PL];
+            unsigned taken = 0;
+#pragma unroll
+            for (int q = 0; q < PL; ++q) {
+                const int e = q * kWaveSize + lane;
+                v[q] = e < d.E ? row[e] : 0.f;
+                if (e >= d.E) taken |= 1u << q;
+            }
+            for (int k = 0; k < d.K; ++k) {
+                float top;
+                int win;
+                router_round<PL>(v, taken, lane, top, win);
+                if (lane == 0) {
+                    sel_i[j][k] = win;
+                    sel_v[j][k] = top;
+                }
             }
         }
         __syncthreads();
-        for (int i = tid; i < ne; i += kLayoutThreads) {
-            int c = 0;
-            for (int w = 0; w < W; ++w)
-                c += __popcll(bits[i * W + w]);
-            const int e = e0 + i;
-            send_count[r * d.E + e] = pair_blocked(mask, d.R, r, e / d.El) ? 0 : c;
-        }
-        for (int p = tid; p < nt * d.K; p += kLayoutThreads) {
-            const int e = idx[p];
-            if (e0 == 0 && (e < 0 || e >= d.E)) my_pos[p] = -1;
-            if (e >= e0 && e < e0 + ne) {
-                const int t = p / d.K;
-                const unsigned long long *row = bits + (e - e0) * W;
-                int c = __popcll(row[t >> 6] & ((1ull << (t & 63)) - 1ull));
-                for (int w = 0; w < (t >> 6); ++w)
-                    c += __popcll(row[w]);
-                my_pos[p] = pair_blocked(mask, d.R, r, e / d.El) ? -1 : c;
+        // softmax over the K selected logits, one thread per token, summed in selection order
+        if (tid < kGroupTokens && t0 + tid < d.T) {
+            const float top = sel_v[tid][0];
+            float sum = 0.f;
+            for (int k = 0; k < d.K; ++k) {
+                const float ex = expf(sel_v[tid][k] - top);
+                sel_v[tid][k] = ex;
+                sum += ex;
             }
+            for (int k = 0; k < d.K; ++k)
+                sel_v[tid][k] = sel_v[tid][k] / sum;
         }
+        __syncthreads();
+        const size_t base = (static_cast<size_t>(r) * d.T + t0) * d.K;
+        for (int p = tid; p < kGroupTokens * d.K && t0 + p / d.K < d.T; p += n_threads) {
+            a.topk_idx[base + p] = sel_i[p / d.K][p % d.K];
+            a.topk_weights[base + p] = sel_v[p / d.K][p % d.K];
+        }
+    } else {
         __syncthreads();
     }
+
+    const int32_t *idx = a.topk_idx + (static_cast<size_t>(r) * d.T + t0) * d.K;
+    for (int p = tid; p < kGroupTokens * d.K; p += n_threads) {
+        const int j = p / d.K;
+        if (t0 + j >= nt) break;
+        const int e = ROUTE ? sel_i[j][p % d.K] : idx[p];
+        if (e < 0 || e >= d.E || pair_blocked(a.mask, d.R, r, e / d.El)) continue;
+        const unsigned long long old = atomicOr(&words[e], 1ull << j);
+        if ((old >> j) & 1ull) dup = 1; // the same expert twice in one token's selection
+    }
+    __syncthreads();
+    const size_t W = static_cast<size_t>(d.R) * a.Wr;
+    for (int e = tid; e < d.E; e += n_threads)
+        a.bits[e * W + blockIdx.x] = words[e];
+    if (tid == 0) a.group_status[blockIdx.x] = dup;
 }
 
 // ---- 2. cast + scatter ----------------------------------------------------------------------------
 
 struct DispatchArgs {
     uint8_t *recv_x;
-    int *src_info;
     float *token_scales; // [R][T][H/128] inverse scales, one row per source token
+    int *src_info;
+    long long *layout_range;
+    int *recv_count;
+    int *stats;
     const uint16_t *x;
     const int32_t *topk_idx;
     const int *num_tokens_per_rank;
-    const int *send_count; // [R][E]
-    const int *rows; // [R][T][K] position inside the (r, e) segment, -1 if none
-    int *rows_out; // [R][T][K] final row e * N + begin + position, -1 if none
+    const unsigned long long *bits; // [E][R][Wr]
+    const int *group_status; // [R * Wr]
+    int *status; // workspace header
+    int *rows_out; // [R][T][K] final row e * N + slot, -1 if none; may be null
     LlDims d;
+    int Wr;
     int round_scale;
     int parts; // workgroups per token; each covers blockDim.x of the token's H/16 lanes
 };
+
+// layout_range, recv_count and statistics of expert e from its bits; one wave.
+__device__ __forceinline__ void
+expert_meta(const DispatchArgs &a, int e, int lane) {
+    const LlDims d = a.d;
+    const unsigned long long *bw = a.bits + static_cast<size_t>(e) * d.R * a.Wr;
+    int carry = 0;
+    for (int r0 = 0; r0 < d.R; r0 += kWaveSize) {
+        const int r = r0 + lane;
+        int n_r = 0;
+        if (r < d.R)
+            for (int w = 0; w < a.Wr; ++w)
+                n_r += __popcll(bw[static_cast<size_t>(r) * a.Wr + w]);
+        int incl = n_r;
+#pragma unroll
+        for (int off = 1; off < kWaveSize; off <<= 1) {
+            const int up = __shfl_up(incl, off);
+            if (lane >= off) incl += up;
+        }
+        incl += carry;
+        if (r < d.R)
+            a.layout_range[static_cast<size_t>(e) * d.R + r] =
+                static_cast<long long>(static_cast<unsigned>(n_r)) | (static_cast<long long>(incl - n_r) << 32);
+        carry = __shfl(incl, kWaveSize - 1);
+    }
+    if (lane == 0) {
+        a.recv_count[e] = carry;
+        if (a.stats) a.stats[e] += carry;
+    }
+}
+
+// 1 if any group of 64 tokens reported a repeated expert; one wave.
+__device__ __forceinline__ void
+reduce_status(const DispatchArgs &a, int lane) {
+    int any = 0;
+    for (int g = lane; g < a.d.R * a.Wr; g += kWaveSize)
+        any |= a.group_status[g];
+    any = wave_sum(any);
+    if (lane == 0) a.status[0] = any ? NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT : 0;
+}
+
+// For a call without tokens: grid = ceil(E / 4) workgroups of 4 waves, a wave per expert.
+__global__ void __launch_bounds__(256)
+ll_meta_kernel(DispatchArgs a) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int e = blockIdx.x * 4 + threadIdx.x / kWaveSize;
+    if (e < a.d.E) expert_meta(a, e, lane);
+    if (e == 0) reduce_status(a, lane);
+}
 
 // grid = R*T*parts workgroups.  A token's row is H/16 "lanes" of 16 consecutive channels
 // (32 bytes of bf16, 16 bytes of fp8), so a 128-channel scale group is 8 neighbouring
@@ -137,15 +236,17 @@ __global__ void __launch_bounds__(1024)
 ll_dispatch_kernel(DispatchArgs a) {
     const LlDims d = a.d;
     const int tid = threadIdx.x;
+    const int wlane = tid & (kWaveSize - 1), wave = tid / kWaveSize, n_waves = blockDim.x / kWaveSize;
     __shared__ int row_of_k[kMaxTopk]; // e * N + slot, or -1
     const int token = blockIdx.x / a.parts, part = blockIdx.x % a.parts;
     const int r = token / d.T, t = token % d.T;
     const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
-    if (t >= nt) return;
 
-    // The row is requested first so that it travels while the rows are being located.
+    // This token's selections, one per lane, ahead of the row so that they arrive first.
+    const int sel = (wlane < d.K && t < nt) ? a.topk_idx[(static_cast<size_t>(r) * d.T + t) * d.K + wlane] : -1;
+    // The row is requested next so that it travels while the rows are being located.
     const int lane = part * blockDim.x + tid; // lane of the token's row
-    const bool active = lane < d.H / 16;
+    const bool active = lane < d.H / 16 && t < nt;
     uint4 raw0 = make_uint4(0, 0, 0, 0), raw1 = raw0;
     if (active) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.x + (static_cast<size_t>(r) * d.T + t) * d.H) + lane * 2;
@@ -153,24 +254,39 @@ ll_dispatch_kernel(DispatchArgs a) {
         raw1 = ld16_nt(src + 1);
     }
 
+    // Receive-side metadata: the workgroup of token i derives it for experts i, i + R*T, ...
+    if (part == 0 && wave == n_waves - 1)
+        for (int e = token; e < d.E; e += d.R * d.T)
+            expert_meta(a, e, wlane);
+    if (blockIdx.x == 0 && wave == 0) reduce_status(a, wlane);
 
-    // Final row of selection k: e * N + (tokens the lower source ranks send to e) + position.
-    // Half a wave per selection: its 32 lanes fetch the lower ranks' counts in parallel.
+    if (t >= nt) {
+        if (part == 0 && tid < d.K && a.rows_out) a.rows_out[(static_cast<size_t>(r) * d.T + t) * d.K + tid] = -1;
+        return;
+    }
+
+    // Row of selection k inside expert e: the bits of e in front of this token's own bit.
+    // Half a wave per selection: its 32 lanes fetch the words in parallel.
+    const int wi = r * a.Wr + (t >> 6); // this token's word
     for (int k = tid >> 5; k < d.K; k += blockDim.x >> 5) {
         const int q0 = tid & 31;
-        const size_t sel = (static_cast<size_t>(r) * d.T + t) * d.K + k;
-        const int p = a.rows[sel];
-        const int e = a.topk_idx[sel];
-        int partial = 0;
-        if (p >= 0)
-            for (int q = q0; q < r; q += 32)
-                partial += a.send_count[q * d.E + e];
-        partial += __shfl_xor(partial, 16);
-        partial += __shfl_xor(partial, 8);
-        partial += __shfl_xor(partial, 4);
-        partial += __shfl_xor(partial, 2);
-        partial += __shfl_xor(partial, 1);
-        if (q0 == 0) row_of_k[k] = p >= 0 ? e * d.N + partial + p : -1;
+        const int e = __shfl(sel, k);
+        int row = -1, cnt = 0;
+        unsigned long long own = 0ull;
+        if (e >= 0 && e < d.E) {
+            const unsigned long long *bw = a.bits + static_cast<size_t>(e) * d.R * a.Wr;
+            own = bw[wi];
+            if (q0 == 0) cnt = __popcll(own & ((1ull << (t & 63)) - 1ull));
+            for (int j = q0; j < wi; j += 32)
+                cnt += __popcll(bw[j]);
+        }
+        cnt += __shfl_xor(cnt, 16);
+        cnt += __shfl_xor(cnt, 8);
+        cnt += __shfl_xor(cnt, 4);
+        cnt += __shfl_xor(cnt, 2);
+        cnt += __shfl_xor(cnt, 1);
+        if ((own >> (t & 63)) & 1ull) row = e * d.N + cnt;
+        if (q0 == 0) row_of_k[k] = row;
     }
     uint4 q = make_uint4(0, 0, 0, 0);
     if constexpr (FP8) {
@@ -193,16 +309,13 @@ ll_dispatch_kernel(DispatchArgs a) {
             a.token_scales[(static_cast<size_t>(r) * d.T + t) * (d.H / 128) + (lane >> 3)] = scale_inv;
         uint32_t out[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            out[j] = f32_to_e4m3(v[4 * j] * scale) | (f32_to_e4m3(v[4 * j + 1] * scale) << 8) |
-                (f32_to_e4m3(v[4 * j + 2] * scale) << 16) | (f32_to_e4m3(v[4 * j + 3] * scale) << 24);
-        }
+        for (int j = 0; j < 4; ++j)
+            out[j] = e4m3_pack4(v[4 * j] * scale, v[4 * j + 1] * scale, v[4 * j + 2] * scale, v[4 * j + 3] * scale);
         q = make_uint4(out[0], out[1], out[2], out[3]);
     }
     __syncthreads();
-    // Publish the rows (combine reads them back as its row map).  They go to an array of
-    // their own: the other workgroups of this token may still be reading the positions.
-    if (part == 0 && tid < d.K) a.rows_out[(static_cast<size_t>(r) * d.T + t) * d.K + tid] = row_of_k[tid];
+    // Publish the rows (combine reads them back as its row map).
+    if (part == 0 && tid < d.K && a.rows_out) a.rows_out[(static_cast<size_t>(r) * d.T + t) * d.K + tid] = row_of_k[tid];
 
     for (int k = 0; k < d.K; ++k) {
         const int row = row_of_k[k];
@@ -210,122 +323,114 @@ ll_dispatch_kernel(DispatchArgs a) {
         if (lane == 0) a.src_info[row] = t;
         if (!active) continue;
         if constexpr (FP8) {
-            st16_nt(reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H) + lane, q);
+            st16_stream(reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H) + lane, q);
         } else {
             uint4 *dst = reinterpret_cast<uint4 *>(a.recv_x + static_cast<size_t>(row) * d.H * 2) + lane * 2;
-            st16_nt(dst, raw0);
-            st16_nt(dst + 1, raw1);
+            st16_stream(dst, raw0);
+            st16_stream(dst + 1, raw1);
         }
     }
 }
 
-// ---- 3. receive-side metadata and scales, column-major per expert ----------------------------------------------------------------
+// ---- 3. scales, column-major per expert ------------------------------------------------------------
+//
+// packed_recv_x_scales[e] is [G][N] with the row index fastest (csrc/nixl_ep.cpp:1093-1100,
+// kernels/nixl_ep_ll.cu:372-391), so the scales of one received row are G isolated words:
+// written from the dispatch kernel they cost more than a quarter of the payload.  Here a
+// workgroup takes 64 consecutive rows of one expert, finds their source tokens (src_info
+// has the token, the segment the row lies in has the rank), gathers the tokens' scale rows
+// (contiguous, 16 bytes per lane) into LDS and writes them out along the row index, 16 bytes
+// per lane.
 
 struct ScalesArgs {
-    void *recv_scales; // null: metadata only
-    const float *token_scales;
-    const int *src_info;
-    const int *send_count; // [R][E]
-    long long *layout_range;
-    int *recv_count;
-    int *stats;
+    void *recv_scales; // [E][G][N] float, or [E][G/4][N] words of four exponent bytes
+    const float *token_scales; // [R][T][G]
+    const int *src_info; // [E][N]
+    const long long *layout_range; // [E][R]
     LlDims d;
     int use_ue8m0;
-    int parts; // workgroups per expert
+    int parts; // workgroups per expert; each takes every parts-th tile of 64 rows
 };
 
-// grid = E * kScaleParts workgroups.  Every workgroup of expert e scans the R per-rank
-// counts into segment ends (part 0 also writes them out as layout_range, recv_count and the
-// statistics); workgroup (e, part) then copies scale groups part, part + kScaleParts, ... of
-// every received row of expert e.  A thread owns row `slot`
-// (= tid, tid + 256, ...): it finds the row's source rank from the segment ends, then
-// gathers that token's scales (contiguous per token) and writes them at stride N, so that
-// for each scale group the threads of a wave write consecutive addresses (the column-major
-// layout of csrc/nixl_ep.cpp:1093-1100, kernels/nixl_ep_ll.cu:372-391).
-constexpr int kScaleParts = 4; // workgroups per expert; 8 and 14 measured slower
-constexpr int kScaleBatch = 8;
+constexpr int kScaleThreads = 256;
+constexpr int kScaleTile = 64; // rows per tile
+constexpr int kScaleParts = 4;
 
+// dynamic LDS: seg_end[R] ints, then tile[64][C + 1] words (C = G, or G / 4 for exponent
+// bytes), then source[64] ints.
 __global__ void __launch_bounds__(kScaleThreads)
 ll_scales_kernel(ScalesArgs a) {
-    extern __shared__ int seg_end[]; // [R] end of each source rank's segment of expert e
+    extern __shared__ int lds[];
     const LlDims d = a.d;
-    const int parts = a.parts;
-    const int e = blockIdx.x / parts, part = blockIdx.x % parts, tid = threadIdx.x;
     const int G = d.H / 128;
-    if (!a.recv_scales && part != 0) return; // metadata only: one workgroup per expert is enough
-    // the first row's source token is fetched before its validity is known (always in bounds)
-    int t_next = a.src_info[static_cast<size_t>(e) * d.N + min(tid, d.N - 1)];
-    for (int r = tid; r < d.R; r += kScaleThreads)
-        seg_end[r] = a.send_count[r * d.E + e];
-    __syncthreads();
-    if (tid < kWaveSize) {
-        // inclusive scan of the R counts by one wave, 64 ranks per step
-        int carry = 0;
-        for (int r0 = 0; r0 < d.R; r0 += kWaveSize) {
-            const int r = r0 + tid;
-            const int n_r = r < d.R ? seg_end[r] : 0;
-            int incl = n_r;
-#pragma unroll
-            for (int off = 1; off < kWaveSize; off <<= 1) {
-                const int up = __shfl_up(incl, off);
-                if (tid >= off) incl += up;
-            }
-            incl += carry;
-            if (r < d.R) {
-                seg_end[r] = incl;
-                if (part == 0)
-                    a.layout_range[static_cast<size_t>(e) * d.R + r] =
-                        static_cast<long long>(static_cast<unsigned>(n_r)) | (static_cast<long long>(incl - n_r) << 32);
-            }
-            carry = __shfl(incl, kWaveSize - 1);
-        }
-        if (part == 0 && tid == 0) {
-            a.recv_count[e] = carry;
-            if (a.stats) a.stats[e] += carry;
-        }
+    const int C = a.use_ue8m0 ? G / 4 : G; // 32-bit words per row in the output
+    int *seg_end = lds; // [R]: end of each source rank's segment
+    uint32_t *tile = reinterpret_cast<uint32_t *>(lds + d.R); // [64][C + 1]
+    int *source = lds + d.R + kScaleTile * (C + 1); // [64]: r * T + t
+    const int e = blockIdx.x / a.parts, part = blockIdx.x % a.parts, tid = threadIdx.x;
+    const int *info = a.src_info + static_cast<size_t>(e) * d.N;
+
+    // the first tile's source tokens are fetched before it is known how many rows exist (in bounds either way)
+    int s0 = part * kScaleTile;
+    int t_src = (tid < kScaleTile && s0 + tid < d.N) ? info[s0 + tid] : 0;
+    for (int r = tid; r < d.R; r += kScaleThreads) {
+        const long long lr = a.layout_range[static_cast<size_t>(e) * d.R + r];
+        seg_end[r] = static_cast<int>(lr >> 32) + static_cast<int>(lr & 0xffffffffll);
     }
     __syncthreads();
-    if (!a.recv_scales) return;
-    const int n = seg_end[d.R - 1];
-    for (int slot = tid; slot < n; slot += kScaleThreads) {
-        const int t = min(max(t_next, 0), d.T - 1); // written by the dispatch kernel; clamped so that a stale buffer cannot fault
-        if (slot + kScaleThreads < n) t_next = a.src_info[static_cast<size_t>(e) * d.N + slot + kScaleThreads];
-        int lo = 0, hi = d.R - 1; // first rank whose segment ends beyond `slot`
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (seg_end[mid] > slot)
-                hi = mid;
-            else
-                lo = mid + 1;
-        }
-        const float *__restrict__ src = a.token_scales + (static_cast<size_t>(lo) * d.T + t) * G;
-        if (!a.use_ue8m0) {
-            float *__restrict__ dst = static_cast<float *>(a.recv_scales) + static_cast<size_t>(e) * G * d.N + slot;
-            for (int g0 = part; g0 < G; g0 += parts * kScaleBatch) {
-                float v[kScaleBatch];
-#pragma unroll
-                for (int j = 0; j < kScaleBatch; ++j) {
-                    const int g = g0 + j * parts;
-                    v[j] = g < G ? src[g] : 0.f;
-                }
-#pragma unroll
-                for (int j = 0; j < kScaleBatch; ++j) {
-                    const int g = g0 + j * parts;
-                    if (g < G) dst[static_cast<size_t>(g) * d.N] = v[j];
-                }
+    const int n = seg_end[d.R - 1]; // segments follow each other in rank order
+    uint32_t *out = static_cast<uint32_t *>(a.recv_scales) + static_cast<size_t>(e) * C * d.N;
+
+    for (; s0 < n; s0 += a.parts * kScaleTile) {
+        const int rows = min(kScaleTile, n - s0);
+        if (tid < rows) {
+            if (s0 != part * kScaleTile) t_src = info[s0 + tid];
+            int lo = 0, hi = d.R - 1; // first rank whose segment ends beyond this row
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (seg_end[mid] > s0 + tid)
+                    hi = mid;
+                else
+                    lo = mid + 1;
             }
-        } else {
-            // one exponent byte per group, four groups per 32-bit word, words [H/512][N]
-            uint32_t *__restrict__ dst =
-                static_cast<uint32_t *>(a.recv_scales) + static_cast<size_t>(e) * (G / 4) * d.N + slot;
-            for (int g4 = part; g4 < G / 4; g4 += parts) {
-                uint32_t word = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    word |= ((__float_as_uint(src[g4 * 4 + j]) >> 23) & 0xffu) << (8 * j);
-                dst[static_cast<size_t>(g4) * d.N] = word;
+            source[tid] = lo * d.T + min(max(t_src, 0), d.T - 1);
+        }
+        __syncthreads();
+        // gather: G / 4 lanes per row, 16 bytes each
+        const int quads = G / 4;
+        for (int i = tid; i < rows * quads; i += kScaleThreads) {
+            const int row = i / quads, q4 = i % quads;
+            const float4 v = *reinterpret_cast<const float4 *>(a.token_scales + static_cast<size_t>(source[row]) * G + q4 * 4);
+            if (!a.use_ue8m0) {
+                uint32_t *dst = tile + row * (C + 1) + q4 * 4;
+                dst[0] = __float_as_uint(v.x);
+                dst[1] = __float_as_uint(v.y);
+                dst[2] = __float_as_uint(v.z);
+                dst[3] = __float_as_uint(v.w);
+            } else {
+                // one exponent byte per group, four groups per 32-bit word
+                tile[row * (C + 1) + q4] = ((__float_as_uint(v.x) >> 23) & 0xffu) | (((__float_as_uint(v.y) >> 23) & 0xffu) << 8) |
+                    (((__float_as_uint(v.z) >> 23) & 0xffu) << 16) | (((__float_as_uint(v.w) >> 23) & 0xffu) << 24);
             }
         }
+        __syncthreads();
+        // scatter: 16 lanes per column of the tile, four consecutive rows per lane
+        const bool wide = (d.N & 3) == 0;
+        for (int i = tid; i < C * (kScaleTile / 4); i += kScaleThreads) {
+            const int c = i / (kScaleTile / 4), r4 = (i % (kScaleTile / 4)) * 4;
+            if (r4 >= rows) continue;
+            uint32_t *dst = out + static_cast<size_t>(c) * d.N + s0 + r4;
+            const uint32_t v0 = tile[r4 * (C + 1) + c];
+            if (wide && r4 + 3 < rows) {
+                *reinterpret_cast<uint4 *>(dst) =
+                    make_uint4(v0, tile[(r4 + 1) * (C + 1) + c], tile[(r4 + 2) * (C + 1) + c], tile[(r4 + 3) * (C + 1) + c]);
+            } else {
+                dst[0] = v0;
+                for (int k = 1; k < 4 && r4 + k < rows; ++k)
+                    dst[k] = tile[(r4 + k) * (C + 1) + c];
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -478,10 +583,18 @@ ll_combine_kernel(CombineArgs a) {
     st16_nt(reinterpret_cast<uint4 *>(a.combined + (static_cast<size_t>(r) * d.T + t) * d.H) + col, out);
 }
 
+// Four values per thread through the same routine as the dispatch kernel, so that a NaN's
+// neighbours are covered too; the last thread pads with zeros.
 __global__ void
 f32_to_e4m3_kernel(const float *in, uint8_t *out, size_t n) {
-    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = static_cast<uint8_t>(f32_to_e4m3(in[i]));
+    const size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (i >= n) return;
+    float v[4];
+    for (int j = 0; j < 4; ++j)
+        v[j] = i + j < n ? in[i + j] : 0.f;
+    const uint32_t codes = e4m3_pack4(v[0], v[1], v[2], v[3]);
+    for (int j = 0; j < 4 && i + j < n; ++j)
+        out[i + j] = static_cast<uint8_t>(codes >> (8 * j));
 }
 
 int
@@ -556,11 +669,162 @@ nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes) {
 size_t
 nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, int num_topk, int hidden) {
     if (num_ranks <= 0 || num_experts <= 0 || num_tokens < 0 || num_topk <= 0 || hidden < 0) return 0;
-    const size_t counts = static_cast<size_t>(num_ranks) * num_experts * sizeof(int);
-    const size_t rows = static_cast<size_t>(num_ranks) * num_tokens * num_topk * sizeof(int);
+    const size_t groups = static_cast<size_t>(num_ranks) * ((num_tokens + kGroupTokens - 1) / kGroupTokens);
+    const size_t flags = (groups * sizeof(int) + 255) / 256 * 256;
+    const size_t bits = static_cast<size_t>(num_experts) * groups * sizeof(unsigned long long);
     const size_t scales = static_cast<size_t>(num_ranks) * num_tokens * (hidden / 128) * sizeof(float);
-    return counts + 2 * rows + scales; // positions and final rows are separate arrays
+    return kWorkspaceHeader + flags + (bits + 255) / 256 * 256 + scales;
 }
+
+} // extern "C"
+
+namespace {
+
+struct LlDispatchCall {
+    void *packed_recv_x;
+    void *packed_recv_x_scales;
+    int *packed_recv_src_info;
+    int64_t *packed_recv_layout_range;
+    int *packed_recv_count;
+    const int *mask_buffer;
+    int *stats;
+    const void *x;
+    int32_t *topk_idx; // input, or output when logits are given
+    const float *logits; // null: indices come from the caller
+    float *topk_weights; // output, with logits only
+    const int *num_tokens_per_rank;
+    int num_tokens, hidden, max_tokens, num_topk, num_ranks, num_experts;
+    int use_fp8, round_scale, use_ue8m0;
+    int *row_map;
+    void *workspace;
+    size_t workspace_bytes;
+    void *stream;
+};
+
+template<bool ROUTE>
+void
+launch_bits(int per_lane, dim3 grid, size_t lds, hipStream_t s, const BitsArgs &a) {
+    constexpr int threads = ROUTE ? kRouteThreads : kBitsThreads;
+    if (!ROUTE || per_lane <= 1)
+        hipLaunchKernelGGL((ll_bits_kernel<ROUTE, 1>), grid, dim3(threads), lds, s, a);
+    else if (per_lane <= 2)
+        hipLaunchKernelGGL((ll_bits_kernel<ROUTE, 2>), grid, dim3(threads), lds, s, a);
+    else if (per_lane <= 4)
+        hipLaunchKernelGGL((ll_bits_kernel<ROUTE, 4>), grid, dim3(threads), lds, s, a);
+    else if (per_lane <= 8)
+        hipLaunchKernelGGL((ll_bits_kernel<ROUTE, 8>), grid, dim3(threads), lds, s, a);
+    else
+        hipLaunchKernelGGL((ll_bits_kernel<ROUTE, 16>), grid, dim3(threads), lds, s, a);
+}
+
+int
+ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
+    auto bad = [&](int code, const std::string &why) { return nixl_amd_fail(code, std::string(who) + ": " + why); };
+    LlDims d;
+    const int rc = check_dims(who, c.num_tokens, c.hidden, c.max_tokens, c.num_topk, c.num_ranks, c.num_experts, d);
+    if (rc) return rc;
+    if (!c.packed_recv_x || !c.packed_recv_src_info || !c.packed_recv_layout_range || !c.packed_recv_count || !c.workspace ||
+        (d.T > 0 && (!c.x || !c.topk_idx || (c.logits && !c.topk_weights)))) // a call without tokens reads no input
+        return bad(NIXL_AMD_ERR_INVALID, "null pointer argument");
+    if (c.use_fp8 && c.hidden % 512 != 0) // same restriction as csrc/nixl_ep.cpp:1091
+        return bad(NIXL_AMD_ERR_INVALID, "fp8 needs hidden % 512 == 0");
+    if (c.use_fp8 && !c.packed_recv_x_scales) return bad(NIXL_AMD_ERR_INVALID, "scales pointer is null");
+    if (c.use_ue8m0 && !(c.use_fp8 && c.round_scale)) // kernels/nixl_ep_ll.cu:428-430
+        return bad(NIXL_AMD_ERR_INVALID, "UE8M0 scales need use_fp8 and round_scale");
+    if (c.workspace_bytes < nixl_amd_ep_ll_workspace_bytes(d.R, d.E, d.T, d.K, d.H))
+        return bad(NIXL_AMD_ERR_INVALID, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(c.workspace) % 16 != 0) return bad(NIXL_AMD_ERR_INVALID, "workspace must be 16-byte aligned");
+    if (c.use_fp8 && reinterpret_cast<uintptr_t>(c.packed_recv_x_scales) % 16 != 0)
+        return bad(NIXL_AMD_ERR_INVALID, "packed_recv_x_scales must be 16-byte aligned");
+    if (static_cast<long long>(d.E) * d.N >= (1ll << 31))
+        return bad(NIXL_AMD_ERR_TOO_LARGE, "num_experts * num_ranks * max tokens must be below 2^31");
+    if (static_cast<size_t>(d.E) * sizeof(unsigned long long) > 48 * 1024) return bad(NIXL_AMD_ERR_TOO_LARGE, "more than 6144 experts");
+    if (static_cast<size_t>(d.R) * sizeof(int) > 32 * 1024) return bad(NIXL_AMD_ERR_TOO_LARGE, "more than 8192 ranks");
+    if (c.logits && (d.E > kRouterMaxPerLane * kWaveSize || d.K > d.E))
+        return bad(NIXL_AMD_ERR_INVALID, "routing needs num_experts <= 1024 and num_topk <= num_experts");
+
+    hipStream_t s = static_cast<hipStream_t>(c.stream);
+    const int Wr = (d.T + kGroupTokens - 1) / kGroupTokens;
+    const size_t groups = static_cast<size_t>(d.R) * Wr;
+    auto *base = static_cast<uint8_t *>(c.workspace);
+    int *status = reinterpret_cast<int *>(base);
+    int *group_status = reinterpret_cast<int *>(base + kWorkspaceHeader);
+    const size_t off_bits = kWorkspaceHeader + (groups * sizeof(int) + 255) / 256 * 256;
+    auto *bits = reinterpret_cast<unsigned long long *>(base + off_bits);
+    auto *token_scales =
+        reinterpret_cast<float *>(base + off_bits + (static_cast<size_t>(d.E) * groups * sizeof(unsigned long long) + 255) / 256 * 256);
+
+    if (groups > 0) {
+        BitsArgs b{};
+        b.bits = bits;
+        b.group_status = group_status;
+        b.topk_idx = c.topk_idx;
+        b.topk_weights = c.topk_weights;
+        b.logits = c.logits;
+        b.num_tokens_per_rank = c.num_tokens_per_rank;
+        b.mask = c.mask_buffer;
+        b.d = d;
+        b.Wr = Wr;
+        const size_t lds = static_cast<size_t>(d.E) * sizeof(unsigned long long);
+        if (c.logits)
+            launch_bits<true>((d.E + kWaveSize - 1) / kWaveSize, dim3(static_cast<unsigned>(groups)), lds, s, b);
+        else
+            launch_bits<false>(1, dim3(static_cast<unsigned>(groups)), lds, s, b);
+        HIP_TRY(hipGetLastError());
+    }
+
+    DispatchArgs a{};
+    a.recv_x = static_cast<uint8_t *>(c.packed_recv_x);
+    a.token_scales = token_scales;
+    a.src_info = c.packed_recv_src_info;
+    a.layout_range = reinterpret_cast<long long *>(c.packed_recv_layout_range);
+    a.recv_count = c.packed_recv_count;
+    a.stats = c.stats;
+    a.x = static_cast<const uint16_t *>(c.x);
+    a.topk_idx = c.topk_idx;
+    a.num_tokens_per_rank = c.num_tokens_per_rank;
+    a.bits = bits;
+    a.group_status = group_status;
+    a.status = status;
+    a.rows_out = c.row_map;
+    a.d = d;
+    a.Wr = Wr;
+    a.round_scale = c.round_scale;
+    if (d.T == 0) {
+        hipLaunchKernelGGL(ll_meta_kernel, dim3((d.E + 3) / 4), dim3(256), 0, s, a);
+        HIP_TRY(hipGetLastError());
+        return NIXL_AMD_OK;
+    }
+    const int wg = std::min(round_up_wave(d.H / 16), g_dispatch_lanes);
+    a.parts = (d.H / 16 + wg - 1) / wg;
+    const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
+    const dim3 block(wg);
+    if (c.use_fp8)
+        hipLaunchKernelGGL(ll_dispatch_kernel<true>, grid, block, 0, s, a);
+    else
+        hipLaunchKernelGGL(ll_dispatch_kernel<false>, grid, block, 0, s, a);
+    HIP_TRY(hipGetLastError());
+
+    if (c.use_fp8) {
+        ScalesArgs sa{};
+        sa.recv_scales = c.packed_recv_x_scales;
+        sa.token_scales = token_scales;
+        sa.src_info = c.packed_recv_src_info;
+        sa.layout_range = reinterpret_cast<const long long *>(c.packed_recv_layout_range);
+        sa.d = d;
+        sa.use_ue8m0 = c.use_ue8m0;
+        sa.parts = kScaleParts;
+        const int C = c.use_ue8m0 ? d.H / 512 : d.H / 128;
+        const size_t lds = (static_cast<size_t>(d.R) + static_cast<size_t>(kScaleTile) * (C + 1) + kScaleTile) * sizeof(int);
+        hipLaunchKernelGGL(ll_scales_kernel, dim3(static_cast<unsigned>(d.E) * sa.parts), dim3(kScaleThreads), lds, s, sa);
+        HIP_TRY(hipGetLastError());
+    }
+    return NIXL_AMD_OK;
+}
+
+} // namespace
+
+extern "C" {
 
 int
 nixl_amd_ep_ll_dispatch(void *packed_recv_x,
@@ -586,81 +850,55 @@ nixl_amd_ep_ll_dispatch(void *packed_recv_x,
                         void *workspace,
                         size_t workspace_bytes,
                         void *stream) {
-    LlDims d;
-    const int rc = check_dims("ll_dispatch", num_tokens, hidden, num_max_dispatch_tokens_per_rank, num_topk, num_ranks,
-                              num_experts, d);
-    if (rc) return rc;
-    if (!packed_recv_x || !packed_recv_src_info || !packed_recv_layout_range || !packed_recv_count || !x || !topk_idx ||
-        !workspace)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: null pointer argument");
-    if (use_fp8 && hidden % 512 != 0) // same restriction as csrc/nixl_ep.cpp:1091
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: fp8 needs hidden % 512 == 0");
-    if (use_fp8 && !packed_recv_x_scales) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: scales pointer is null");
-    if (use_ue8m0 && !(use_fp8 && round_scale)) // kernels/nixl_ep_ll.cu:428-430
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: UE8M0 scales need use_fp8 and round_scale");
-    if (workspace_bytes < nixl_amd_ep_ll_workspace_bytes(num_ranks, num_experts, num_tokens, num_topk, hidden))
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: workspace too small");
-    if (reinterpret_cast<uintptr_t>(workspace) % 4 != 0)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch: workspace must be 4-byte aligned");
-    if (static_cast<long long>(d.E) * d.N >= (1ll << 31))
-        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: num_experts * num_ranks * max tokens must be below 2^31");
-    if (static_cast<size_t>(d.E) * sizeof(int) > 48 * 1024 || static_cast<size_t>(d.R) * sizeof(int) > 48 * 1024)
-        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: too many experts or ranks");
+    const LlDispatchCall c{packed_recv_x, packed_recv_x_scales, packed_recv_src_info, packed_recv_layout_range,
+                           packed_recv_count, mask_buffer, cumulative_local_expert_recv_stats, x,
+                           const_cast<int32_t *>(topk_idx), nullptr, nullptr, num_tokens_per_rank, num_tokens, hidden,
+                           num_max_dispatch_tokens_per_rank, num_topk, num_ranks, num_experts, use_fp8, round_scale,
+                           use_ue8m0, row_map, workspace, workspace_bytes, stream};
+    return ll_dispatch_impl("ll_dispatch", c);
+}
 
+int
+nixl_amd_ep_ll_route_dispatch(void *packed_recv_x,
+                              void *packed_recv_x_scales,
+                              int *packed_recv_src_info,
+                              int64_t *packed_recv_layout_range,
+                              int *packed_recv_count,
+                              const int *mask_buffer,
+                              int *cumulative_local_expert_recv_stats,
+                              const void *x,
+                              const float *logits,
+                              int32_t *topk_idx,
+                              float *topk_weights,
+                              const int *num_tokens_per_rank,
+                              int num_tokens,
+                              int hidden,
+                              int num_max_dispatch_tokens_per_rank,
+                              int num_topk,
+                              int num_ranks,
+                              int num_experts,
+                              int use_fp8,
+                              int round_scale,
+                              int use_ue8m0,
+                              int *row_map,
+                              void *workspace,
+                              size_t workspace_bytes,
+                              void *stream) {
+    if (!logits) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_route_dispatch: logits is null");
+    const LlDispatchCall c{packed_recv_x, packed_recv_x_scales, packed_recv_src_info, packed_recv_layout_range,
+                           packed_recv_count, mask_buffer, cumulative_local_expert_recv_stats, x, topk_idx, logits,
+                           topk_weights, num_tokens_per_rank, num_tokens, hidden, num_max_dispatch_tokens_per_rank,
+                           num_topk, num_ranks, num_experts, use_fp8, round_scale, use_ue8m0, row_map, workspace,
+                           workspace_bytes, stream};
+    return ll_dispatch_impl("ll_route_dispatch", c);
+}
+
+int
+nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status) {
+    if (!workspace || !status) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_dispatch_status: null pointer argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t n_sel = static_cast<size_t>(d.R) * d.T * d.K;
-    int *send_count = static_cast<int *>(workspace);
-    int *positions = send_count + static_cast<size_t>(d.R) * d.E;
-    int *rows_ws = positions + n_sel;
-    float *token_scales = reinterpret_cast<float *>(rows_ws + n_sel);
-    int *rows = row_map ? row_map : rows_ws;
-
-    const int W = (d.T + 63) / 64 > 0 ? (d.T + 63) / 64 : 1;
-    int per_pass = kLayoutLdsBytes / (W * 8);
-    if (per_pass < 1) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "ll_dispatch: too many tokens per rank for the layout pass");
-    if (per_pass > d.E) per_pass = d.E;
-    hipLaunchKernelGGL(ll_layout_kernel, dim3(d.R), dim3(kLayoutThreads), static_cast<size_t>(per_pass) * W * 8, s, topk_idx,
-                       num_tokens_per_rank, mask_buffer, send_count, positions, d, per_pass);
-    HIP_TRY(hipGetLastError());
-
-    if (d.T > 0) {
-        DispatchArgs a{};
-        a.recv_x = static_cast<uint8_t *>(packed_recv_x);
-        a.src_info = packed_recv_src_info;
-        a.token_scales = token_scales;
-        a.x = static_cast<const uint16_t *>(x);
-        a.topk_idx = topk_idx;
-        a.num_tokens_per_rank = num_tokens_per_rank;
-        a.send_count = send_count;
-        a.rows = positions;
-        a.rows_out = rows;
-        a.d = d;
-        a.round_scale = round_scale;
-        const int wg = std::min(round_up_wave(d.H / 16), g_dispatch_lanes);
-        a.parts = (d.H / 16 + wg - 1) / wg;
-        const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
-        const dim3 block(wg);
-        if (use_fp8)
-            hipLaunchKernelGGL(ll_dispatch_kernel<true>, grid, block, 0, s, a);
-        else
-            hipLaunchKernelGGL(ll_dispatch_kernel<false>, grid, block, 0, s, a);
-        HIP_TRY(hipGetLastError());
-    }
-
-    ScalesArgs sa{};
-    sa.recv_scales = use_fp8 ? packed_recv_x_scales : nullptr;
-    sa.token_scales = token_scales;
-    sa.src_info = packed_recv_src_info;
-    sa.send_count = send_count;
-    sa.layout_range = reinterpret_cast<long long *>(packed_recv_layout_range);
-    sa.recv_count = packed_recv_count;
-    sa.stats = cumulative_local_expert_recv_stats;
-    sa.d = d;
-    sa.use_ue8m0 = use_ue8m0;
-    sa.parts = kScaleParts;
-    hipLaunchKernelGGL(ll_scales_kernel, dim3(d.E * sa.parts), dim3(kScaleThreads),
-                       static_cast<size_t>(d.R) * sizeof(int), s, sa);
-    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(status, workspace, sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
     return NIXL_AMD_OK;
 }
 
@@ -696,7 +934,7 @@ nixl_amd_ep_ll_dispatch_static(void *packed_recv_x,
     const int rc = static_scratch(&ws);
     if (rc) return rc;
     // Every word of the workspace that a kernel reads is written earlier in the same call
-    // (counts and positions by the layout kernel, rows and scales by the dispatch kernel), so
+    // (selection bits and group flags by the first kernel, the status word by the second), so
     // what the previous call left behind needs no clearing.
     return nixl_amd_ep_ll_dispatch(packed_recv_x, packed_recv_x_scales, packed_recv_src_info, packed_recv_layout_range,
                                    packed_recv_count, mask_buffer, cumulative_local_expert_recv_stats, x, topk_idx,
@@ -757,7 +995,7 @@ nixl_amd_ep_f32_to_e4m3(const float *in, uint8_t *out, size_t n, void *stream) {
     if ((!in || !out) && n) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "f32_to_e4m3: null pointer argument");
     if (n == 0) return NIXL_AMD_OK;
     if (n > (1ull << 38)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "f32_to_e4m3: too many elements");
-    hipLaunchKernelGGL(f32_to_e4m3_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(f32_to_e4m3_kernel, dim3(static_cast<unsigned>((n + 1023) / 1024)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), in, out, n);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;

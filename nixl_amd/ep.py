@@ -278,7 +278,7 @@ class Buffer:
     def low_latency_dispatch(self, x, topk_idx, num_max_dispatch_tokens_per_rank, num_experts=None,
                              cumulative_local_expert_recv_stats=None, dispatch_wait_recv_cost_stats=None,
                              use_fp8=True, round_scale=False, use_ue8m0=False, async_finish=False,
-                             return_recv_hook=False, num_tokens_per_rank=None):
+                             return_recv_hook=False, num_tokens_per_rank=None, check_duplicates=False):
         """Reference: buffer.py:329-437, csrc/nixl_ep.cpp:1030-1143.
 
         x [R, T, H] bf16, topk_idx [R, T, K] int32 (-1 = no selection).  Returns
@@ -288,21 +288,41 @@ class Buffer:
         worlds: rank r only owns the first num_tokens_per_rank[r] rows of x[r].
         dispatch_wait_recv_cost_stats (cycles spent waiting for each source rank's data,
         nixl_ep_ll.cu:349-350) is left as it is: nothing here waits for another rank.
+        `check_duplicates` waits for the kernels and raises if a token named an expert twice
+        (the reference delivers such a token twice, nixl_ep_ll.cu:186-190; here it arrives once).
         """
+        if topk_idx.dim() != 3 or not topk_idx.is_contiguous() or topk_idx.dtype != topk_idx_t:
+            raise EPError("topk_idx must be a contiguous [R, T, K] int32 tensor")
+        return self._ll_dispatch(x, topk_idx, None, topk_idx.shape[2], num_max_dispatch_tokens_per_rank, num_experts,
+                                 cumulative_local_expert_recv_stats, use_fp8, round_scale, use_ue8m0, async_finish,
+                                 return_recv_hook, num_tokens_per_rank, check_duplicates)[2:]
+
+    def route_dispatch(self, x, logits, num_topk, num_max_dispatch_tokens_per_rank,
+                       cumulative_local_expert_recv_stats=None, use_fp8=True, round_scale=False, use_ue8m0=False,
+                       async_finish=False, return_recv_hook=False, num_tokens_per_rank=None):
+        """Routing and dispatch in one call (no reference counterpart: its callers bring
+        their own top-k).  logits [R, T, E] float32.  Returns (topk_idx, topk_weights) followed
+        by what low_latency_dispatch returns; the selection is that of route()."""
+        if logits.dim() != 3 or not logits.is_contiguous() or logits.dtype != torch.float32:
+            raise EPError("logits must be a contiguous [R, T, E] float32 tensor")
+        return self._ll_dispatch(x, None, logits, num_topk, num_max_dispatch_tokens_per_rank, logits.shape[2],
+                                 cumulative_local_expert_recv_stats, use_fp8, round_scale, use_ue8m0, async_finish,
+                                 return_recv_hook, num_tokens_per_rank, False)
+
+    def _ll_dispatch(self, x, topk_idx, logits, K, num_max_dispatch_tokens_per_rank, num_experts, stats, use_fp8,
+                     round_scale, use_ue8m0, async_finish, return_recv_hook, num_tokens_per_rank, check_duplicates):
         if not self.low_latency_mode:
             raise EPError("dispatch() requires low-latency mode (low_latency_mode=True)")
         if x.dim() != 3 or not x.is_contiguous() or x.dtype != torch.bfloat16:
             raise EPError("x must be a contiguous [R, T, H] bfloat16 tensor")
-        if topk_idx.dim() != 3 or not topk_idx.is_contiguous() or topk_idx.dtype != topk_idx_t:
-            raise EPError("topk_idx must be a contiguous [R, T, K] int32 tensor")
         R, T, H = x.shape
-        if R != self.num_ranks or topk_idx.shape[0] != R or topk_idx.shape[1] != T:
-            raise EPError("x and topk_idx must agree on ranks and tokens")
+        sel = topk_idx if logits is None else logits
+        if R != self.num_ranks or sel.shape[0] != R or sel.shape[1] != T:
+            raise EPError("x and the selection must agree on ranks and tokens")
         if T > num_max_dispatch_tokens_per_rank:
             raise EPError("more tokens than num_max_dispatch_tokens_per_rank")
         if num_experts is None:
             raise EPError("num_experts is required")
-        K = topk_idx.shape[2]
         El, N = num_experts // R, R * num_max_dispatch_tokens_per_rank
         dev = x.device
         packed_recv_x = torch.empty((R, El, N, H), dtype=torch.float8_e4m3fn if use_fp8 else torch.bfloat16, device=dev)
@@ -318,12 +338,23 @@ class Buffer:
         row_map = torch.empty((R, T, K), dtype=torch.int32, device=dev)
         ws_bytes = self._k.nixl_amd_ep_ll_workspace_bytes(R, num_experts, T, K, H)
         ws = self._get_workspace(ws_bytes)
-        rc = self._k.nixl_amd_ep_ll_dispatch(
-            _ptr(packed_recv_x), _ptr(scales), _ptr(packed_recv_src_info), _ptr(packed_recv_layout_range),
-            _ptr(packed_recv_count), self._mask_ptr(), _ptr(cumulative_local_expert_recv_stats), _ptr(x),
-            _ptr(topk_idx), _ptr(num_tokens_per_rank), T, H, num_max_dispatch_tokens_per_rank, K, R, num_experts,
-            int(use_fp8), int(round_scale), int(use_ue8m0), _ptr(row_map), _ptr(ws), ws.numel(), _stream())
+        head = (_ptr(packed_recv_x), _ptr(scales), _ptr(packed_recv_src_info), _ptr(packed_recv_layout_range),
+                _ptr(packed_recv_count), self._mask_ptr(), _ptr(stats), _ptr(x))
+        tail = (_ptr(num_tokens_per_rank), T, H, num_max_dispatch_tokens_per_rank, K, R, num_experts, int(use_fp8),
+                int(round_scale), int(use_ue8m0), _ptr(row_map), _ptr(ws), ws.numel(), _stream())
+        topk_weights = None
+        if logits is None:
+            rc = self._k.nixl_amd_ep_ll_dispatch(*head, _ptr(topk_idx), *tail)
+        else:
+            topk_idx = torch.empty((R, T, K), dtype=topk_idx_t, device=dev)
+            topk_weights = torch.empty((R, T, K), dtype=torch.float32, device=dev)
+            rc = self._k.nixl_amd_ep_ll_route_dispatch(*head, _ptr(logits), _ptr(topk_idx), _ptr(topk_weights), *tail)
         _check(rc, "low_latency_dispatch")
+        if check_duplicates:
+            status = ctypes.c_int(0)
+            _check(self._k.nixl_amd_ep_ll_dispatch_status(_ptr(ws), _stream(), ctypes.byref(status)), "dispatch status")
+            if status.value:
+                raise EPError("a token's top-k names the same expert twice")
         event = None
         if async_finish:
             event = torch.cuda.Event()
@@ -332,7 +363,7 @@ class Buffer:
         handle.row_map = row_map
         recv = (packed_recv_x, scales.transpose(2, 3)) if use_fp8 else packed_recv_x
         hook = (lambda: None) if return_recv_hook else None
-        return recv, packed_recv_count, handle, EventOverlap(event), hook
+        return topk_idx, topk_weights, recv, packed_recv_count, handle, EventOverlap(event), hook
 
     def dispatch(self, *args, **kwargs):
         return self.low_latency_dispatch(*args, **kwargs)

@@ -75,10 +75,15 @@ def run_low_latency(dev, warmup=20, iters=50):
 
     t_both = _timed(both, flush, warmup, iters)
 
-    def routed():  # the router in front as well: logits -> top-k -> dispatch -> combine
-        state["routed_topk"], state["routed_w"] = buf.route(logits, K)
-        state["out"] = buf.dispatch(x, state["routed_topk"], M, E, use_fp8=True)
-        buf.combine(y, state["routed_topk"], state["routed_w"], state["out"][2])
+    def route_dispatch():  # logits in: routing done by the kernel that prepares the dispatch
+        state["routed"] = buf.route_dispatch(x, logits, K, M, use_fp8=True)
+
+    t_route_dispatch = _timed(route_dispatch, flush, warmup, iters)
+
+    def routed():  # logits -> top-k -> dispatch -> combine under one event pair
+        route_dispatch()
+        idx, wts, _, _, handle_r, _, _ = state["routed"]
+        buf.combine(y, idx, wts, handle_r)
 
     t_routed = _timed(routed, flush, warmup, iters)
 
@@ -94,6 +99,8 @@ def run_low_latency(dev, warmup=20, iters=50):
         "dispatch_plus_combine_us": round(both_us, 2),
         "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
         "dispatch_then_combine_one_event_pair": {**t_both, **_rate(dispatch_bytes + combine_bytes, t_both["avg_us"])},
+        "route_dispatch": {**t_route_dispatch, **_rate(dispatch_bytes + tokens * E * 4, t_route_dispatch["avg_us"]),
+                           "note": "dispatch from logits (top-k + softmax inside); adds 4.2 MB of logits and the written selection"},
         "route_dispatch_combine_one_event_pair": {
             **t_routed, **_rate(dispatch_bytes + combine_bytes + tokens * E * 4, t_routed["avg_us"]),
             "note": "router (logits -> top-k + softmax) included; its logits add 4.2 MB"},

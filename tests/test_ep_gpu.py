@@ -655,6 +655,72 @@ def test_router_matches_oracle(cuda):
         buf.route(torch.zeros((4, 2000), device=cuda), 2)
 
 
+@pytest.mark.parametrize("shape", [(4, 70, 512, 3, 16, 80), (2, 130, 1024, 8, 256, 130), (8, 5, 512, 4, 1024, 8)])
+@pytest.mark.parametrize("use_fp8", [True, False])
+def test_route_dispatch_equals_route_then_dispatch(cuda, shape, use_fp8):
+    """Routing folded into the dispatch call: the selection is the oracle router's, and every
+    dispatch output equals the oracle's dispatch of that selection."""
+    R, T, H, K, E, M = shape
+    rng = np.random.default_rng(R * 100 + T)
+    x = torch.from_numpy(rng.standard_normal((R, T, H)).astype(np.float32)).to(torch.bfloat16)
+    logits = rng.standard_normal((R, T, E)).astype(np.float32)
+    logits[0, 0, :] = 0.0  # all equal: ties go to the lower expert index
+    nt = np.full(R, T, np.int32)
+    nt[-1] = T // 2
+    buf = Buffer(R, device=cuda)
+    stats = torch.zeros((R, E // R), dtype=torch.int32, device=cuda)
+    idx, w, recv, cnt, handle, _, _ = buf.route_dispatch(
+        x.to(cuda), torch.from_numpy(logits).to(cuda), K, M, cumulative_local_expert_recv_stats=stats, use_fp8=use_fp8,
+        num_tokens_per_rank=torch.from_numpy(nt).to(cuda))
+    torch.cuda.synchronize()
+    oi, ow = eo.router(logits.reshape(R * T, E), K)
+    assert np.array_equal(idx.cpu().numpy().reshape(R * T, K), oi)
+    assert np.allclose(w.cpu().numpy().reshape(R * T, K), ow, rtol=2e-6, atol=0)
+    want = eo.ll_dispatch(bits16(x).reshape(R, T, H), oi.reshape(R, T, K), E, M, use_fp8, num_tokens=nt, fill=0)
+    assert np.array_equal(cnt.cpu().numpy(), want["recv_count"])
+    assert np.array_equal(stats.cpu().numpy(), want["recv_count"])
+    assert np.array_equal(handle[1].cpu().numpy(), want["layout_range"])
+    El, N = E // R, R * M
+    rx = (recv[0] if use_fp8 else recv).view(torch.uint8).cpu().numpy().reshape(R, El, N, -1)
+    wx = want["recv_x"].view(np.uint8).reshape(R, El, N, -1)
+    si, wsi = handle[0].cpu().numpy(), want["src_info"].reshape(R, El, N)
+    sc = recv[1].transpose(2, 3).contiguous().cpu().numpy() if use_fp8 else None  # back to [R][El][G][N]
+    for r in range(R):
+        for e in range(El):
+            n = int(want["recv_count"][r, e])
+            assert np.array_equal(rx[r, e, :n], wx[r, e, :n])
+            assert np.array_equal(si[r, e, :n], wsi[r, e, :n])
+            if use_fp8:
+                assert np.array_equal(sc[r, e, :, :n].view(np.uint32), want["scales"].reshape(R, El, H // 128, N)[r, e, :, :n].view(np.uint32))
+
+
+def test_ll_dispatch_reports_a_repeated_expert(cuda):
+    """The K entries of a token must differ; a repeat is reported through the status word
+    (and raised by Buffer.dispatch(check_duplicates=True)), a clean selection reports 0."""
+    R, T, H, K, E, M = 2, 70, 512, 4, 8, 70
+    x, topk, _ = make_world(3, R, T, H, K, E, drop=0.0)
+    buf = Buffer(R, device=cuda)
+    xd = x.to(cuda)
+    buf.dispatch(xd, torch.from_numpy(topk).to(cuda), M, E, check_duplicates=True)
+    bad = topk.copy()
+    bad[1, 66, 3] = bad[1, 66, 0]
+    with pytest.raises(EPError):
+        buf.dispatch(xd, torch.from_numpy(bad).to(cuda), M, E, check_duplicates=True)
+    bad[1, 66, 3] = -1  # "no selection" twice is not a repeat
+    bad[1, 66, 2] = -1
+    buf.dispatch(xd, torch.from_numpy(bad).to(cuda), M, E, check_duplicates=True)
+
+
+def test_ll_dispatch_without_tokens(cuda):
+    R, H, K, E, M = 4, 512, 2, 8, 4
+    x = torch.zeros((R, 0, H), dtype=torch.bfloat16)
+    topk = np.zeros((R, 0, K), np.int32)
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, True)
+    assert rc == 0, _lib.kernels_error()
+    assert not got["recv_count"].any() and not got["layout_range"].any()
+    assert (got["recv_x"] == 0x55).all()
+
+
 # ---- committed golden vectors (tests/golden, independent of the oracle) ---------------------------
 
 def _golden(name):
@@ -741,7 +807,8 @@ def test_golden_normal_mode_world(cuda):
     assert np.array_equal(comb_w.cpu().numpy(), g["combined_topk_weights"])
 
 
-@pytest.mark.parametrize("shape", [(64, 3, 512, 2, 128, 4), (2, 1, 8192, 16, 32, 1), (16, 64, 1024, 6, 48, 64), (1, 40, 512, 4, 8, 64)])
+@pytest.mark.parametrize("shape", [(64, 3, 512, 2, 128, 4), (2, 1, 8192, 16, 32, 1), (16, 64, 1024, 6, 48, 64), (1, 40, 512, 4, 8, 64),
+                                   (3, 300, 512, 5, 12, 320), (80, 65, 512, 2, 160, 65)])
 def test_ll_wide_and_narrow_worlds(cuda, shape):
     """Many ranks with few tokens, the largest hidden size and top-k, one rank alone:
     dispatch (fp8 and bf16) and combine against the oracle."""

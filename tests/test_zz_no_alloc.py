@@ -13,7 +13,7 @@ from nixl_amd import _lib
 
 pytestmark = pytest.mark.gpu
 
-STATIC_BYTES = 4 << 20  # NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES
+STATIC_BYTES = 2 << 20  # NIXL_AMD_EP_LL_STATIC_SCRATCH_BYTES
 
 
 def _world(seed, R, T, H, K, E):
