@@ -4,6 +4,7 @@
 #ifndef NIXL_AMD_LOG_H
 #define NIXL_AMD_LOG_H
 
+#include <cassert>
 #include <cstdlib>
 #include <cstring>
 #include <iostream>

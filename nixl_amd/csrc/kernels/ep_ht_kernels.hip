@@ -706,21 +706,26 @@ router_kernel(const float *__restrict__ logits, int32_t *__restrict__ topk_idx, 
         v[j] = e < E ? logits[static_cast<size_t>(token) * E + e] : 0.f;
         if (e >= E) taken |= 1u << j;
     }
-    float sel_v[16];
-    int sel_i[16];
+    float mine = 0.f, first = 0.f; // lane k keeps the k-th selected logit
+    int mine_i = 0;
+    for (int k = 0; k < K; ++k) {
+        float top;
+        int win;
+        router_round<PL>(v, taken, lane, top, win);
+        if (k == 0) first = top;
+        if (lane == k) {
+            mine = top;
+            mine_i = win;
+        }
+    }
+    // softmax over the K selected logits; every lane adds them up in selection order
+    const float ex = lane < K ? expf(mine - first) : 0.f;
+    float sum = 0.f;
     for (int k = 0; k < K; ++k)
-        router_round<PL>(v, taken, lane, sel_v[k], sel_i[k]);
-    if (lane == 0) {
-        const float top = sel_v[0];
-        float ex[16], sum = 0.f;
-        for (int k = 0; k < K; ++k) {
-            ex[k] = expf(sel_v[k] - top);
-            sum += ex[k];
-        }
-        for (int k = 0; k < K; ++k) {
-            topk_idx[static_cast<size_t>(token) * K + k] = sel_i[k];
-            topk_w[static_cast<size_t>(token) * K + k] = ex[k] / sum;
-        }
+        sum += __shfl(ex, k);
+    if (lane < K) {
+        topk_idx[static_cast<size_t>(token) * K + lane] = mine_i;
+        topk_w[static_cast<size_t>(token) * K + lane] = ex / sum;
     }
 }
 

@@ -42,7 +42,8 @@
 namespace {
 
 constexpr int kBitsThreads = 256; // index path: two (token, k) entries per thread at top-8
-constexpr int kRouteThreads = 1024; // routing path: 16 waves, four tokens each
+constexpr int kRouteThreads = 1024; // routing path: 16 waves, a token each
+constexpr int kRouteTokens = 16;
 constexpr int kGroupTokens = 64; // tokens per word of the selection bits
 constexpr int kMaxTopk = 16; // reference limit, kernels/nixl_ep_ll.cu:412,421
 constexpr int kRouterMaxPerLane = 16; // E <= 1024 when routing
@@ -79,17 +80,21 @@ struct BitsArgs {
     int Wr; // words (groups of 64 tokens) per rank
 };
 
-// grid = R * Wr workgroups; dynamic LDS: E words.
+// Index path: grid = R * Wr workgroups, one per word (64 tokens).  Routing path: grid =
+// R * Wr * 4 workgroups, one per quarter word (16 tokens, a wave each), so that the routing
+// runs as wide as a token-per-wave router; a quarter is written as its own 16-bit word.
+// Dynamic LDS: E words.
 template<bool ROUTE, int PL>
 __global__ void __launch_bounds__(ROUTE ? kRouteThreads : kBitsThreads)
 ll_bits_kernel(BitsArgs a) {
+    constexpr int kTokens = ROUTE ? kRouteTokens : kGroupTokens; // tokens of this workgroup
     extern __shared__ unsigned long long words[]; // [E]
     __shared__ int dup;
-    __shared__ int sel_i[ROUTE ? kGroupTokens : 1][kMaxTopk];
-    __shared__ float sel_v[ROUTE ? kGroupTokens : 1][kMaxTopk];
+    __shared__ int sel_i[ROUTE ? kTokens : 1][kMaxTopk];
     const LlDims d = a.d;
     const int tid = threadIdx.x, n_threads = blockDim.x;
-    const int r = blockIdx.x / a.Wr, t0 = (blockIdx.x % a.Wr) * kGroupTokens;
+    const int per_rank = a.Wr * (kGroupTokens / kTokens); // workgroups per rank
+    const int r = blockIdx.x / per_rank, t0 = (blockIdx.x % per_rank) * kTokens;
     const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
     for (int e = tid; e < d.E; e += n_threads)
         words[e] = 0ull;
@@ -97,8 +102,8 @@ ll_bits_kernel(BitsArgs a) {
 
     if constexpr (ROUTE) {
         // K rounds of a wave-wide argmax per token; lane l holds experts l, l + 64, ...
-        const int lane = tid & (kWaveSize - 1), wave = tid / kWaveSize, n_waves = n_threads / kWaveSize;
-        for (int j = wave; j < kGroupTokens && t0 + j < d.T; j += n_waves) {
+        const int lane = tid & (kWaveSize - 1), j = tid / kWaveSize;
+        if (t0 + j < d.T) {
             const float *row = a.logits + (static_cast<size_t>(r) * d.T + t0 + j) * d.E;
             float v[PL];
             unsigned taken = 0;
@@ -108,41 +113,35 @@ ll_bits_kernel(BitsArgs a) {
                 v[q] = e < d.E ? row[e] : 0.f;
                 if (e >= d.E) taken |= 1u << q;
             }
+            float mine = 0.f, first = 0.f; // lane k keeps the k-th selected logit
+            int mine_i = 0;
             for (int k = 0; k < d.K; ++k) {
                 float top;
                 int win;
                 router_round<PL>(v, taken, lane, top, win);
-                if (lane == 0) {
-                    sel_i[j][k] = win;
-                    sel_v[j][k] = top;
+                if (k == 0) first = top;
+                if (lane == k) {
+                    mine = top;
+                    mine_i = win;
                 }
             }
-        }
-        __syncthreads();
-        // softmax over the K selected logits, one thread per token, summed in selection order
-        if (tid < kGroupTokens && t0 + tid < d.T) {
-            const float top = sel_v[tid][0];
+            // softmax over the K selected logits, summed in selection order by lane 0
+            const float ex = lane < d.K ? expf(mine - first) : 0.f;
             float sum = 0.f;
-            for (int k = 0; k < d.K; ++k) {
-                const float ex = expf(sel_v[tid][k] - top);
-                sel_v[tid][k] = ex;
-                sum += ex;
-            }
             for (int k = 0; k < d.K; ++k)
-                sel_v[tid][k] = sel_v[tid][k] / sum;
+                sum += __shfl(ex, k);
+            if (lane < d.K) {
+                const size_t at = (static_cast<size_t>(r) * d.T + t0 + j) * d.K + lane;
+                a.topk_idx[at] = mine_i;
+                a.topk_weights[at] = ex / sum;
+                sel_i[j][lane] = mine_i;
+            }
         }
-        __syncthreads();
-        const size_t base = (static_cast<size_t>(r) * d.T + t0) * d.K;
-        for (int p = tid; p < kGroupTokens * d.K && t0 + p / d.K < d.T; p += n_threads) {
-            a.topk_idx[base + p] = sel_i[p / d.K][p % d.K];
-            a.topk_weights[base + p] = sel_v[p / d.K][p % d.K];
-        }
-    } else {
-        __syncthreads();
     }
+    __syncthreads();
 
     const int32_t *idx = a.topk_idx + (static_cast<size_t>(r) * d.T + t0) * d.K;
-    for (int p = tid; p < kGroupTokens * d.K; p += n_threads) {
+    for (int p = tid; p < kTokens * d.K; p += n_threads) {
         const int j = p / d.K;
         if (t0 + j >= nt) break;
         const int e = ROUTE ? sel_i[j][p % d.K] : idx[p];
@@ -152,9 +151,15 @@ ll_bits_kernel(BitsArgs a) {
     }
     __syncthreads();
     const size_t W = static_cast<size_t>(d.R) * a.Wr;
-    for (int e = tid; e < d.E; e += n_threads)
-        a.bits[e * W + blockIdx.x] = words[e];
-    if (tid == 0) a.group_status[blockIdx.x] = dup;
+    if constexpr (ROUTE) {
+        auto *quarters = reinterpret_cast<unsigned short *>(a.bits);
+        for (int e = tid; e < d.E; e += n_threads)
+            quarters[e * W * (kGroupTokens / kTokens) + blockIdx.x] = static_cast<unsigned short>(words[e]);
+    } else {
+        for (int e = tid; e < d.E; e += n_threads)
+            a.bits[e * W + blockIdx.x] = words[e];
+        if (tid == 0) a.group_status[blockIdx.x] = dup;
+    }
 }
 
 // ---- 2. cast + scatter ----------------------------------------------------------------------------
@@ -170,7 +175,8 @@ struct DispatchArgs {
     const int32_t *topk_idx;
     const int *num_tokens_per_rank;
     const unsigned long long *bits; // [E][R][Wr]
-    const int *group_status; // [R * Wr]
+    const int *group_status; // [n_flags]
+    int n_flags; // R * Wr, or 0 when the selection was made here (a top-k never repeats an expert)
     int *status; // workspace header
     int *rows_out; // [R][T][K] final row e * N + slot, -1 if none; may be null
     LlDims d;
@@ -213,7 +219,7 @@ expert_meta(const DispatchArgs &a, int e, int lane) {
 __device__ __forceinline__ void
 reduce_status(const DispatchArgs &a, int lane) {
     int any = 0;
-    for (int g = lane; g < a.d.R * a.Wr; g += kWaveSize)
+    for (int g = lane; g < a.n_flags; g += kWaveSize)
         any |= a.group_status[g];
     any = wave_sum(any);
     if (lane == 0) a.status[0] = any ? NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT : 0;
@@ -767,7 +773,8 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
         b.Wr = Wr;
         const size_t lds = static_cast<size_t>(d.E) * sizeof(unsigned long long);
         if (c.logits)
-            launch_bits<true>((d.E + kWaveSize - 1) / kWaveSize, dim3(static_cast<unsigned>(groups)), lds, s, b);
+            launch_bits<true>((d.E + kWaveSize - 1) / kWaveSize, dim3(static_cast<unsigned>(groups) * (kGroupTokens / kRouteTokens)), lds,
+                              s, b);
         else
             launch_bits<false>(1, dim3(static_cast<unsigned>(groups)), lds, s, b);
         HIP_TRY(hipGetLastError());
@@ -785,6 +792,7 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
     a.num_tokens_per_rank = c.num_tokens_per_rank;
     a.bits = bits;
     a.group_status = group_status;
+    a.n_flags = c.logits ? 0 : static_cast<int>(groups);
     a.status = status;
     a.rows_out = c.row_map;
     a.d = d;
