@@ -2,11 +2,13 @@
 """Benchmark of the hot path on one MI355X.
 
 Headline (``value``): paged-KV transfer throughput in decimal GB/s of payload, on the
-Llama-3-8B-shaped configuration: pool [32 layers][K,V][8192 blocks][32 KiB] of bf16 N(0,1)
-in HBM, 1024 blocks chosen without replacement, gathered into a contiguous staging buffer
-(65 536 descriptors) and then scattered to a seeded permutation of destination block ids in
-a second pool (65 536 descriptors).  One step = one gather request + one scatter request
-posted through the agent API (postXferReq -> poll getXferStatus) to the HIP backend plugin.
+Llama-3-8B-shaped configuration with the 16 KiB descriptors the metric names: pool
+[32 layers][K,V][8192 blocks][16 KiB] of bf16 N(0,1) in HBM, 1024 blocks chosen without
+replacement, gathered into a contiguous staging buffer (65 536 descriptors) and then
+scattered to a seeded permutation of destination block ids in a second pool (65 536
+descriptors).  One step = one gather request + one scatter request posted through the agent
+API (postXferReq -> poll getXferStatus) to the HIP backend plugin.  The 32 KiB point (16
+tokens per block) and the other descriptor order are reported beside it.
 The throughput formula is the reference benchmark's: bytes moved / wall time
 (benchmark/nixlbench/src/utils/utils.cpp:1357-1368).
 
@@ -29,11 +31,12 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 
-# HBM bytes per launch of the copy kernel from hardware counters (FETCH_SIZE and WRITE_SIZE,
-# one rocprofv3 --pmc run each, scaled by a plain 1 GiB element-wise kernel in the same run;
-# profiles/copy_uniform_kernel_kv_llama3_32KiB.txt).  Keyed by (blocks, pool blocks, block
-# bytes); counters cannot be read from inside this process, so other shapes report null.
-MEASURED_TRAFFIC_BYTES = {(1024, 8192, 32768): 4311669989}
+# HBM bytes per launch of the dominant kernel from hardware counters.  Counters cannot be read
+# from inside this process: these figures come from rocprofv3 --pmc runs of this same file
+# (FETCH_SIZE and WRITE_SIZE, one run each, scaled by a plain 1 GiB element-wise kernel in the
+# same run); the summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks,
+# descriptor bytes, order); a shape without a counter run reports null.
+MEASURED_TRAFFIC = {}
 
 
 def _kv_layout():
@@ -53,18 +56,30 @@ def _kv_descs(base, layers, pool_blocks, blk, block_ids, order):
     return (addr if order == "layer" else addr.T).reshape(-1)
 
 
+def _kv_indices(lk, pool_blocks, block_ids, order):
+    """Positions, in a prepared list that holds the whole pool in memory order
+    ([layer][K|V][block]), of the sub-blocks of `block_ids`, in the request's order."""
+    idx = np.arange(lk, dtype=np.int64)[:, None] * pool_blocks + np.asarray(block_ids, dtype=np.int64)[None, :]
+    return np.ascontiguousarray((idx if order == "layer" else idx.T).reshape(-1), dtype=np.int32)
+
+
 def _triples(addrs, blk):
     n = addrs.size
     return np.stack([addrs, np.full(n, blk, np.uint64), np.zeros(n, np.uint64)], 1)
 
 
-def run_kv(args):
+def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
+    """Gather + scatter of config 2's shape with `blk`-byte descriptors.  The pools and the
+    staging buffer are prepared ONCE as descriptor lists (prep_xfer_dlist); every request is
+    made from index vectors into those lists (make_prepped_xfer), the call pattern of the
+    reference's test/python/prep_xfer_perf.py:35-67.  Timed: (a) steady state, the same two
+    requests re-posted; (b) requests whose block list is new every time, prepare included."""
     import torch
     from nixl_amd import nixl_agent, nixl_agent_config
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     kv = _kv_layout()
-    layers, pool_blocks, n_sel, blk = kv.layers, args.pool_blocks, args.blocks, args.block_bytes
+    layers, pool_blocks, n_sel = kv.layers, args.pool_blocks, args.blocks
     lk = layers * kv.sub_blocks_per_layer
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
@@ -78,32 +93,68 @@ def run_kv(args):
     # bracket every kernel launch of the timed region.
     stream = torch.cuda.Stream(device=dev)
     agent = nixl_agent("bench", nixl_agent_config(backends=()))
-    agent.create_backend("HIP", {"stream": str(stream.cuda_stream)})
+    agent.create_backend("HIP", {"stream": str(stream.cuda_stream), **dict(kv.split("=", 1) for kv in args.backend_param)})
     agent.register_memory([src_pool, dst_pool, staging])
 
-    rng = np.random.default_rng(99)
-    sel = rng.choice(pool_blocks, n_sel, replace=False)
-    dst_ids = rng.permutation(pool_blocks)[:n_sel]
-    n_desc = n_sel * lk
-    src_addrs = _kv_descs(src_pool.data_ptr(), layers, pool_blocks, blk, sel, args.order)
-    dst_addrs = _kv_descs(dst_pool.data_ptr(), layers, pool_blocks, blk, dst_ids, args.order)
+    n_desc, n_pool = n_sel * lk, lk * pool_blocks
+    pool_offsets = np.arange(n_pool, dtype=np.uint64) * np.uint64(blk)
     stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
-
     t0 = time.perf_counter()
-    h_src = agent.prep_xfer_dlist("", _triples(src_addrs, blk), "VRAM")
+    h_src = agent.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+    h_dst = agent.prep_xfer_dlist("bench", _triples(np.uint64(dst_pool.data_ptr()) + pool_offsets, blk), "VRAM")
     h_stg_r = agent.prep_xfer_dlist("bench", _triples(stg_addrs, blk), "VRAM")
     h_stg_l = agent.prep_xfer_dlist("", _triples(stg_addrs, blk), "VRAM")
-    h_dst = agent.prep_xfer_dlist("bench", _triples(dst_addrs, blk), "VRAM")
-    idx = np.arange(n_desc)
-    gather = agent.make_prepped_xfer("WRITE", h_src, idx, h_stg_r, idx)
-    scatter = agent.make_prepped_xfer("WRITE", h_stg_l, idx, h_dst, idx)
-    prep_ms = (time.perf_counter() - t0) * 1e3
-    assert gather.desc_count() == (n_desc, n_desc * blk)
+    prep_dlist_ms = (time.perf_counter() - t0) * 1e3
+    stg_idx = np.arange(n_desc, dtype=np.int32)
 
+    def make(rng):
+        sel = rng.choice(pool_blocks, n_sel, replace=False)
+        dst_ids = rng.permutation(pool_blocks)[:n_sel]
+        src_idx, dst_idx = _kv_indices(lk, pool_blocks, sel, order), _kv_indices(lk, pool_blocks, dst_ids, order)
+        t = time.perf_counter()
+        gather = agent.make_prepped_xfer("WRITE", h_src, src_idx, h_stg_r, stg_idx)
+        scatter = agent.make_prepped_xfer("WRITE", h_stg_l, stg_idx, h_dst, dst_idx)
+        return gather, scatter, sel, dst_ids, (time.perf_counter() - t) * 1e3
+
+    def run(req):
+        state = agent.transfer(req)
+        while state == "PROC":
+            state = agent.check_xfer_state(req)
+        if state != "DONE":
+            raise RuntimeError(f"transfer ended in state {state}")
+
+    def check(sel, dst_ids):
+        sel_t, dst_t = torch.from_numpy(sel).to(dev), torch.from_numpy(dst_ids).to(dev)
+        if not torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16)):
+            raise RuntimeError("scattered blocks differ from the source blocks")
+
+    # (b) a new block list per request pair: make + post + wait, wall clock
+    rng = np.random.default_rng(99)
+    make_ms, fresh_ms, pairs = [], [], []
+    for i in range(max(fresh_requests, 1) + 1):
+        torch.cuda.synchronize()
+        w0 = time.perf_counter()
+        gather, scatter, sel, dst_ids, m = make(rng)
+        run(gather)
+        run(scatter)
+        w = (time.perf_counter() - w0) * 1e3
+        check(sel, dst_ids)
+        if i == 0:  # the first pair also pays one-off allocations: not counted, not kept
+            gather.release()
+            scatter.release()
+            continue
+        make_ms.append(m)
+        fresh_ms.append(w)
+        pairs.append((gather, scatter, sel, dst_ids))
+        n_g, bytes_g = gather.desc_count()
+        assert bytes_g == n_desc * blk and n_g <= n_desc  # neighbouring blocks may have been merged
+
+    # (a) steady state: the prepared pairs re-posted in turn.  Which blocks a pair names moves
+    # its time by several per cent (placement in DRAM), so the figure is the mean over the pairs.
     post_us, xfer_us = [], []  # wall clock of the post call and of post -> completion, as nixlbench splits them
 
-    def step(events=None):
-        for req in (gather, scatter):
+    def step(k, events=None):
+        for req in pairs[k % len(pairs)][:2]:
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
@@ -122,45 +173,55 @@ def run_kv(args):
                 raise RuntimeError(f"transfer ended in state {state}")
 
     torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
+    for k in range(warmup):
+        step(k)
     torch.cuda.synchronize()
     events = []
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(events)
+    for k in range(steps):
+        step(k, events)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-
-    # correctness of what was just timed (bit-exact)
-    sel_t = torch.from_numpy(sel).to(dev)
-    dst_t = torch.from_numpy(dst_ids).to(dev)
-    if not torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16)):
-        raise RuntimeError("scattered blocks differ from the source blocks")
+    check(*pairs[(steps - 1) % len(pairs)][2:])  # correctness of what was just timed (bit-exact)
 
     payload_per_step = 2 * n_desc * blk  # gather + scatter
     kernel_ms = [a.elapsed_time(b) for a, b in events]
     avg_launch_ms = float(np.mean(kernel_ms))
     algorithmic_bytes_per_launch = 2 * n_desc * blk  # every payload byte read once, written once
     achieved = algorithmic_bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC.get((n_sel, pool_blocks, blk, order))
     out = {
-        "value": payload_per_step * args.steps / wall / 1e9,
-        "ms_per_step": wall / args.steps * 1e3,
+        "value": payload_per_step * steps / wall / 1e9,
+        "ms_per_step": wall / steps * 1e3,
+        "steps": steps,
+        "warmup": warmup,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((n_sel, pool_blocks, blk)),
-                     "kernel": "copy_uniform_kernel<1,true,1>",
+                     "traffic": traffic["bytes"] if traffic else None,
+                     "traffic_source": traffic["source"] if traffic else None,
+                     "kernel": "copy_uniform_kernel<1,policy,1>",
                      "avg_launch_ms": round(avg_launch_ms, 4),
                      "min_launch_ms": round(float(np.min(kernel_ms)), 4),
                      "p99_launch_ms": round(float(np.percentile(kernel_ms, 99)), 4),
                      "gather_ms": round(float(np.mean(kernel_ms[0::2])), 4),
                      "scatter_ms": round(float(np.mean(kernel_ms[1::2])), 4),
                      "algorithmic_bytes_per_launch": algorithmic_bytes_per_launch},
-        "kv": {"descriptors_per_request": n_desc, "descriptor_bytes": blk, "prep_ms": round(prep_ms, 2),
+        "kv": {"descriptors_per_request": n_desc, "descriptor_bytes": blk, "descriptor_order": order,
+               "prepared_list_descriptors": {"pool": n_pool, "staging": n_desc},
+               "prep_dlist_ms_once": round(prep_dlist_ms, 2),
+               "make_request_pair_ms": round(float(np.mean(make_ms)), 3),
+               "value_including_prepare": round(payload_per_step / (float(np.mean(fresh_ms)) * 1e-3) / 1e9, 1),
+               "value_including_prepare_note": f"new block list per request pair: make_prepped_xfer x2 + post + wait, "
+                                               f"mean of {len(fresh_ms)} pairs, wall clock",
+               "block_sets_timed": len(pairs),
+               "scatter_ms_by_block_set": [round(float(np.mean(kernel_ms[2 * k + 1::2 * len(pairs)])), 4) for k in range(len(pairs))],
                "post_us": {"avg": round(float(np.mean(post_us)), 1), "p99": round(float(np.percentile(post_us, 99)), 1)},
                "xfer_us": {"avg": round(float(np.mean(xfer_us)), 1), "p99": round(float(np.percentile(xfer_us, 99)), 1)}},
     }
-    for h in (gather, scatter, h_src, h_stg_r, h_stg_l, h_dst):
+    for g, sc, _, _ in pairs:
+        g.release()
+        sc.release()
+    for h in (h_src, h_stg_r, h_stg_l, h_dst):
         h.release()
     agent.close()
     del src_pool, dst_pool, staging
@@ -192,9 +253,12 @@ def run_small_descriptors(steps=20, warmup=3):
     hr = agent.prep_xfer_dlist("small", np.stack([np.uint64(dst.data_ptr()) + do, lens, zeros], 1), "VRAM")
     idx = np.arange(n)
     req = agent.make_prepped_xfer("WRITE", hl, idx, hr, idx)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)  # twice the last-level cache
     torch.cuda.synchronize()
     times = []
     for i in range(warmup + steps):
+        with torch.cuda.stream(stream):
+            flush.fill_(i & 1)  # on the launch stream, so that it is over before the timed launch starts
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         state = agent.transfer(req)
@@ -211,12 +275,15 @@ def run_small_descriptors(steps=20, warmup=3):
     for h in (req, hl, hr):
         h.release()
     agent.close()
-    del src, dst
+    del src, dst, flush
     torch.cuda.empty_cache()
     gbps = 2 * payload / (us * 1e-6) / 1e9
+    traffic = MEASURED_TRAFFIC.get(("small", n))
     return {"descriptors": n, "payload_bytes": payload, "avg_launch_us": round(us, 1), "achieved_GBps": round(gbps, 1),
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "ns_per_descriptor": round(us * 1e3 / n, 3),
-            "kernel": "copy_piece_kernel<true,4>"}
+            "traffic": traffic["bytes"] if traffic else None, "traffic_source": traffic["source"] if traffic else None,
+            "cache_flush": "512 MB written on the launch stream before every timed launch",
+            "kernel": "copy_piece_kernel<policy,4,1>"}
 
 
 def run_calibration_copy():
@@ -231,35 +298,85 @@ def run_calibration_copy():
     torch.cuda.empty_cache()
 
 
-def run_ep_cpu_baseline(seconds=10.0, threads=1):
+def run_ep_cpu_baseline(seconds=10.0, threads=1, full=False):
     """Scalar CPU restatement of the low-latency kernels (the oracle) on `threads` host
-    threads, on a bounded sample: 4 virtual ranks x 128 tokens x 7168, 32 experts, top-8,
-    fp8."""
+    threads.  full=True: BASELINE config 4 at its own size (32 virtual ranks x 128 tokens x
+    7168, 256 experts, top-8, fp8), a few passes; otherwise a bounded sample of 1/8 of its
+    tokens and experts for `seconds`."""
     from oracle import ep_oracle as eo
-    R, T, H, K, E, M = 4, 128, 7168, 8, 32, 128
+    R, T, H, K, E, M = (32, 128, 7168, 8, 256, 128) if full else (4, 128, 7168, 8, 32, 128)
     rng = np.random.default_rng(4)
     x = eo.f32_to_bf16(rng.standard_normal((R, T, H)).astype(np.float32))
     logits = rng.standard_normal((R * T, E)).astype(np.float32)
     topk, w = eo.router(logits, K)
     topk, w = topk.reshape(R, T, K), w.reshape(R, T, K)
+    y = np.zeros((R, E // R, R * M, H), np.uint16)  # expert outputs; only the received rows are ever touched
     t0 = time.perf_counter()
     n = 0
     d_us, c_us = [], []
-    while time.perf_counter() - t0 < seconds or n < 2:
+    while (n < 3) if full else (time.perf_counter() - t0 < seconds or n < 2):
         a = time.perf_counter()
-        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True, threads=threads)
+        o = eo.ll_dispatch(x, topk, E, M, use_fp8=True, threads=threads, fill=None)
         b = time.perf_counter()
-        y = np.zeros((R, E // R, R * M, H), np.uint16)
-        c = time.perf_counter()
         eo.ll_combine(y, topk, w, o["src_info"], o["layout_range"], E, M, threads=threads)
-        d = time.perf_counter()
-        d_us.append((b - a) * 1e6)
-        c_us.append((d - c) * 1e6)
+        c = time.perf_counter()
+        if n or not full:  # at full size the first pass also faults the output pages in
+            d_us.append((b - a) * 1e6)
+            c_us.append((c - b) * 1e6)
         n += 1
+        del o
     return {"dispatch_us": round(float(np.mean(d_us)), 1), "combine_us": round(float(np.mean(c_us)), 1),
             "cores": threads, "kind": "port", "host_cpus": os.cpu_count(),
-            "sample": f"{n} iterations, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8 "
-                      "(1/8 of the GPU workload's tokens)"}
+            "sample": f"{len(d_us)} passes, {R} virtual ranks x {T} tokens x {H}, {E} experts, top-{K}, fp8"
+                      + (" (config 4 at full size)" if full else " (1/8 of config 4's tokens and experts)")}
+
+
+def run_config1(seconds=6.0):
+    """BASELINE config 1 as stated: DRAM->DRAM loopback through one agent, 4096 descriptors of
+    16 KiB (64 MiB), payload uniform random bytes from a seed, destination block ids a seeded
+    permutation of 0..4095, WRITE, verified bit for bit.  Backend: the per-descriptor memcpy
+    plugin (the semantics of the reference's UCX loopback puts; libucp is not in this image).
+    Stages split as the reference benchmark splits them
+    (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:1583-1644): prepare = createXferReq,
+    post = postXferReq, transfer = post until completion."""
+    from nixl_amd import nixl_agent, nixl_agent_config
+    n, blk = 4096, 16384
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, n * blk, dtype=np.uint8)
+    dst = np.zeros(n * blk, dtype=np.uint8)
+    perm = rng.permutation(n).astype(np.uint64)
+    agent = nixl_agent("c1", nixl_agent_config(backends=()), plugin_dirs=[os.path.join(ROOT, "oracle", "_build")])
+    agent.create_backend("MEMCPY", {"threads": "1"})
+    for a in (src, dst):
+        agent.register_memory(np.array([[a.ctypes.data, a.nbytes, 0]], dtype=np.uint64), "DRAM")
+    lens, zeros = np.full(n, blk, np.uint64), np.zeros(n, np.uint64)
+    local = agent.get_xfer_descs(np.stack([np.uint64(src.ctypes.data) + np.arange(n, dtype=np.uint64) * np.uint64(blk), lens, zeros], 1), "DRAM")
+    remote = agent.get_xfer_descs(np.stack([np.uint64(dst.ctypes.data) + perm * np.uint64(blk), lens, zeros], 1), "DRAM")
+    prep, post, xfer = [], [], []
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end or len(xfer) < 3:
+        t0 = time.perf_counter()
+        req = agent.initialize_xfer("WRITE", local, remote, "c1")
+        t1 = time.perf_counter()
+        state = agent.transfer(req)
+        t2 = time.perf_counter()
+        while state == "PROC":
+            state = agent.check_xfer_state(req)
+        t3 = time.perf_counter()
+        if state != "DONE":
+            raise RuntimeError("config 1 transfer failed")
+        req.release()
+        prep.append((t1 - t0) * 1e6)
+        post.append((t2 - t1) * 1e6)
+        xfer.append((t3 - t1) * 1e6)
+    if not np.array_equal(dst.reshape(n, blk)[perm.astype(np.int64)], src.reshape(n, blk)):
+        raise RuntimeError("config 1: destination bytes differ")
+    agent.close()
+    stat = lambda v: {"avg": round(float(np.mean(v)), 1), "p99": round(float(np.percentile(v, 99)), 1)}
+    return {"value": round(n * blk / (float(np.mean(xfer)) * 1e-6) / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{len(xfer)} iterations of {n} descriptors x {blk} B (64 MiB), DRAM->DRAM loopback, permuted "
+                      "destinations, agent + per-descriptor memcpy backend, verified bit for bit",
+            "prepare_us": stat(prep), "post_us": stat(post), "transfer_us": stat(xfer)}
 
 
 def run_posix_analogue(seconds=4.0):
@@ -297,15 +414,15 @@ def run_posix_analogue(seconds=4.0):
                       "Python call overhead per descriptor included"}
 
 
-def run_cpu_baseline(seconds=12.0, threads=1):
+def run_cpu_baseline(seconds=12.0, threads=1, blk=16384):
     """Reference-shaped CPU path: one agent, loopback, DRAM->DRAM, one memcpy per descriptor
     (the semantics of the reference's UCX loopback puts, src/plugins/ucx/ucx_backend.cpp:
     1216-1262).  Same KV shape as the GPU workload with the pool cut to 512 blocks and 64
-    selected blocks (4096 descriptors of 32 KiB per request), single thread."""
+    selected blocks (4096 descriptors of `blk` bytes per request)."""
     from nixl_amd import nixl_agent, nixl_agent_config
     plugin_dir = os.path.join(ROOT, "oracle", "_build")
     kv = _kv_layout()
-    layers, pool_blocks, n_sel, blk = kv.layers, 512, 64, kv.bytes_per_sub_block
+    layers, pool_blocks, n_sel = kv.layers, 512, 64
     lk = layers * kv.sub_blocks_per_layer
     rng = np.random.default_rng(7)
     src_pool = rng.integers(0, 256, lk * pool_blocks * blk, dtype=np.uint8)
@@ -359,7 +476,13 @@ def main():
     ap.add_argument("--blocks", type=int, default=1024, help="KV blocks moved per request")
     ap.add_argument("--pool-blocks", type=int, default=8192)
     ap.add_argument("--block-bytes", type=int, default=0,
-                    help="bytes per (layer, K|V) sub-block; 0: what the model gives (32768)")
+                    help="bytes per (layer, K|V) descriptor; 0: 16384, the size the metric names, with the 32 KiB point "
+                         "(16 tokens per block) and the other descriptor order reported beside it")
+    ap.add_argument("--backend-param", action="append", default=[], metavar="KEY=VALUE",
+                    help="extra parameter for the HIP backend of the KV legs (units_per_lane, nontemporal, ...)")
+    ap.add_argument("--fresh-requests", type=int, default=4,
+                    help="request pairs with a new block list each, timed with their preparation")
+    ap.add_argument("--quick", action="store_true", help="headline point only, no other sizes or orders")
     ap.add_argument("--order", choices=("layer", "block"), default="layer",
                     help="descriptor list order: layer by layer, or block by block")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -378,11 +501,11 @@ def main():
     import __graft_entry__ as entry
     entry._ensure_built()
 
-    if not args.block_bytes:
-        args.block_bytes = _kv_layout().bytes_per_sub_block
     if args.calibrate_copy:
         run_calibration_copy()
-    kv = run_kv(args)
+    blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
+    kv = run_kv(args, blk, args.order, args.steps, args.warmup, fresh_requests=args.fresh_requests)
+    tokens_per_block = blk // (_kv_layout().bytes_per_sub_block // 16)
     line = {
         "metric": "KV xfer GB/s (% HBM peak) @16KB blocks; EP dispatch+combine µs @7168 top-8",
         "value": round(kv["value"], 1),
@@ -396,39 +519,43 @@ def main():
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": f"Llama-3-8B paged KV, VRAM->VRAM on one GPU: 32 layers x {{K,V}}, pool "
-                               f"{args.pool_blocks} blocks, {args.blocks} blocks gathered to staging then scattered, "
-                               f"{kv['kv']['descriptors_per_request']} descriptors x {args.block_bytes} B per request",
-                   "payload_bytes_per_step": 2 * kv["kv"]["descriptors_per_request"] * args.block_bytes,
+        "config": {"workload": f"Llama-3-8B paged KV, VRAM->VRAM on one GPU: 32 layers x {{K,V}}, {tokens_per_block} tokens per "
+                               f"block ({blk} B per layer/K-or-V block), pool {args.pool_blocks} blocks, {args.blocks} blocks "
+                               f"gathered to staging then scattered, {kv['kv']['descriptors_per_request']} descriptors x "
+                               f"{blk} B per request, listed {args.order} by {args.order}",
+                   "payload_bytes_per_step": 2 * kv["kv"]["descriptors_per_request"] * blk,
                    "pct_hbm_peak_payload_x2": round(2 * kv["value"] / HBM_PEAK_GBPS * 100, 1)},
         "roofline": kv["roofline"],
         "kv": kv["kv"],
     }
-    if args.block_bytes != 16384:
-        # the "@16KB" point the metric's name mentions: same shape with 16 KiB sub-blocks
-        half = argparse.Namespace(**vars(args))
-        half.block_bytes, half.steps, half.warmup = 16384, max(args.steps // 2, 1), max(args.warmup // 2, 1)
-        kv16 = run_kv(half)
-        line["kv"]["at_16KiB_descriptors"] = {
-            "value_GBps": round(kv16["value"], 1), "avg_launch_ms": kv16["roofline"]["avg_launch_ms"],
-            "achieved_GBps": kv16["roofline"]["achieved"], "frac": kv16["roofline"]["frac"],
-            "descriptors_per_request": kv16["kv"]["descriptors_per_request"]}
+    if not args.block_bytes and not args.quick:
+        # beside the headline: config 2 as BASELINE words it (16 tokens per block, 32 KiB), and
+        # both sizes with the descriptors listed the other way round; each with its own roofline
+        others = {}
+        other_order = "block" if args.order == "layer" else "layer"
+        for b, o in ((32768, args.order), (16384, other_order), (32768, other_order)):
+            r = run_kv(args, b, o, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2)
+            others[f"{b // 1024}KiB_{o}_order"] = {
+                "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
+                "make_request_pair_ms": r["kv"]["make_request_pair_ms"],
+                "value_including_prepare": r["kv"]["value_including_prepare"]}
+        line["kv"]["other_points"] = others
     if not args.no_small:
         line["kv"]["small_descriptor_stress"] = run_small_descriptors()
+    many = min(16, os.cpu_count() or 1)
     if not args.no_ep:
         from nixl_amd import ep_bench
         line["ep"] = ep_bench.run(args)
         if not args.no_cpu_baseline:
-            line["ep"]["cpu_baseline"] = run_ep_cpu_baseline()
-            many = min(16, os.cpu_count() or 1)
+            line["ep"]["cpu_baseline"] = run_ep_cpu_baseline(seconds=6.0)
             if many > 1:
-                line["ep"]["cpu_baseline"]["all_cores"] = run_ep_cpu_baseline(seconds=4.0, threads=many)
+                line["ep"]["cpu_baseline"]["all_cores_full_size"] = run_ep_cpu_baseline(threads=many, full=True)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = run_cpu_baseline()
+        line["cpu_baseline"] = run_cpu_baseline(blk=blk)
         # the same path with the descriptor list split over the box's CPU share, reported beside
-        many = min(16, os.cpu_count() or 1)
         if many > 1:
-            line["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=5.0, threads=many)
+            line["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=5.0, threads=many, blk=blk)
+        line["cpu_baseline"]["config1"] = run_config1()
         line["cpu_baseline"]["posix_path_analogue"] = run_posix_analogue()
         # the reference's own loopback needs libucp, which this image does not ship
         import ctypes.util

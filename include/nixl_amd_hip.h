@@ -55,6 +55,8 @@ typedef struct nixl_amd_copy_tuning {
     int max_workgroups; /* grid cap of the mixed and byte-path kernels; waves loop beyond it */
     int waves_per_workgroup; /* uniform-chunk kernel: 1, 2, 4, 8 or 16 */
     int xcd_swizzle; /* 1 = each accelerator die walks a contiguous slice of the chunk list, 2 = off */
+    int sort_scatter; /* a plan that scatters consecutive memory over irregular destinations has its records put
+                       * into ascending destination order inside windows of 1024 (on the device): 1 = on, 2 = off */
 } nixl_amd_copy_tuning_t;
 
 typedef struct nixl_amd_copy_plan nixl_amd_copy_plan_t;

@@ -37,7 +37,7 @@ class CopyDesc(Structure):
 
 class CopyTuning(Structure):
     _fields_ = [("units_per_lane", c_int), ("nontemporal", c_int), ("max_workgroups", c_int),
-                ("waves_per_workgroup", c_int), ("xcd_swizzle", c_int)]
+                ("waves_per_workgroup", c_int), ("xcd_swizzle", c_int), ("sort_scatter", c_int)]
 
 
 class CopyPlanInfo(Structure):

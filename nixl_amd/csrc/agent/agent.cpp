@@ -740,6 +740,7 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
     const size_t rguess = (rflat + rruns.descCount() - 1) / rruns.descCount();
 
     size_t total = 0;
+    const nixlStrideDesc *lrun_p = nullptr, *rrun_p = nullptr;
     for (size_t i = 0, step = 1; i < count; i += step) {
         if (local_indices[i] < 0 || static_cast<size_t>(local_indices[i]) >= lflat) {
             NIXL_ERROR_FUNC << "local index out of range at index " << i << " with value " << local_indices[i];
@@ -751,8 +752,10 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
         }
         const size_t li = static_cast<size_t>(local_indices[i]);
         const size_t ri = static_cast<size_t>(remote_indices[i]);
-        const nixlStrideDesc lrun = lruns.find(li, lguess);
-        const nixlStrideDesc rrun = rruns.find(ri, rguess);
+        // the run of the previous index usually holds this one as well
+        if (!lrun_p || li - lrun_p->start_idx >= lrun_p->count) lrun_p = &lruns.find(li, lguess);
+        if (!rrun_p || ri - rrun_p->start_idx >= rrun_p->count) rrun_p = &rruns.find(ri, rguess);
+        const nixlStrideDesc &lrun = *lrun_p, &rrun = *rrun_p;
         if (lrun.len != rrun.len) {
             NIXL_ERROR_FUNC << "length mismatch at index " << i << " with local index " << li
                             << " and remote index " << ri;

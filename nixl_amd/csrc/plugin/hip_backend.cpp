@@ -95,6 +95,7 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     const nixl_b_params_t *p = init_params->customParams;
     tuning_.units_per_lane = paramInt(p, "units_per_lane", 0);
     tuning_.nontemporal = paramInt(p, "nontemporal", 0);
+    tuning_.sort_scatter = paramInt(p, "sort_scatter", 0);
     tuning_.max_workgroups = paramInt(p, "max_workgroups", 0);
     tuning_.waves_per_workgroup = paramInt(p, "waves_per_workgroup", 0);
     tuning_.xcd_swizzle = paramInt(p, "xcd_swizzle", 0);
@@ -278,9 +279,11 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
         return NIXL_ERR_INVALID_PARAM;
     }
 
-    std::vector<nixl_amd_copy_desc_t> lowered(static_cast<size_t>(n));
+    const auto t_start = std::chrono::steady_clock::now();
+    const std::unique_ptr<nixl_amd_copy_desc_t[]> lowered(new nixl_amd_copy_desc_t[static_cast<size_t>(n)]); // not zero-filled
     int device = -1;
     size_t bytes = 0;
+    const nixlHipMD *prev_lmd = nullptr, *prev_rmd = nullptr;
     for (int i = 0; i < n; ++i) {
         const nixlMetaDesc &l = local[i];
         const nixlMetaDesc &r = remote[i];
@@ -296,7 +299,11 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
         }
         // The kernel runs on the device that owns the VRAM side(s); two VRAM regions on
         // different devices would need peer mappings, which this backend does not set up.
-        for (const nixlHipMD *md : {lmd, rmd}) {
+        // Checked once per pair of regions: consecutive descriptors mostly share theirs.
+        const bool same_regions = (lmd == prev_lmd && rmd == prev_rmd);
+        prev_lmd = lmd;
+        prev_rmd = rmd;
+        if (!same_regions) for (const nixlHipMD *md : {lmd, rmd}) {
             if (md->mem != VRAM_SEG) continue;
             if (device < 0) device = md->device;
             if (md->device != device) {
@@ -312,10 +319,11 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
     }
     if (device < 0) device = static_cast<const nixlHipMD *>(local[0].metadataP)->device;
 
+    const auto t_lowered = std::chrono::steady_clock::now();
     auto req = std::make_unique<nixlHipReqH>();
     req->device = device;
     req->bytes = bytes;
-    if (nixl_amd_copy_plan_create(lowered.data(), lowered.size(), device, &tuning_, &req->plan) !=
+    if (nixl_amd_copy_plan_create(lowered.get(), static_cast<size_t>(n), device, &tuning_, &req->plan) !=
         NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
         return NIXL_ERR_BACKEND;
@@ -326,6 +334,10 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
     req->stream = pickStream(device);
     if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
 
+    const auto t_done = std::chrono::steady_clock::now();
+    NIXL_DEBUG << "HIP backend: prepXfer of " << n << " descriptors: checks and lowering "
+               << std::chrono::duration<double, std::micro>(t_lowered - t_start).count() << " us, device plan and event "
+               << std::chrono::duration<double, std::micro>(t_done - t_lowered).count() << " us";
     handle = req.release();
     return NIXL_SUCCESS;
 }
@@ -749,6 +761,7 @@ nixl_plugin_init() {
                                 "0.1.0",
                                 {{"units_per_lane", "0"},
                                  {"nontemporal", "0"},
+                                 {"sort_scatter", "0"},
                                  {"max_workgroups", "0"},
                                  {"waves_per_workgroup", "0"},
                                  {"xcd_swizzle", "0"},

@@ -99,13 +99,15 @@ def cast_row_fp8(row_bf16, round_scale=False):
 def ll_dispatch(x, topk_idx, num_experts, max_tok, use_fp8=True, round_scale=False, use_ue8m0=False,
                 num_tokens=None, mask=None, threads=1, fill=0):
     """x [R,T,H] uint16 (bf16 bits), topk_idx [R,T,K] int32.  Returns a dict of outputs;
-    rows beyond recv_count keep the value `fill`."""
+    rows beyond recv_count keep the value `fill` (fill=None: they are not initialised at all)."""
     x = _c(x, np.uint16)
     topk_idx = _c(topk_idx, np.int32)
     R, T, H = x.shape
     K = topk_idx.shape[2]
     El, N = num_experts // R, R * max_tok
-    def filled(shape, dtype):  # every byte = fill
+    def filled(shape, dtype):  # every byte = fill; fill=None leaves the memory as allocated (untouched pages)
+        if fill is None:
+            return np.empty(shape, dtype)
         return np.full(int(np.prod(shape)) * np.dtype(dtype).itemsize, fill, np.uint8).view(dtype).reshape(shape)
 
     recv_x = filled((R, El, N, H), np.uint8 if use_fp8 else np.uint16)

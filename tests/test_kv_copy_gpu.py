@@ -73,6 +73,32 @@ def test_aligned_descriptors_match_oracle(cuda, upl, nt):
     assert info.payload_bytes == sum(lens)
 
 
+@pytest.mark.parametrize("sort_scatter", [0, 2])
+@pytest.mark.parametrize("n", [1024, 3000, 5121])
+def test_scatter_of_consecutive_memory_matches_oracle(cuda, n, sort_scatter):
+    """Equal blocks out of consecutive memory into a random permutation of places: the plan
+    takes the single-pass lowering and (sort_scatter=0) reorders its records on the device;
+    with the reordering off (2) the same bytes must arrive.  A few neighbouring blocks are
+    merged into longer descriptors, as the agent does."""
+    import torch
+    rng = np.random.default_rng(n)
+    blk = 8192
+    half = (n + 8) * blk
+    perm = rng.permutation(n)
+    src_off = [i * blk for i in range(n)]
+    dst_off = [half + int(p) * blk for p in perm]
+    lens = [blk] * n
+    # merge what happens to be adjacent on both sides
+    so, do, ln = [src_off[0]], [dst_off[0]], [blk]
+    for i in range(1, n):
+        if dst_off[i] == do[-1] + ln[-1] and src_off[i] == so[-1] + ln[-1]:
+            ln[-1] += blk
+        else:
+            so.append(src_off[i]); do.append(dst_off[i]); ln.append(blk)
+    info = _check_against_oracle(torch, cuda, 2 * half, so, do, ln, (0, 0, 0, 0, 0, sort_scatter), seed=n)
+    assert info.uniform_chunks == n * (blk // 1024) and info.mixed_chunks == 0 and info.piece_items == 0
+
+
 def test_ragged_small_descriptors_match_oracle(cuda):
     # BASELINE config 3 in miniature: sizes log-uniform in [512, 4096] rounded to 16.
     import torch
