@@ -229,7 +229,7 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
     return out
 
 
-def run_small_descriptors(steps=20, warmup=3):
+def run_small_descriptors(steps=20, warmup=3, backend_params=None):
     """Small-descriptor stress: 262 144 VRAM->VRAM descriptors with sizes log-uniform in
     [512 B, 4 KiB] rounded to 16 B, random 16-byte-aligned offsets in two 4 GiB buffers,
     destinations non-overlapping.  One request through the agent; HIP events on the launch
@@ -244,7 +244,7 @@ def run_small_descriptors(steps=20, warmup=3):
     dst = torch.zeros(buf_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.Stream(device=dev)
     agent = nixl_agent("small", nixl_agent_config(backends=()))
-    agent.create_backend("HIP", {"stream": str(stream.cuda_stream)})
+    agent.create_backend("HIP", {"stream": str(stream.cuda_stream), **(backend_params or {})})
     agent.register_memory([src, dst])
     so = (rng.integers(0, (buf_bytes - 4096) // 16, n) * 16).astype(np.uint64)
     do = (rng.permutation(buf_bytes // 8192)[:n] * 8192 + rng.integers(0, (8192 - 4096) // 16, n) * 16).astype(np.uint64)

@@ -1,5 +1,8 @@
 #include "hip_backend.h"
 
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
 #include <unistd.h>
 
 #include <algorithm>
@@ -70,7 +73,8 @@ private:
 std::mutex g_registryMutex;
 std::unordered_map<std::string, const nixlHipEngine *> g_registry;
 
-// What a peer needs to address a region (getPublicData / loadRemoteMD).
+// What a peer needs to address a region (getPublicData / loadRemoteMD).  A peer of another
+// process also needs the IPC handle of the allocation the region lies in.
 struct PublicRegion {
     uint64_t magic;
     uint64_t addr;
@@ -78,11 +82,116 @@ struct PublicRegion {
     int64_t pid;
     int32_t device;
     int32_t mem;
+    uint64_t alloc_base;
+    uint64_t alloc_size;
+    uint32_t has_ipc;
+    uint32_t reserved;
+    hipIpcMemHandle_t ipc;
 };
-constexpr uint64_t kRegionMagic = 0x314e474552504948ull; // "HIPREGN1"
-constexpr const char *kConnPrefix = "HIP1:pid=";
+constexpr uint64_t kRegionMagic = 0x324e474552504948ull; // "HIPREGN2"
+constexpr const char *kConnPrefix = "HIP2:pid=";
+constexpr const char *kConnMailbox = ";mbox=";
+// Allocations of 2 GiB and more are not shared between processes: opening such a mapping has
+// been seen not to return.
+constexpr size_t kMaxIpcAllocation = (size_t{2} << 30) - 1;
+
+constexpr uint32_t kMailboxSlots = 256;
+constexpr uint32_t kMailboxSlotBytes = 4096 - 16;
+constexpr uint32_t kMailboxMagic = 0x584f424du; // "MBOX"
+std::atomic<unsigned> g_mailboxCounter{0};
 
 } // namespace
+
+// A bounded multi-producer, single-consumer ring in POSIX shared memory (cell sequence numbers
+// as in Vyukov's bounded queue): producers are the engines of other processes, the consumer is
+// the engine that created it.  A message is the sender's agent name followed by the payload.
+struct nixlHipEngine::Mailbox {
+    struct Cell {
+        std::atomic<uint64_t> sequence;
+        uint32_t senderLen;
+        uint32_t msgLen;
+        char data[kMailboxSlotBytes];
+    };
+    std::atomic<uint32_t> magic;
+    std::atomic<uint64_t> head; // next position to write
+    std::atomic<uint64_t> tail; // next position to read
+    Cell cells[kMailboxSlots];
+
+    bool
+    push(const std::string &sender, const std::string &msg) {
+        if (sender.size() + msg.size() > kMailboxSlotBytes) return false;
+        uint64_t pos = head.load(std::memory_order_relaxed);
+        for (;;) {
+            Cell &c = cells[pos % kMailboxSlots];
+            const uint64_t seq = c.sequence.load(std::memory_order_acquire);
+            const int64_t dif = static_cast<int64_t>(seq) - static_cast<int64_t>(pos);
+            if (dif == 0) {
+                if (head.compare_exchange_weak(pos, pos + 1, std::memory_order_relaxed)) {
+                    c.senderLen = static_cast<uint32_t>(sender.size());
+                    c.msgLen = static_cast<uint32_t>(msg.size());
+                    std::memcpy(c.data, sender.data(), sender.size());
+                    std::memcpy(c.data + sender.size(), msg.data(), msg.size());
+                    c.sequence.store(pos + 1, std::memory_order_release);
+                    return true;
+                }
+            } else if (dif < 0) {
+                return false; // full: the owner has not drained it
+            } else {
+                pos = head.load(std::memory_order_relaxed);
+            }
+        }
+    }
+
+    bool
+    pop(std::string &sender, std::string &msg) {
+        const uint64_t pos = tail.load(std::memory_order_relaxed);
+        Cell &c = cells[pos % kMailboxSlots];
+        if (c.sequence.load(std::memory_order_acquire) != pos + 1) return false; // empty
+        const uint32_t sl = std::min(c.senderLen, kMailboxSlotBytes), ml = std::min(c.msgLen, kMailboxSlotBytes - sl);
+        sender.assign(c.data, sl);
+        msg.assign(c.data + sl, ml);
+        tail.store(pos + 1, std::memory_order_relaxed);
+        c.sequence.store(pos + kMailboxSlots, std::memory_order_release);
+        return true;
+    }
+};
+
+nixlHipEngine::Mailbox *
+nixlHipEngine::mapMailbox(const std::string &name, bool create) {
+    static_assert(std::atomic<uint64_t>::is_always_lock_free, "the mailbox needs lock-free 64-bit atomics");
+    const int fd = shm_open(name.c_str(), create ? (O_RDWR | O_CREAT | O_EXCL) : O_RDWR, 0600);
+    if (fd < 0) return nullptr;
+    if (create && ftruncate(fd, sizeof(Mailbox)) != 0) {
+        close(fd);
+        shm_unlink(name.c_str());
+        return nullptr;
+    }
+    struct stat st {};
+    if (fstat(fd, &st) != 0 || static_cast<size_t>(st.st_size) < sizeof(Mailbox)) {
+        close(fd);
+        return nullptr;
+    }
+    void *mem = mmap(nullptr, sizeof(Mailbox), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    close(fd);
+    if (mem == MAP_FAILED) return nullptr;
+    auto *m = static_cast<Mailbox *>(mem);
+    if (create) {
+        for (uint32_t i = 0; i < kMailboxSlots; ++i)
+            m->cells[i].sequence.store(i, std::memory_order_relaxed);
+        m->head.store(0, std::memory_order_relaxed);
+        m->tail.store(0, std::memory_order_relaxed);
+        m->magic.store(kMailboxMagic, std::memory_order_release);
+    } else if (m->magic.load(std::memory_order_acquire) != kMailboxMagic) {
+        munmap(mem, sizeof(Mailbox));
+        return nullptr;
+    }
+    return m;
+}
+
+void
+nixlHipEngine::unmapMailbox(Mailbox *m) {
+    if (m) munmap(m, sizeof(Mailbox));
+}
 
 nixlHipReqH::~nixlHipReqH() {
     const DeviceScope on_device(device);
@@ -129,6 +238,16 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
         std::lock_guard<std::mutex> lock(g_registryMutex);
         g_registry[localAgent] = this;
     }
+    // Where agents of other processes leave their notifications.  Without it (no /dev/shm)
+    // the engine still serves this process.
+    mailboxName_ = "/nixl_amd_hip_" + std::to_string(static_cast<long long>(getpid())) + "_" +
+        std::to_string(g_mailboxCounter.fetch_add(1));
+    mailbox_ = mapMailbox(mailboxName_, true);
+    if (!mailbox_) {
+        NIXL_WARN << "HIP backend: no shared-memory mailbox (" << std::strerror(errno) << "); agents of other processes cannot notify '"
+                  << localAgent << "'";
+        mailboxName_.clear();
+    }
     if (init_params->enableProgTh) {
         progressOn_ = true;
         progressDelayUs_ = init_params->pthrDelay;
@@ -151,6 +270,16 @@ nixlHipEngine::~nixlHipEngine() {
         if (it != g_registry.end() && it->second == this) g_registry.erase(it);
     }
     reapRetired(true);
+    if (mailbox_) {
+        unmapMailbox(mailbox_);
+        shm_unlink(mailboxName_.c_str());
+    }
+    for (auto &[name, peer] : peers_)
+        unmapMailbox(peer.mailbox);
+    for (auto &[key, map] : ipcMaps_) {
+        const DeviceScope on_device(map.device);
+        (void)hipIpcCloseMemHandle(map.base);
+    }
     for (const auto &[table, device] : memViews_) {
         const DeviceScope on_device(device);
         (void)hipFree(table);
@@ -234,6 +363,7 @@ nixlHipEngine::registerMem(const nixlBlobDesc &mem, const nixl_mem_t &nixl_mem, 
 
     void *base = nullptr;
     size_t size = 0;
+    bool have_range = false;
     if (hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t *>(&base), &size,
                               reinterpret_cast<hipDeviceptr_t>(const_cast<void *>(ptr))) == hipSuccess) {
         const uintptr_t b = reinterpret_cast<uintptr_t>(base);
@@ -242,11 +372,25 @@ nixlHipEngine::registerMem(const nixlBlobDesc &mem, const nixl_mem_t &nixl_mem, 
                        << ") exceeds its allocation";
             return NIXL_ERR_INVALID_PARAM;
         }
+        have_range = true;
     } else {
         (void)hipGetLastError();
     }
 
-    out = new nixlHipMD(mem.addr, mem.len, device, nixl_mem);
+    auto *md = new nixlHipMD(mem.addr, mem.len, device, nixl_mem);
+    if (nixl_mem == VRAM_SEG && have_range && size <= kMaxIpcAllocation) {
+        // What an agent of another process needs to map this allocation.  A failure only means
+        // that the region stays private to this process.
+        const DeviceScope on_device(device);
+        if (on_device.ok() && hipIpcGetMemHandle(&md->ipc, base) == hipSuccess) {
+            md->hasIpc = true;
+            md->allocBase = reinterpret_cast<uintptr_t>(base);
+            md->allocSize = size;
+        } else {
+            (void)hipGetLastError();
+        }
+    }
+    out = md;
     return NIXL_SUCCESS;
 }
 
@@ -312,8 +456,9 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
             }
         }
         const bool write = (operation == NIXL_WRITE);
-        lowered[i].src = write ? l.addr : r.addr;
-        lowered[i].dst = write ? r.addr : l.addr;
+        const uintptr_t la = lmd->here(l.addr), ra = rmd->here(r.addr); // a peer's region may be mapped elsewhere here
+        lowered[i].src = write ? la : ra;
+        lowered[i].dst = write ? ra : la;
         lowered[i].len = l.len;
         bytes += l.len;
     }
@@ -423,7 +568,7 @@ bool
 nixlHipEngine::knowsAgent(const std::string &name) const {
     if (name == localAgent) return true;
     std::lock_guard<std::mutex> lock(peersMutex_);
-    return std::find(peers_.begin(), peers_.end(), name) != peers_.end();
+    return peers_.count(name) != 0;
 }
 
 // Takes the request off the progress thread's list and, if its copy completed, queues its
@@ -489,7 +634,7 @@ nixlHipEngine::progressLoop() {
 
 nixl_status_t
 nixlHipEngine::getConnInfo(std::string &str) const {
-    str = kConnPrefix + std::to_string(static_cast<long long>(getpid()));
+    str = kConnPrefix + std::to_string(static_cast<long long>(getpid())) + kConnMailbox + mailboxName_;
     return NIXL_SUCCESS;
 }
 
@@ -499,15 +644,30 @@ nixlHipEngine::loadRemoteConnInfo(const std::string &remote_agent, const std::st
     if (remote_conn_info.compare(0, n, kConnPrefix) != 0) return NIXL_ERR_MISMATCH;
     char *end = nullptr;
     const long long pid = std::strtoll(remote_conn_info.c_str() + n, &end, 10);
-    if (end == remote_conn_info.c_str() + n || *end != '\0') return NIXL_ERR_MISMATCH;
+    if (end == remote_conn_info.c_str() + n || std::strncmp(end, kConnMailbox, std::strlen(kConnMailbox)) != 0)
+        return NIXL_ERR_MISMATCH;
+    peerInfo peer;
+    peer.pid = pid;
+    peer.mailboxName = end + std::strlen(kConnMailbox);
     if (pid != static_cast<long long>(getpid())) {
-        // Its addresses mean nothing here without IPC memory handles.
-        NIXL_WARN << "HIP backend: agent '" << remote_agent << "' lives in process " << pid
-                  << "; only agents of this process are reachable";
-        return NIXL_ERR_NOT_SUPPORTED;
+        // An agent of another process is reached through its mailbox: without one it could
+        // never be told that a transfer has landed.
+        if (peer.mailboxName.empty() || peer.mailboxName[0] != '/') return NIXL_ERR_MISMATCH;
+        peer.mailbox = mapMailbox(peer.mailboxName, false);
+        if (!peer.mailbox) {
+            NIXL_ERROR << "HIP backend: mailbox '" << peer.mailboxName << "' of agent '" << remote_agent << "' (process " << pid
+                       << ") cannot be opened";
+            return NIXL_ERR_NOT_FOUND;
+        }
     }
     std::lock_guard<std::mutex> lock(peersMutex_);
-    if (std::find(peers_.begin(), peers_.end(), remote_agent) == peers_.end()) peers_.push_back(remote_agent);
+    const auto it = peers_.find(remote_agent);
+    if (it != peers_.end()) {
+        unmapMailbox(it->second.mailbox);
+        it->second = peer;
+    } else {
+        peers_.emplace(remote_agent, peer);
+    }
     return NIXL_SUCCESS;
 }
 
@@ -520,8 +680,9 @@ nixl_status_t
 nixlHipEngine::disconnect(const std::string &remote_agent) {
     if (remote_agent == localAgent) return NIXL_SUCCESS;
     std::lock_guard<std::mutex> lock(peersMutex_);
-    const auto it = std::find(peers_.begin(), peers_.end(), remote_agent);
+    const auto it = peers_.find(remote_agent);
     if (it == peers_.end()) return NIXL_ERR_NOT_FOUND;
+    unmapMailbox(it->second.mailbox);
     peers_.erase(it);
     return NIXL_SUCCESS;
 }
@@ -537,6 +698,10 @@ nixlHipEngine::getPublicData(const nixlBackendMD *meta, std::string &str) const 
     region.pid = static_cast<int64_t>(getpid());
     region.device = md->device;
     region.mem = static_cast<int32_t>(md->mem);
+    region.alloc_base = md->allocBase;
+    region.alloc_size = md->allocSize;
+    region.has_ipc = md->hasIpc ? 1u : 0u;
+    region.ipc = md->ipc;
     str.assign(reinterpret_cast<const char *>(&region), sizeof(region));
     return NIXL_SUCCESS;
 }
@@ -551,13 +716,70 @@ nixlHipEngine::loadRemoteMD(const nixlBlobDesc &input,
     PublicRegion region{};
     if (input.metaInfo.size() != sizeof(region)) return NIXL_ERR_MISMATCH;
     std::memcpy(&region, input.metaInfo.data(), sizeof(region));
-    if (region.magic != kRegionMagic || region.pid != static_cast<int64_t>(getpid())) return NIXL_ERR_MISMATCH;
+    if (region.magic != kRegionMagic) return NIXL_ERR_MISMATCH;
     if (region.addr != input.addr || region.len != input.len || region.mem != static_cast<int32_t>(nixl_mem) ||
         region.len == 0 || region.device < 0 || region.device >= numDevices_) {
         NIXL_ERROR << "HIP backend: published data of agent '" << remote_agent << "' does not match its descriptor";
         return NIXL_ERR_MISMATCH;
     }
-    output = new nixlHipMD(region.addr, region.len, region.device, nixl_mem, /*of_peer=*/true);
+
+    if (region.pid == static_cast<int64_t>(getpid())) {
+        // A peer of this process: the region must be memory the runtime knows NOW, of the
+        // stated kind, on the stated device, inside one allocation.  A blob that outlived its
+        // registration (the peer freed the memory) would otherwise send kernels to unmapped
+        // addresses.
+        hipPointerAttribute_t attr{};
+        const void *ptr = reinterpret_cast<const void *>(static_cast<uintptr_t>(region.addr));
+        void *base = nullptr;
+        size_t size = 0;
+        const bool known = hipPointerGetAttributes(&attr, ptr) == hipSuccess &&
+            attr.type == (nixl_mem == VRAM_SEG ? hipMemoryTypeDevice : hipMemoryTypeHost) &&
+            (nixl_mem != VRAM_SEG || attr.device == region.device) &&
+            hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t *>(&base), &size,
+                                  reinterpret_cast<hipDeviceptr_t>(const_cast<void *>(ptr))) == hipSuccess &&
+            region.len <= size && region.addr - reinterpret_cast<uintptr_t>(base) <= size - region.len;
+        if (!known) {
+            (void)hipGetLastError(); // a failed query leaves a sticky error behind
+            NIXL_ERROR << "HIP backend: region [" << region.addr << ", +" << region.len << ") published by agent '" << remote_agent
+                       << "' is not live memory of the stated kind";
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        output = new nixlHipMD(region.addr, region.len, region.device, nixl_mem, /*of_peer=*/true);
+        return NIXL_SUCCESS;
+    }
+
+    // A peer of another process: map the allocation the region lies in (once per allocation).
+    if (nixl_mem != VRAM_SEG || !region.has_ipc) {
+        NIXL_ERROR << "HIP backend: agent '" << remote_agent << "' (process " << region.pid
+                   << ") published a region that cannot be shared between processes (pinned host memory, or an allocation of 2 GiB or more)";
+        return NIXL_ERR_NOT_SUPPORTED;
+    }
+    if (region.alloc_size == 0 || region.alloc_size > kMaxIpcAllocation || region.addr < region.alloc_base ||
+        region.len > region.alloc_size || region.addr - region.alloc_base > region.alloc_size - region.len)
+        return NIXL_ERR_MISMATCH;
+    const std::string key = std::to_string(region.pid) + ":" + std::to_string(region.alloc_base);
+    void *mapped = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(ipcMutex_);
+        auto it = ipcMaps_.find(key);
+        if (it == ipcMaps_.end()) {
+            const DeviceScope on_device(region.device);
+            void *base = nullptr;
+            if (!on_device.ok() || hipIpcOpenMemHandle(&base, region.ipc, hipIpcMemLazyEnablePeerAccess) != hipSuccess || !base) {
+                (void)hipGetLastError();
+                NIXL_ERROR << "HIP backend: the allocation of agent '" << remote_agent << "' (process " << region.pid
+                           << ") cannot be opened; it may have been freed";
+                return NIXL_ERR_INVALID_PARAM;
+            }
+            it = ipcMaps_.emplace(key, ipcMapping{base, region.device, 0}).first;
+        }
+        ++it->second.refs;
+        mapped = it->second.base;
+    }
+    const intptr_t delta = static_cast<intptr_t>(reinterpret_cast<uintptr_t>(mapped)) - static_cast<intptr_t>(region.alloc_base);
+    auto *md = new nixlHipMD(region.addr, region.len, region.device, nixl_mem, /*of_peer=*/true, delta);
+    md->ipcKey = key;
+    output = md;
     return NIXL_SUCCESS;
 }
 
@@ -565,18 +787,48 @@ nixl_status_t
 nixlHipEngine::unloadMD(nixlBackendMD *input) {
     // loadLocalMD hands out the registration itself, which deregisterMem frees
     const auto *md = static_cast<const nixlHipMD *>(input);
-    if (md && md->ofPeer) delete md;
+    if (!md || !md->ofPeer) return NIXL_SUCCESS;
+    if (!md->ipcKey.empty()) {
+        // Kernels of transfers still in flight may be using the mapping.
+        reapRetired(true);
+        std::lock_guard<std::mutex> lock(ipcMutex_);
+        const auto it = ipcMaps_.find(md->ipcKey);
+        if (it != ipcMaps_.end() && --it->second.refs == 0) {
+            const DeviceScope on_device(it->second.device);
+            (void)hipDeviceSynchronize();
+            (void)hipIpcCloseMemHandle(it->second.base);
+            ipcMaps_.erase(it);
+        }
+    }
+    delete md;
     return NIXL_SUCCESS;
 }
 
 nixl_status_t
 nixlHipEngine::genNotif(const std::string &remote_agent, const std::string &msg) const {
-    std::lock_guard<std::mutex> registry(g_registryMutex);
-    const auto it = g_registry.find(remote_agent);
-    if (it == g_registry.end()) return NIXL_ERR_NOT_FOUND;
-    const nixlHipEngine *target = it->second;
-    std::lock_guard<std::mutex> lock(target->notifMutex_);
-    target->notifs_.emplace_back(localAgent, msg);
+    {
+        std::lock_guard<std::mutex> registry(g_registryMutex);
+        const auto it = g_registry.find(remote_agent);
+        if (it != g_registry.end()) {
+            const nixlHipEngine *target = it->second;
+            std::lock_guard<std::mutex> lock(target->notifMutex_);
+            target->notifs_.emplace_back(localAgent, msg);
+            return NIXL_SUCCESS;
+        }
+    }
+    // not an engine of this process: a peer with a mailbox in shared memory
+    std::lock_guard<std::mutex> lock(peersMutex_);
+    const auto it = peers_.find(remote_agent);
+    if (it == peers_.end() || !it->second.mailbox) return NIXL_ERR_NOT_FOUND;
+    if (localAgent.size() + msg.size() > kMailboxSlotBytes) {
+        NIXL_ERROR << "HIP backend: a notification to another process holds at most " << kMailboxSlotBytes
+                   << " bytes (agent name included)";
+        return NIXL_ERR_NOT_SUPPORTED;
+    }
+    if (!it->second.mailbox->push(localAgent, msg)) {
+        NIXL_ERROR << "HIP backend: the mailbox of agent '" << remote_agent << "' is full";
+        return NIXL_ERR_BACKEND;
+    }
     return NIXL_SUCCESS;
 }
 
@@ -588,6 +840,11 @@ nixlHipEngine::getNotifs(notif_list_t &notif_list) {
     for (auto &n : notifs_)
         notif_list.push_back(std::move(n));
     notifs_.clear();
+    if (mailbox_) {
+        std::string sender, msg;
+        while (mailbox_->pop(sender, msg))
+            notif_list.emplace_back(std::move(sender), std::move(msg));
+    }
     return NIXL_SUCCESS;
 }
 
@@ -681,7 +938,7 @@ nixlHipEngine::buildMemView(const std::vector<viewEntry> &entries, uint32_t kind
                     return NIXL_ERR_NOT_SUPPORTED;
                 }
             }
-            out.addr = e.addr;
+            out.addr = e.md->here(e.addr);
             out.len = e.len;
         }
         std::memcpy(&image[2 + 2 * i], &out, sizeof(out));

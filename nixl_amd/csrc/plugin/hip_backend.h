@@ -1,5 +1,8 @@
 // nixlHipEngine: a NIXL backend for VRAM<->VRAM descriptor transfers on one AMD GPU, between
-// the regions of one agent (loopback) or of several agents that live in the same process.  It fills the same slot as the reference's local backends (shape of
+// the regions of one agent (loopback), of several agents that live in the same process, or of
+// agents in other processes on the same GPU (their memory is mapped through HIP IPC handles,
+// their notifications travel through a shared-memory mailbox).  It fills the same slot as the
+// reference's local backends (shape of
 // src/plugins/posix/posix_backend.h:78-158; request life-cycle split of
 // src/plugins/cuda_gds/gds_backend.cpp:159-391): prepXfer lowers the two descriptor
 // lists once into a device-resident copy plan, postXfer enqueues one kernel launch and
@@ -22,25 +25,45 @@
 #include "nixl_amd_hip.h"
 
 // Registration record returned by registerMem and handed back in nixlMetaDesc::metadataP.
+// `addr` is the region's address in its OWNER's address space, which is the space the
+// descriptors of that agent are written in; `delta` takes such an address to where the region
+// is mapped in this process (0 for this process's own memory, the offset of the opened IPC
+// mapping for a region of another process).
 class nixlHipMD : public nixlBackendMD {
 public:
-    nixlHipMD(uintptr_t addr_, size_t len_, int device_, nixl_mem_t mem_, bool of_peer = false)
+    nixlHipMD(uintptr_t addr_, size_t len_, int device_, nixl_mem_t mem_, bool of_peer = false, intptr_t delta_ = 0)
         : nixlBackendMD(!of_peer),
           addr(addr_),
           len(len_),
           device(device_),
           mem(mem_),
-          ofPeer(of_peer) {}
+          ofPeer(of_peer),
+          delta(delta_) {}
 
     const uintptr_t addr;
     const size_t len;
     const int device; // HIP device whose kernels may touch the region
     const nixl_mem_t mem;
     const bool ofPeer; // made by loadRemoteMD from a peer's published data; unloadMD frees it
+    const intptr_t delta;
+    // What another process needs to map the allocation the region lies in (own VRAM regions
+    // whose allocation is small enough to be shared).
+    bool hasIpc = false;
+    hipIpcMemHandle_t ipc{};
+    uintptr_t allocBase = 0;
+    size_t allocSize = 0;
+    // For a region of another process: the key of the opened mapping, released by unloadMD.
+    std::string ipcKey;
 
     bool
     contains(uintptr_t a, size_t l) const noexcept {
         return a >= addr && l <= len && (a - addr) <= (len - l);
+    }
+
+    // Address in this process of the owner's address `a`.
+    uintptr_t
+    here(uintptr_t a) const noexcept {
+        return static_cast<uintptr_t>(static_cast<intptr_t>(a) + delta);
     }
 };
 
@@ -66,8 +89,8 @@ public:
     explicit nixlHipEngine(const nixlBackendInitParams *init_params);
     ~nixlHipEngine() override;
 
-    // "Remote" means another agent of this process: its regions are plain addresses here.
-    // An agent in another process would need IPC memory handles, which are left out.
+    // "Remote" means another agent on the same GPU: of this process (its regions are plain
+    // addresses here) or of another one (its allocations are opened through IPC handles).
     bool
     supportsRemote() const override {
         return true;
@@ -215,9 +238,31 @@ private:
     bool progressOn_ = false;
     uint64_t progressDelayUs_ = 0;
     std::thread progress_;
-    // Peers whose connection info was loaded (agents of this process).
+    // Peers whose connection info was loaded: agents of this process (no mailbox: their
+    // engine is found in the process-wide registry) or of another one.
+    struct Mailbox; // shared-memory ring of notifications, defined with its users
+    struct peerInfo {
+        long long pid = 0;
+        std::string mailboxName;
+        Mailbox *mailbox = nullptr; // mapped on first use
+    };
     mutable std::mutex peersMutex_;
-    std::vector<std::string> peers_;
+    mutable std::unordered_map<std::string, peerInfo> peers_;
+    // This engine's own mailbox, where agents of other processes leave notifications.
+    std::string mailboxName_;
+    Mailbox *mailbox_ = nullptr;
+    // Allocations of other processes opened here: "<pid>:<allocation base>" -> mapping.
+    struct ipcMapping {
+        void *base = nullptr;
+        int device = 0;
+        int refs = 0;
+    };
+    mutable std::mutex ipcMutex_;
+    mutable std::unordered_map<std::string, ipcMapping> ipcMaps_;
+    static Mailbox *
+    mapMailbox(const std::string &name, bool create);
+    static void
+    unmapMailbox(Mailbox *m);
     // Notifications other agents (or this one) left for this agent.
     mutable std::mutex notifMutex_;
     mutable notif_list_t notifs_;

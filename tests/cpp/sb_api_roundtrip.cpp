@@ -207,7 +207,10 @@ main(int argc, char **argv) {
         REQUIRE(target->getPublicData(t_md, t_public) == NIXL_SUCCESS && !t_public.empty());
         // nothing of the peer is usable before its connection info is loaded
         REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public), VRAM_SEG, peer, t_at_initiator) < 0);
-        REQUIRE(engine->loadRemoteConnInfo(peer, "HIP1:pid=1") == NIXL_ERR_NOT_SUPPORTED); // another process
+        REQUIRE(engine->loadRemoteConnInfo(peer, "HIP1:pid=1") < 0); // an older format
+        // another process whose mailbox does not exist cannot be connected to
+        REQUIRE(engine->loadRemoteConnInfo(peer, "HIP2:pid=1;mbox=/nixl_amd_hip_no_such_mailbox") == NIXL_ERR_NOT_FOUND);
+        REQUIRE(engine->loadRemoteConnInfo(peer, "HIP2:pid=1;mbox=") < 0);
         REQUIRE(engine->loadRemoteConnInfo(peer, "garbage") < 0);
         REQUIRE(engine->loadRemoteConnInfo(peer, t_conn) == NIXL_SUCCESS);
         REQUIRE(engine->connect(peer) == NIXL_SUCCESS);
@@ -215,6 +218,25 @@ main(int argc, char **argv) {
         REQUIRE(engine->loadRemoteMD(nixlBlobDesc(reinterpret_cast<uintptr_t>(tbuf), total / 2, 0, t_public), VRAM_SEG, peer,
                                      t_at_initiator) < 0);
         REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public.substr(1)), VRAM_SEG, peer, t_at_initiator) < 0);
+        {
+            // a blob that names memory the runtime does not know (a region freed since it was
+            // published, a forged record) is refused on the host: no kernel may ever see it
+            std::string stale = t_public;
+            const uint64_t nowhere = 0x7f0000001000ull;
+            std::memcpy(&stale[8], &nowhere, sizeof(nowhere)); // the record's address field
+            REQUIRE(engine->loadRemoteMD(nixlBlobDesc(nowhere, total, 0, stale), VRAM_SEG, peer, t_at_initiator) ==
+                    NIXL_ERR_INVALID_PARAM);
+            REQUIRE(t_at_initiator == nullptr);
+            // live memory of the wrong kind: a host buffer published as VRAM
+            void *pinned = nullptr;
+            REQUIRE(hipHostMalloc(&pinned, 4096, hipHostMallocDefault) == hipSuccess);
+            const uint64_t host_addr = reinterpret_cast<uint64_t>(pinned), host_len = 4096;
+            std::memcpy(&stale[8], &host_addr, sizeof(host_addr));
+            std::memcpy(&stale[16], &host_len, sizeof(host_len));
+            REQUIRE(engine->loadRemoteMD(nixlBlobDesc(host_addr, host_len, 0, stale), VRAM_SEG, peer, t_at_initiator) ==
+                    NIXL_ERR_INVALID_PARAM);
+            REQUIRE(hipHostFree(pinned) == hipSuccess);
+        }
         REQUIRE(engine->loadRemoteMD(nixlBlobDesc(t_region, t_public), VRAM_SEG, peer, t_at_initiator) == NIXL_SUCCESS);
         REQUIRE(t_at_initiator && t_at_initiator != t_md);
 

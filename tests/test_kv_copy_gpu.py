@@ -289,7 +289,7 @@ def test_two_agents_in_one_process(cuda):
     b.register_memory([dst])
     torch.cuda.synchronize()
     md = b.get_agent_metadata()
-    assert md.startswith(b"nixlSerDes|Agent") and b"HIP1:pid=" in md and b"bknd" in md
+    assert md.startswith(b"nixlSerDes|Agent") and b"HIP2:pid=" in md and b"bknd" in md
     assert a.add_remote_agent(md) == "target"
     assert b.add_remote_agent(a.get_agent_metadata()) == "initiator"
     a.make_connection("target")
