@@ -456,7 +456,7 @@ nixl_capi_xfer_req_get_desc(nixl_capi_xfer_req_t req, size_t i, uint64_t *local_
 
 nixl_capi_status_t
 nixl_capi_release_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req) {
-    if (!agent || !req) return NIXL_CAPI_ERROR_INVALID_PARAM;
+    if (!agent || !req || !req->req) return NIXL_CAPI_ERROR_INVALID_PARAM; // released before: src/bindings/rust/wrapper.cpp:1590-1592
     return guarded([&] {
         const nixl_status_t st = agent->inner->releaseXferReq(req->req);
         if (st == NIXL_SUCCESS) req->req = nullptr;
@@ -467,7 +467,10 @@ nixl_capi_release_xfer_req(nixl_capi_agent_t agent, nixl_capi_xfer_req_t req) {
 nixl_capi_status_t
 nixl_capi_destroy_xfer_req(nixl_capi_xfer_req_t req) {
     if (!req) return NIXL_CAPI_ERROR_INVALID_PARAM;
-    delete req; // the inner request was handed back by nixl_capi_release_xfer_req
+    // The inner request, its device plan and its event belong to the agent until
+    // nixl_capi_release_xfer_req has handed them back (src/bindings/rust/wrapper.cpp:1606-1609).
+    if (req->req) return NIXL_CAPI_ERROR_INVALID_STATE;
+    delete req;
     return NIXL_CAPI_SUCCESS;
 }
 

@@ -364,6 +364,27 @@ def test_list_and_option_helpers_of_the_c_wrapper(two_agents):
     assert lib.nixl_capi_is_stub() == 0
 
 
+def test_request_handles_are_destroyed_only_after_release(two_agents):
+    """src/bindings/rust/wrapper.cpp:1586-1612: destroying a request wrapper that still owns
+    its request is an INVALID_STATE error (nothing is freed), releasing it twice an
+    INVALID_PARAM error."""
+    from nixl_amd import _lib
+    lib = _lib.agent_lib()
+    a, _ = two_agents
+    src, dst = np.arange(4096, dtype=np.uint8) % 251, np.zeros(4096, np.uint8)
+    _reg(a, src)
+    _reg(a, dst)
+    req = a.initialize_xfer("WRITE", _descs(a, src, [0], [4096]), _descs(a, dst, [0], [4096]), "alpha")
+    _wait(a, req)
+    assert np.array_equal(src, dst)
+    assert lib.nixl_capi_destroy_xfer_req(req._handle) == -3  # NIXL_CAPI_ERROR_INVALID_STATE: still owned
+    _wait(a, req)  # and still usable
+    assert lib.nixl_capi_release_xfer_req(a._h, req._handle) == 0
+    assert lib.nixl_capi_release_xfer_req(a._h, req._handle) == -1  # NIXL_CAPI_ERROR_INVALID_PARAM: released before
+    assert lib.nixl_capi_destroy_xfer_req(req._handle) == 0
+    req._handle = None  # nothing left for the Python wrapper to release
+
+
 def test_descriptor_lists_as_bytes_and_absent_side_channels(two_agents):
     """get_serialized_descs / deserialize_descs (reference _api.py:1201-1221; the reference
     pickles, this build writes a flat record) and the socket / ETCD metadata calls, which say
