@@ -82,6 +82,27 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
                           const nixl_amd_copy_tuning_t *tuning,
                           nixl_amd_copy_plan_t **out);
 
+/* A plan for `n` equal blocks given by index: block i is copied from
+ * src_base + src_index[i] * src_stride to dst_base + dst_index[i] * dst_stride, `len` bytes.
+ * This is what nixlAgent::makeXferReq asks for when both prepared lists are one dense or
+ * strided run each (a paged KV pool and a staging buffer; src/core/nixl_agent.cpp:799-857
+ * expands such indices into descriptors on the host, one by one): only the two index vectors
+ * go to the device, where a kernel writes the records.  Bases and strides must be multiples
+ * of 128 and `len` a whole number of chunks (1 KiB at the default tuning); the caller checks
+ * the indices against the lists they index.  The index arrays may be freed on return. */
+int
+nixl_amd_copy_plan_create_indexed(uint64_t src_base,
+                                  uint64_t src_stride,
+                                  const int32_t *src_index,
+                                  uint64_t dst_base,
+                                  uint64_t dst_stride,
+                                  const int32_t *dst_index,
+                                  size_t n,
+                                  uint64_t len,
+                                  int device,
+                                  const nixl_amd_copy_tuning_t *tuning,
+                                  nixl_amd_copy_plan_t **out);
+
 /* Enqueue the whole plan on `stream`: the per-post work of
  * nixlUcxEngine::postXfer -> sendXferRange (src/plugins/ucx/ucx_backend.cpp:1183-1310).
  * Re-launching re-reads the current source bytes; nothing is cached at plan creation

@@ -61,6 +61,9 @@ def kernels():
     lib.nixl_amd_device_count.restype = c_int
     lib.nixl_amd_copy_plan_create.argtypes = [POINTER(CopyDesc), c_size_t, c_int,
                                               POINTER(CopyTuning), POINTER(c_void_p)]
+    lib.nixl_amd_copy_plan_create_indexed.argtypes = [c_uint64, c_uint64, c_void_p, c_uint64, c_uint64, c_void_p, c_size_t,
+                                                      c_uint64, c_int, POINTER(CopyTuning), POINTER(c_void_p)]
+    lib.nixl_amd_copy_plan_create_indexed.restype = c_int
     lib.nixl_amd_copy_plan_launch.argtypes = [c_void_p, c_void_p]
     lib.nixl_amd_copy_plan_destroy.argtypes = [c_void_p]
     lib.nixl_amd_copy_plan_query.argtypes = [c_void_p, POINTER(CopyPlanInfo)]
@@ -113,7 +116,7 @@ def ep_kernels():
 
 
 def kernel_symbols():
-    return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create",
+    return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create", "nixl_amd_copy_plan_create_indexed",
                    "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
                    "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
 

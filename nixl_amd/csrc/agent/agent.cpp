@@ -349,6 +349,12 @@ nixlAgent::createBackend(const nixl_backend_t &type, const nixl_b_params_t &para
     auto slot = std::make_unique<nixlAgentData::engineSlot>();
     slot->params = params;
     slot->plugin = plugin;
+    if (plugin->dl) // an optional entry some plugins export beside the two required ones
+    {
+        std::string symbol = "nixl_" + type + "_prep_xfer_indexed"; // e.g. nixl_hip_prep_xfer_indexed
+        std::transform(symbol.begin(), symbol.end(), symbol.begin(), [](unsigned char c) { return std::tolower(c); });
+        slot->prepIndexed = reinterpret_cast<nixlAgentData::prepIndexedFn>(dlsym(plugin->dl, symbol.c_str()));
+    }
 
     nixlBackendInitParams init;
     init.localAgent = data->name_;
@@ -730,6 +736,31 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
     const nixl_stride_dlist_t &lruns = *local_side->descs.at(backend);
     const nixl_stride_dlist_t &rruns = *remote_side->descs.at(backend);
     auto req = std::make_unique<nixlXferReqH>(remote_side->remoteAgent, operation, lruns.getType(), rruns.getType());
+
+    // Both lists one run each (a pool, a staging buffer) and a backend that lowers index
+    // vectors itself: the descriptors are never written out here.  The request then carries
+    // no descriptor lists; its backend handle holds everything postXfer needs.
+    if (lruns.descCount() == 1 && rruns.descCount() == 1) {
+        const nixlAgentData::engineSlot *slot = data->slotOf(backend->getType());
+        if (slot && slot->prepIndexed && slot->engine == backend) {
+            const nixl_status_t st = static_cast<nixl_status_t>(
+                slot->prepIndexed(backend, static_cast<int>(req->backendOp), &lruns[0], local_indices.data(), &rruns[0],
+                                  remote_indices.data(), count, req->remoteAgent.c_str(), &req->backendHandle));
+            if (st == NIXL_SUCCESS) {
+                req->engine = backend;
+                req->notifMsg = opt.notifMsg;
+                req->hasNotif = opt.hasNotif;
+                req->telemetry.totalBytes = count * lruns[0].len;
+                req->telemetry.descCount = count;
+                req_hndl = req.release();
+                return NIXL_SUCCESS;
+            }
+            if (st != NIXL_ERR_NOT_SUPPORTED) {
+                NIXL_ERROR_FUNC << "backend '" << backend->getType() << "' failed to prepare the indexed transfer request with status " << st;
+                return st;
+            }
+        }
+    }
     req->initiatorDescs.reserve(count);
     req->targetDescs.reserve(count);
 

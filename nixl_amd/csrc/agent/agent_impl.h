@@ -184,11 +184,17 @@ public:
     const std::string name_;
     const nixlAgentConfig config_;
 
+    // Optional entry of a backend plugin ("nixl_hip_prep_xfer_indexed" in the HIP plugin): a
+    // request given as two index vectors into two single-run prepared lists, lowered by the
+    // backend itself.  Null for plugins that do not export it.
+    using prepIndexedFn = int (*)(nixlBackendEngine *, int, const nixlStrideDesc *, const int *, const nixlStrideDesc *,
+                                  const int *, size_t, const char *, nixlBackendReqH **);
     struct engineSlot {
         nixlBackendEngine *engine = nullptr;
         const nixlLoadedPlugin *plugin = nullptr;
         std::unique_ptr<nixlBackendH> handle;
         nixl_b_params_t params;
+        prepIndexedFn prepIndexed = nullptr;
     };
     // Creation order is preference order.
     std::vector<std::unique_ptr<engineSlot>> engines_;

@@ -32,6 +32,7 @@
 // handle, reads them once and accumulates in fp32 with fused multiply-adds in top-k order
 // (kernels/nixl_ep_ll.cu:959-1012).  Traffic per token: read K * 2H, write 2H.
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <mutex>
 
@@ -622,8 +623,10 @@ round_up_wave(int n) {
 
 // Largest workgroup (in lanes) of the dispatch and combine kernels; a token whose row needs
 // more lanes is split over several workgroups.
-int g_dispatch_lanes = 1024;
-int g_combine_lanes = 1024;
+// Read by every call, set by nixl_amd_ep_ll_set_tuning from any thread: a call sees the old or the
+// new value, never a torn one.
+std::atomic<int> g_dispatch_lanes{1024};
+std::atomic<int> g_combine_lanes{1024};
 
 } // namespace
 
@@ -667,8 +670,8 @@ nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes) {
     auto ok = [](int v) { return v == 0 || (v >= 64 && v <= 1024 && v % 64 == 0); };
     if (!ok(dispatch_lanes) || !ok(combine_lanes))
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_set_tuning: lanes must be 0 or a multiple of 64 in [64, 1024]");
-    if (dispatch_lanes) g_dispatch_lanes = dispatch_lanes;
-    if (combine_lanes) g_combine_lanes = combine_lanes;
+    if (dispatch_lanes) g_dispatch_lanes.store(dispatch_lanes, std::memory_order_relaxed);
+    if (combine_lanes) g_combine_lanes.store(combine_lanes, std::memory_order_relaxed);
     return NIXL_AMD_OK;
 }
 
@@ -803,7 +806,7 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
         HIP_TRY(hipGetLastError());
         return NIXL_AMD_OK;
     }
-    const int wg = std::min(round_up_wave(d.H / 16), g_dispatch_lanes);
+    const int wg = std::min(round_up_wave(d.H / 16), g_dispatch_lanes.load(std::memory_order_relaxed));
     a.parts = (d.H / 16 + wg - 1) / wg;
     const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
     const dim3 block(wg);
@@ -987,7 +990,7 @@ nixl_amd_ep_ll_combine(void *combined_x,
     a.num_tokens_per_rank = num_tokens_per_rank;
     a.row_map = row_map;
     a.d = d;
-    const int wg = std::min(round_up_wave(d.H / 8), g_combine_lanes);
+    const int wg = std::min(round_up_wave(d.H / 8), g_combine_lanes.load(std::memory_order_relaxed));
     a.parts = (d.H / 8 + wg - 1) / wg;
     const dim3 grid(static_cast<unsigned>(d.R) * d.T * a.parts);
     if (use_logfmt)

@@ -488,6 +488,76 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
 }
 
 nixl_status_t
+nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
+                               const nixlStrideDesc &local_run,
+                               const int *local_indices,
+                               const nixlStrideDesc &remote_run,
+                               const int *remote_indices,
+                               size_t count,
+                               const std::string &remote_agent,
+                               nixlBackendReqH *&handle) const {
+    handle = nullptr;
+    reapRetired(false);
+    if (!knowsAgent(remote_agent)) return NIXL_ERR_NOT_FOUND;
+    if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
+    if (!local_indices || !remote_indices || count == 0) return NIXL_ERR_INVALID_PARAM;
+    if (local_run.start_idx != 0 || remote_run.start_idx != 0 || local_run.count == 0 || remote_run.count == 0)
+        return NIXL_ERR_NOT_SUPPORTED;
+    if (local_run.len != remote_run.len) {
+        NIXL_ERROR << "HIP backend: block length mismatch (local " << local_run.len << ", remote " << remote_run.len << ")";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    const auto *lmd = static_cast<const nixlHipMD *>(local_run.metadataP);
+    const auto *rmd = static_cast<const nixlHipMD *>(remote_run.metadataP);
+    auto span = [](const nixlStrideDesc &run) { return (run.count - 1) * run.stride + run.len; };
+    if (!lmd || !rmd || !lmd->contains(local_run.addr, span(local_run)) || !rmd->contains(remote_run.addr, span(remote_run))) {
+        NIXL_ERROR << "HIP backend: a prepared list reaches outside its registered region";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    int device = -1;
+    for (const nixlHipMD *md : {lmd, rmd}) {
+        if (md->mem != VRAM_SEG) continue;
+        if (device < 0) device = md->device;
+        if (md->device != device) return NIXL_ERR_NOT_SUPPORTED;
+    }
+    if (device < 0) device = lmd->device;
+    // every index must name a block of its list: one pass over each vector
+    int lmin = local_indices[0], lmax = lmin, rmin = remote_indices[0], rmax = rmin;
+    for (size_t i = 1; i < count; ++i) {
+        lmin = std::min(lmin, local_indices[i]);
+        lmax = std::max(lmax, local_indices[i]);
+        rmin = std::min(rmin, remote_indices[i]);
+        rmax = std::max(rmax, remote_indices[i]);
+    }
+    if (lmin < 0 || static_cast<size_t>(lmax) >= local_run.count || rmin < 0 || static_cast<size_t>(rmax) >= remote_run.count) {
+        NIXL_ERROR << "HIP backend: index outside its prepared list";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    const bool write = (operation == NIXL_WRITE);
+    const uint64_t la = lmd->here(local_run.addr), ra = rmd->here(remote_run.addr);
+    auto req = std::make_unique<nixlHipReqH>();
+    req->device = device;
+    req->bytes = count * local_run.len;
+    const int rc = write ? nixl_amd_copy_plan_create_indexed(la, local_run.stride, local_indices, ra, remote_run.stride,
+                                                             remote_indices, count, local_run.len, device, &tuning_, &req->plan)
+                         : nixl_amd_copy_plan_create_indexed(ra, remote_run.stride, remote_indices, la, local_run.stride,
+                                                             local_indices, count, local_run.len, device, &tuning_, &req->plan);
+    if (rc == NIXL_AMD_ERR_INVALID) return NIXL_ERR_NOT_SUPPORTED; // shape or alignment: the descriptor path handles it
+    if (rc != NIXL_AMD_OK) {
+        NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+        return NIXL_ERR_BACKEND;
+    }
+    const DeviceScope on_device(device);
+    if (!on_device.ok() || !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
+        return NIXL_ERR_BACKEND;
+    req->stream = pickStream(device);
+    if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
+    handle = req.release();
+    return NIXL_SUCCESS;
+}
+
+nixl_status_t
 nixlHipEngine::postXfer(const nixl_xfer_op_t &,
                         const nixl_meta_dlist_t &,
                         const nixl_meta_dlist_t &,
@@ -1029,3 +1099,26 @@ nixl_plugin_init() {
 
 extern "C" NIXL_PLUGIN_EXPORT void
 nixl_plugin_fini() {}
+
+// Optional entry of this plugin (not part of the reference's plugin interface): see
+// nixlHipEngine::prepXferIndexed.  `engine` must be an engine this plugin created.
+extern "C" NIXL_PLUGIN_EXPORT int
+nixl_hip_prep_xfer_indexed(nixlBackendEngine *engine,
+                           int operation,
+                           const nixlStrideDesc *local_run,
+                           const int *local_indices,
+                           const nixlStrideDesc *remote_run,
+                           const int *remote_indices,
+                           size_t count,
+                           const char *remote_agent,
+                           nixlBackendReqH **handle) {
+    if (!engine || !local_run || !remote_run || !remote_agent || !handle) return NIXL_ERR_INVALID_PARAM;
+    try {
+        return static_cast<nixlHipEngine *>(engine)->prepXferIndexed(static_cast<nixl_xfer_op_t>(operation), *local_run,
+                                                                     local_indices, *remote_run, remote_indices, count,
+                                                                     remote_agent, *handle);
+    } catch (const std::exception &e) {
+        NIXL_ERROR << "HIP backend: " << e.what();
+        return NIXL_ERR_BACKEND;
+    }
+}

@@ -214,6 +214,51 @@ def test_prepared_lists_three_requests(hip_agent, cuda):
         h.release()
 
 
+@pytest.mark.parametrize("op", ["WRITE", "READ"])
+def test_index_vectors_into_single_run_lists(hip_agent, cuda, op):
+    """A dense pool and a strided one, each prepared as ONE list that compresses into one
+    run: the request is then lowered on the device from the two index vectors (no descriptor
+    is written out on the host).  3000 blocks in random order (more than one sorting window,
+    not a multiple of it), both directions, against the per-descriptor oracle; the same
+    indices through lists that do not qualify (two regions) must give the same bytes."""
+    import torch
+    a = hip_agent
+    blk, n_pool, n = 8192, 4096, 3000
+    rng = np.random.default_rng(5)
+    host = rng.integers(0, 256, (3 * n_pool) * blk, dtype=np.uint8)
+    mem = torch.from_numpy(host.copy()).to(cuda)
+    a.register_memory([mem])
+    base = mem.data_ptr()
+    dense_offs = np.arange(n_pool) * blk  # blocks 0..n_pool-1, adjoining
+    strided_offs = n_pool * blk + np.arange(n_pool) * 2 * blk  # every other block of the rest
+    h_local = a.prep_xfer_dlist("", _descs(mem, dense_offs, [blk] * n_pool), "VRAM")
+    h_remote = a.prep_xfer_dlist("agent", _descs(mem, strided_offs, [blk] * n_pool), "VRAM")
+    assert h_local.run_count() == 1 and h_remote.run_count() == 1
+    li = rng.permutation(n_pool)[:n].astype(np.int32)
+    ri = rng.permutation(n_pool)[:n].astype(np.int32)
+    req = a.make_prepped_xfer(op, h_local, li, h_remote, ri)
+    assert req.desc_count() == (n, n * blk)
+    _wait(a, req)
+    l_off, r_off = dense_offs[li], strided_offs[ri]
+    src, dst = (l_off, r_off) if op == "WRITE" else (r_off, l_off)
+    want = ko.copy_descs(host, src, dst, [blk] * n)
+    assert np.array_equal(mem.cpu().numpy(), want)
+    # an index outside its list is refused before anything is launched
+    bad = li.copy()
+    bad[7] = n_pool
+    with pytest.raises(Exception):
+        a.make_prepped_xfer(op, h_local, bad, h_remote, ri)
+    # the ordinary path (explicit descriptors) on fresh memory gives the same bytes
+    mem.copy_(torch.from_numpy(host))
+    torch.cuda.synchronize()
+    req2 = a.initialize_xfer(op, a.get_xfer_descs(_descs(mem, l_off, [blk] * n), "VRAM"),
+                             a.get_xfer_descs(_descs(mem, r_off, [blk] * n), "VRAM"), "agent")
+    _wait(a, req2)
+    assert np.array_equal(mem.cpu().numpy(), want)
+    for h in (req, req2, h_local, h_remote):
+        h.release()
+
+
 def test_write_zero_read_roundtrip_and_repost(hip_agent, cuda):
     # transfer_handler round trip (test/gtest/plugins/transfer_handler.h:182-209 with
     # memory_handler.h:42-58): WRITE, clear the source, READ back, expect the increasing
