@@ -35,8 +35,16 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 # from inside this process: these figures come from rocprofv3 --pmc runs of this same file
 # (FETCH_SIZE and WRITE_SIZE, one run each, scaled by a plain 1 GiB element-wise kernel in the
 # same run); the summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks,
-# descriptor bytes, order); a shape without a counter run reports null.
-MEASURED_TRAFFIC = {}
+# descriptor bytes) - the two descriptor orders move the same bytes; a shape without a counter
+# run reports null.
+_KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, not this run)"
+MEASURED_TRAFFIC = {
+    (1024, 8192, 16384): {"bytes": 2164238281, "source": _KV_PROFILE},
+    (1024, 8192, 32768): {"bytes": 4311689866, "source": _KV_PROFILE},
+    ("small", 262144): {"bytes": 983229066,
+                        "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
+                                  "this file, not this run)"},
+}
 
 
 def _kv_layout():
@@ -189,7 +197,7 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
     avg_launch_ms = float(np.mean(kernel_ms))
     algorithmic_bytes_per_launch = 2 * n_desc * blk  # every payload byte read once, written once
     achieved = algorithmic_bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC.get((n_sel, pool_blocks, blk, order))
+    traffic = MEASURED_TRAFFIC.get((n_sel, pool_blocks, blk))
     out = {
         "value": payload_per_step * steps / wall / 1e9,
         "ms_per_step": wall / steps * 1e3,
