@@ -21,6 +21,10 @@
 //       descriptor j, prefix[n] = total) in a per-wave LDS slice and walks them.
 //   Descriptors that are not 16-byte aligned in src, dst and len are cut into byte-range
 //   work items handled by a third, byte-exact kernel.
+//   Lists of equal-length, line-aligned descriptors of whole chunks (KV blocks) take none of
+//   these steps: one pass writes their records, or, when the request is two index vectors
+//   into two strided runs, a kernel writes them from the indices on the device.  Arenas and
+//   the pinned buffers they are uploaded from are pooled.
 //
 // What is equal to the reference: the bytes.  For every descriptor, in list order,
 // dst[0..len) = src[0..len), the result of the per-descriptor put/get loop at
