@@ -103,6 +103,35 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
                                   const nixl_amd_copy_tuning_t *tuning,
                                   nixl_amd_copy_plan_t **out);
 
+/* One run of a prepared list: blocks first_index .. first_index + count - 1 of the list lie
+ * at base, base + stride, ...  (the stride runs a prepared descriptor list compresses into,
+ * src/api/cpp/backend/backend_aux.h:140-208). */
+typedef struct nixl_amd_copy_run {
+    uint64_t base;
+    uint64_t stride;
+    uint64_t first_index;
+    uint64_t count;
+} nixl_amd_copy_run_t;
+
+/* The same for lists of several runs (a pool registered as several regions): index i of a
+ * list names block i - first_index of the run that holds it.  Between 1 and 256 runs a side,
+ * in index order from 0 without gaps (runs[r + 1].first_index == runs[r].first_index +
+ * runs[r].count; the last run's count is not looked at); every base and stride a multiple
+ * of 128.  The run tables travel to the device with the index vectors and are searched
+ * there. */
+int
+nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
+                                       size_t n_src_runs,
+                                       const int32_t *src_index,
+                                       const nixl_amd_copy_run_t *dst_runs,
+                                       size_t n_dst_runs,
+                                       const int32_t *dst_index,
+                                       size_t n,
+                                       uint64_t len,
+                                       int device,
+                                       const nixl_amd_copy_tuning_t *tuning,
+                                       nixl_amd_copy_plan_t **out);
+
 /* Enqueue the whole plan on `stream`: the per-post work of
  * nixlUcxEngine::postXfer -> sendXferRange (src/plugins/ucx/ucx_backend.cpp:1183-1310).
  * Re-launching re-reads the current source bytes; nothing is cached at plan creation

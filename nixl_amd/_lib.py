@@ -40,6 +40,10 @@ class CopyTuning(Structure):
                 ("waves_per_workgroup", c_int), ("xcd_swizzle", c_int), ("sort_scatter", c_int)]
 
 
+class CopyRun(Structure):
+    _fields_ = [("base", c_uint64), ("stride", c_uint64), ("first_index", c_uint64), ("count", c_uint64)]
+
+
 class CopyPlanInfo(Structure):
     _fields_ = [("payload_bytes", c_uint64), ("vec_descs", c_uint64), ("generic_descs", c_uint64),
                 ("plan_device_bytes", c_uint64), ("vec_chunks", c_uint32),
@@ -64,6 +68,10 @@ def kernels():
     lib.nixl_amd_copy_plan_create_indexed.argtypes = [c_uint64, c_uint64, c_void_p, c_uint64, c_uint64, c_void_p, c_size_t,
                                                       c_uint64, c_int, POINTER(CopyTuning), POINTER(c_void_p)]
     lib.nixl_amd_copy_plan_create_indexed.restype = c_int
+    lib.nixl_amd_copy_plan_create_indexed_runs.argtypes = [POINTER(CopyRun), c_size_t, c_void_p, POINTER(CopyRun), c_size_t,
+                                                           c_void_p, c_size_t, c_uint64, c_int, POINTER(CopyTuning),
+                                                           POINTER(c_void_p)]
+    lib.nixl_amd_copy_plan_create_indexed_runs.restype = c_int
     lib.nixl_amd_copy_plan_launch.argtypes = [c_void_p, c_void_p]
     lib.nixl_amd_copy_plan_destroy.argtypes = [c_void_p]
     lib.nixl_amd_copy_plan_query.argtypes = [c_void_p, POINTER(CopyPlanInfo)]
@@ -117,6 +125,7 @@ def ep_kernels():
 
 def kernel_symbols():
     return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create", "nixl_amd_copy_plan_create_indexed",
+                   "nixl_amd_copy_plan_create_indexed_runs",
                    "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
                    "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
 

@@ -737,14 +737,18 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
     const nixl_stride_dlist_t &rruns = *remote_side->descs.at(backend);
     auto req = std::make_unique<nixlXferReqH>(remote_side->remoteAgent, operation, lruns.getType(), rruns.getType());
 
-    // Both lists one run each (a pool, a staging buffer) and a backend that lowers index
-    // vectors itself: the descriptors are never written out here.  The request then carries
-    // no descriptor lists; its backend handle holds everything postXfer needs.
-    if (lruns.descCount() == 1 && rruns.descCount() == 1) {
+    // Both lists a few runs each (a pool in one or several regions, a staging buffer) and a
+    // backend that lowers index vectors itself: the descriptors are never written out here.
+    // The request then carries no descriptor lists; its backend handle holds everything
+    // postXfer needs.  Lists of many runs are cheaper to expand here than to search there.
+    constexpr int kIndexedRuns = 256;
+    if (lruns.descCount() >= 1 && rruns.descCount() >= 1 && lruns.descCount() <= kIndexedRuns &&
+        rruns.descCount() <= kIndexedRuns) {
         const nixlAgentData::engineSlot *slot = data->slotOf(backend->getType());
         if (slot && slot->prepIndexed && slot->engine == backend) {
             const nixl_status_t st = static_cast<nixl_status_t>(
-                slot->prepIndexed(backend, static_cast<int>(req->backendOp), &lruns[0], local_indices.data(), &rruns[0],
+                slot->prepIndexed(backend, static_cast<int>(req->backendOp), &lruns[0], static_cast<size_t>(lruns.descCount()),
+                                  local_indices.data(), &rruns[0], static_cast<size_t>(rruns.descCount()),
                                   remote_indices.data(), count, req->remoteAgent.c_str(), &req->backendHandle));
             if (st == NIXL_SUCCESS) {
                 req->engine = backend;

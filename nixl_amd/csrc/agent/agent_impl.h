@@ -185,10 +185,10 @@ public:
     const nixlAgentConfig config_;
 
     // Optional entry of a backend plugin ("nixl_hip_prep_xfer_indexed" in the HIP plugin): a
-    // request given as two index vectors into two single-run prepared lists, lowered by the
-    // backend itself.  Null for plugins that do not export it.
-    using prepIndexedFn = int (*)(nixlBackendEngine *, int, const nixlStrideDesc *, const int *, const nixlStrideDesc *,
-                                  const int *, size_t, const char *, nixlBackendReqH **);
+    // request given as two index vectors into two prepared lists (passed as their stride runs),
+    // lowered by the backend itself.  Null for plugins that do not export it.
+    using prepIndexedFn = int (*)(nixlBackendEngine *, int, const nixlStrideDesc *, size_t, const int *,
+                                  const nixlStrideDesc *, size_t, const int *, size_t, const char *, nixlBackendReqH **);
     struct engineSlot {
         nixlBackendEngine *engine = nullptr;
         const nixlLoadedPlugin *plugin = nullptr;

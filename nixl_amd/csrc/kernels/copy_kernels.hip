@@ -350,6 +350,45 @@ index_records_kernel(UniformRec *recs, const int32_t *src_index, const int32_t *
                              dst_base + static_cast<uint64_t>(dst_index[i]) * dst_stride};
 }
 
+// The same for lists of several runs (a pool registered as several regions): index i of a
+// list lies in the run r with first[r] <= i < first[r + 1], at base[r] + (i - first[r]) *
+// stride[r].  The run tables (at most kMaxIndexRuns entries a side) are staged in LDS and
+// searched by bisection.
+constexpr uint32_t kMaxIndexRuns = 256;
+
+__device__ __forceinline__ uint64_t
+run_address(const uint64_t *first, const uint64_t *base, const uint64_t *stride, uint32_t n_runs, uint64_t index) {
+    uint32_t lo = 0, hi = n_runs; // first[lo] <= index < first[hi] (first[n_runs] = infinity)
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) / 2;
+        if (first[mid] <= index) lo = mid;
+        else hi = mid;
+    }
+    return base[lo] + (index - first[lo]) * stride[lo];
+}
+
+__global__ void __launch_bounds__(256)
+index_records_runs_kernel(UniformRec *recs, const int32_t *src_index, const int32_t *dst_index, uint32_t n,
+                          const nixl_amd_copy_run_t *src_runs, uint32_t n_src, const nixl_amd_copy_run_t *dst_runs,
+                          uint32_t n_dst) {
+    __shared__ uint64_t first[2][kMaxIndexRuns], base[2][kMaxIndexRuns], stride[2][kMaxIndexRuns];
+    for (uint32_t r = threadIdx.x; r < n_src; r += blockDim.x) {
+        first[0][r] = src_runs[r].first_index;
+        base[0][r] = src_runs[r].base;
+        stride[0][r] = src_runs[r].stride;
+    }
+    for (uint32_t r = threadIdx.x; r < n_dst; r += blockDim.x) {
+        first[1][r] = dst_runs[r].first_index;
+        base[1][r] = dst_runs[r].base;
+        stride[1][r] = dst_runs[r].stride;
+    }
+    __syncthreads();
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        recs[i] = UniformRec{run_address(first[0], base[0], stride[0], n_src, static_cast<uint64_t>(src_index[i])),
+                             run_address(first[1], base[1], stride[1], n_dst, static_cast<uint64_t>(dst_index[i]))};
+}
+
 // Largest grid of one launch: HIP refuses grids of 2^32 or more threads, i.e. 2^22 workgroups of
 // 16 waves; a plan with more work than that goes out as several launches.
 constexpr uint32_t kMaxGrid = 1u << 21;
@@ -919,13 +958,13 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
 }
 
 int
-nixl_amd_copy_plan_create_indexed(uint64_t src_base,
-                                  uint64_t src_stride,
-                                  const int32_t *src_index,
-                                  uint64_t dst_base,
-                                  uint64_t dst_stride,
-                                  const int32_t *dst_index,
-                                  size_t n,
+nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
+                                       size_t n_src_runs,
+                                       const int32_t *src_index,
+                                       const nixl_amd_copy_run_t *dst_runs,
+                                       size_t n_dst_runs,
+                                       const int32_t *dst_index,
+                                       size_t n,
                                   uint64_t len,
                                   int device,
                                   const nixl_amd_copy_tuning_t *tuning,
@@ -945,10 +984,21 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
         (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16))
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: bad tuning value");
     const uint64_t chunk_bytes = static_cast<uint64_t>(kWaveSize) * upl * 16u;
-    if (len == 0 || len % chunk_bytes != 0 || ((src_base | dst_base | src_stride | dst_stride) & 127u) != 0 || src_base == 0 ||
-        dst_base == 0)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID,
-                             "plan_create_indexed: blocks must be whole chunks and start on 128-byte lines");
+    if (!src_runs || !dst_runs || n_src_runs == 0 || n_dst_runs == 0 || n_src_runs > kMaxIndexRuns || n_dst_runs > kMaxIndexRuns)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: between 1 and 256 runs a side");
+    bool src_all_dense = true, dst_all_dense = true;
+    for (int side = 0; side < 2; ++side) {
+        const nixl_amd_copy_run_t *runs = side ? dst_runs : src_runs;
+        const size_t n_runs = side ? n_dst_runs : n_src_runs;
+        for (size_t r = 0; r < n_runs; ++r) {
+            if (runs[r].base == 0 || ((runs[r].base | runs[r].stride) & 127u) != 0 || len == 0 || len % chunk_bytes != 0)
+                return nixl_amd_fail(NIXL_AMD_ERR_INVALID,
+                                     "plan_create_indexed: blocks must be whole chunks and start on 128-byte lines");
+            if (runs[r].first_index != (r ? runs[r - 1].first_index + runs[r - 1].count : 0))
+                return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: runs must follow each other from index 0");
+            (side ? dst_all_dense : src_all_dense) &= runs[r].stride == len;
+        }
+    }
     if (n >= (1ull << 31) || n * (len / chunk_bytes) >= (1ull << 32))
         return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create_indexed: request too large for 32-bit chunk index");
     int ndev = 0;
@@ -963,12 +1013,16 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
     const size_t index_bytes = n * sizeof(int32_t);
     void *staging = nullptr;
     size_t staging_cap = 0;
-    hipError_t e = upload_cache().get(device, 2 * index_bytes, &staging, &staging_cap);
+    const bool tables = n_src_runs > 1 || n_dst_runs > 1;
+    const size_t table_at = (2 * index_bytes + 15) & ~size_t(15); // the run tables follow the index vectors
+    const size_t table_bytes = tables ? (n_src_runs + n_dst_runs) * sizeof(nixl_amd_copy_run_t) : 0;
+    const size_t upload_bytes = tables ? table_at + table_bytes : 2 * index_bytes;
+    hipError_t e = upload_cache().get(device, upload_bytes, &staging, &staging_cap);
     if (e != hipSuccess)
         return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
     auto *up_src = static_cast<int32_t *>(staging), *up_dst = up_src + n;
     uint64_t regular = 0, src_follows = 0;
-    const int64_t dst_dense = dst_stride == len ? 1 : INT64_MIN, src_dense = src_stride == len ? 1 : INT64_MIN;
+    const int64_t dst_dense = dst_all_dense ? 1 : INT64_MIN, src_dense = src_all_dense ? 1 : INT64_MIN;
     int64_t prev_step = 0;
     for (size_t i = 0; i < n; ++i) {
         up_src[i] = src_index[i];
@@ -980,6 +1034,11 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
             src_follows += (static_cast<int64_t>(src_index[i]) - src_index[i - 1] == src_dense);
         }
     }
+    if (tables) {
+        auto *up_runs = reinterpret_cast<nixl_amd_copy_run_t *>(static_cast<uint8_t *>(staging) + table_at);
+        std::memcpy(up_runs, src_runs, n_src_runs * sizeof(nixl_amd_copy_run_t));
+        std::memcpy(up_runs + n_src_runs, dst_runs, n_dst_runs * sizeof(nixl_amd_copy_run_t));
+    }
     const bool scattered = !(n == 1 || 2 * regular >= n - 1);
     const bool sort = scattered && sort_scatter != 2 && 2 * src_follows >= n - 1 && n >= kSortWindow;
 
@@ -989,17 +1048,27 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
     plan->waves = waves;
     plan->swizzle = swizzle;
     plan->policy = nt ? nt : ((!scattered || sort) ? kPolNtSc1Nt : kPolPlainSc1Nt);
-    // one arena: the records, then the two index vectors the records are built from
+    // one arena: the records, then the two index vectors (and run tables) the records are built from
     const size_t rec_bytes = (n * sizeof(UniformRec) + 255) & ~size_t(255);
     hipStream_t up = nullptr;
-    e = arena_cache().get(device, rec_bytes + 2 * index_bytes, &plan->arena, &plan->arena_cap);
+    e = arena_cache().get(device, rec_bytes + upload_bytes, &plan->arena, &plan->arena_cap);
     if (e == hipSuccess) e = upload_stream(device, &up);
     auto *recs = static_cast<UniformRec *>(plan->arena);
     auto *dev_index = reinterpret_cast<int32_t *>(static_cast<uint8_t *>(plan->arena) + rec_bytes);
-    if (e == hipSuccess) e = hipMemcpyAsync(dev_index, staging, 2 * index_bytes, hipMemcpyHostToDevice, up);
+    if (e == hipSuccess) e = hipMemcpyAsync(dev_index, staging, upload_bytes, hipMemcpyHostToDevice, up);
     if (e == hipSuccess) {
-        hipLaunchKernelGGL(index_records_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, up, recs, dev_index,
-                           dev_index + n, static_cast<uint32_t>(n), src_base, src_stride, dst_base, dst_stride);
+        const dim3 grid(static_cast<uint32_t>((n + 255) / 256));
+        if (tables) {
+            const auto *dev_runs =
+                reinterpret_cast<const nixl_amd_copy_run_t *>(reinterpret_cast<const uint8_t *>(dev_index) + table_at);
+            hipLaunchKernelGGL(index_records_runs_kernel, grid, dim3(256), 0, up, recs, dev_index, dev_index + n,
+                               static_cast<uint32_t>(n), dev_runs, static_cast<uint32_t>(n_src_runs), dev_runs + n_src_runs,
+                               static_cast<uint32_t>(n_dst_runs));
+        } else {
+            hipLaunchKernelGGL(index_records_kernel, grid, dim3(256), 0, up, recs, dev_index, dev_index + n,
+                               static_cast<uint32_t>(n), src_runs[0].base, src_runs[0].stride, dst_runs[0].base,
+                               dst_runs[0].stride);
+        }
         e = hipGetLastError();
     }
     if (e == hipSuccess && sort) {
@@ -1014,7 +1083,7 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
         delete plan;
         return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan upload: ") + hipGetErrorString(e));
     }
-    plan->arena_bytes = rec_bytes + 2 * index_bytes;
+    plan->arena_bytes = rec_bytes + upload_bytes;
     plan->uniform_recs = recs;
     plan->chunks_per_rec = static_cast<uint32_t>(len / chunk_bytes);
     plan->n_uniform = static_cast<uint32_t>(n * plan->chunks_per_rec);
@@ -1028,6 +1097,22 @@ nixl_amd_copy_plan_create_indexed(uint64_t src_base,
     plan->info.uniform_workgroups = plan->uniform_wgs;
     *out = plan;
     return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_copy_plan_create_indexed(uint64_t src_base,
+                                  uint64_t src_stride,
+                                  const int32_t *src_index,
+                                  uint64_t dst_base,
+                                  uint64_t dst_stride,
+                                  const int32_t *dst_index,
+                                  size_t n,
+                                  uint64_t len,
+                                  int device,
+                                  const nixl_amd_copy_tuning_t *tuning,
+                                  nixl_amd_copy_plan_t **out) {
+    const nixl_amd_copy_run_t src{src_base, src_stride, 0, 0}, dst{dst_base, dst_stride, 0, 0};
+    return nixl_amd_copy_plan_create_indexed_runs(&src, 1, src_index, &dst, 1, dst_index, n, len, device, tuning, out);
 }
 
 int

@@ -489,9 +489,11 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
 
 nixl_status_t
 nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
-                               const nixlStrideDesc &local_run,
+                               const nixlStrideDesc *local_runs,
+                               size_t n_local_runs,
                                const int *local_indices,
-                               const nixlStrideDesc &remote_run,
+                               const nixlStrideDesc *remote_runs,
+                               size_t n_remote_runs,
                                const int *remote_indices,
                                size_t count,
                                const std::string &remote_agent,
@@ -500,27 +502,41 @@ nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
     reapRetired(false);
     if (!knowsAgent(remote_agent)) return NIXL_ERR_NOT_FOUND;
     if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
-    if (!local_indices || !remote_indices || count == 0) return NIXL_ERR_INVALID_PARAM;
-    if (local_run.start_idx != 0 || remote_run.start_idx != 0 || local_run.count == 0 || remote_run.count == 0)
+    if (!local_runs || !remote_runs || !local_indices || !remote_indices || count == 0) return NIXL_ERR_INVALID_PARAM;
+    constexpr size_t kMaxRuns = 256; // what the kernels library takes a side
+    if (n_local_runs == 0 || n_remote_runs == 0 || n_local_runs > kMaxRuns || n_remote_runs > kMaxRuns)
         return NIXL_ERR_NOT_SUPPORTED;
-    if (local_run.len != remote_run.len) {
-        NIXL_ERROR << "HIP backend: block length mismatch (local " << local_run.len << ", remote " << remote_run.len << ")";
-        return NIXL_ERR_INVALID_PARAM;
-    }
-    const auto *lmd = static_cast<const nixlHipMD *>(local_run.metadataP);
-    const auto *rmd = static_cast<const nixlHipMD *>(remote_run.metadataP);
-    auto span = [](const nixlStrideDesc &run) { return (run.count - 1) * run.stride + run.len; };
-    if (!lmd || !rmd || !lmd->contains(local_run.addr, span(local_run)) || !rmd->contains(remote_run.addr, span(remote_run))) {
-        NIXL_ERROR << "HIP backend: a prepared list reaches outside its registered region";
-        return NIXL_ERR_INVALID_PARAM;
-    }
+
+    // Every run inside its registered region, one block length and one device throughout;
+    // addresses of another process's regions become the addresses they are mapped at here.
+    const size_t len = local_runs[0].len;
     int device = -1;
-    for (const nixlHipMD *md : {lmd, rmd}) {
-        if (md->mem != VRAM_SEG) continue;
-        if (device < 0) device = md->device;
-        if (md->device != device) return NIXL_ERR_NOT_SUPPORTED;
+    const nixlHipMD *first_md = nullptr;
+    std::vector<nixl_amd_copy_run_t> tables[2];
+    size_t flat[2] = {0, 0};
+    for (int side = 0; side < 2; ++side) {
+        const nixlStrideDesc *runs = side ? remote_runs : local_runs;
+        const size_t n_runs = side ? n_remote_runs : n_local_runs;
+        tables[side].reserve(n_runs);
+        for (size_t r = 0; r < n_runs; ++r) {
+            const nixlStrideDesc &run = runs[r];
+            if (run.count == 0 || run.start_idx != flat[side]) return NIXL_ERR_NOT_SUPPORTED;
+            if (run.len != len) return NIXL_ERR_NOT_SUPPORTED; // mixed lengths: the descriptor path judges them
+            const auto *md = static_cast<const nixlHipMD *>(run.metadataP);
+            if (!md || !md->contains(run.addr, (run.count - 1) * run.stride + run.len)) {
+                NIXL_ERROR << "HIP backend: a prepared list reaches outside its registered region";
+                return NIXL_ERR_INVALID_PARAM;
+            }
+            if (!first_md) first_md = md;
+            if (md->mem == VRAM_SEG) {
+                if (device < 0) device = md->device;
+                if (md->device != device) return NIXL_ERR_NOT_SUPPORTED;
+            }
+            tables[side].push_back(nixl_amd_copy_run_t{md->here(run.addr), run.stride, flat[side], run.count});
+            flat[side] += run.count;
+        }
     }
-    if (device < 0) device = lmd->device;
+    if (device < 0) device = first_md->device;
     // every index must name a block of its list: one pass over each vector
     int lmin = local_indices[0], lmax = lmin, rmin = remote_indices[0], rmax = rmin;
     for (size_t i = 1; i < count; ++i) {
@@ -529,20 +545,20 @@ nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
         rmin = std::min(rmin, remote_indices[i]);
         rmax = std::max(rmax, remote_indices[i]);
     }
-    if (lmin < 0 || static_cast<size_t>(lmax) >= local_run.count || rmin < 0 || static_cast<size_t>(rmax) >= remote_run.count) {
+    if (lmin < 0 || static_cast<size_t>(lmax) >= flat[0] || rmin < 0 || static_cast<size_t>(rmax) >= flat[1]) {
         NIXL_ERROR << "HIP backend: index outside its prepared list";
         return NIXL_ERR_INVALID_PARAM;
     }
 
     const bool write = (operation == NIXL_WRITE);
-    const uint64_t la = lmd->here(local_run.addr), ra = rmd->here(remote_run.addr);
     auto req = std::make_unique<nixlHipReqH>();
     req->device = device;
-    req->bytes = count * local_run.len;
-    const int rc = write ? nixl_amd_copy_plan_create_indexed(la, local_run.stride, local_indices, ra, remote_run.stride,
-                                                             remote_indices, count, local_run.len, device, &tuning_, &req->plan)
-                         : nixl_amd_copy_plan_create_indexed(ra, remote_run.stride, remote_indices, la, local_run.stride,
-                                                             local_indices, count, local_run.len, device, &tuning_, &req->plan);
+    req->bytes = count * len;
+    const int src = write ? 0 : 1, dst = 1 - src;
+    const int *index_of[2] = {local_indices, remote_indices};
+    const int rc = nixl_amd_copy_plan_create_indexed_runs(tables[src].data(), tables[src].size(), index_of[src],
+                                                          tables[dst].data(), tables[dst].size(), index_of[dst], count, len,
+                                                          device, &tuning_, &req->plan);
     if (rc == NIXL_AMD_ERR_INVALID) return NIXL_ERR_NOT_SUPPORTED; // shape or alignment: the descriptor path handles it
     if (rc != NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
@@ -1105,18 +1121,20 @@ nixl_plugin_fini() {}
 extern "C" NIXL_PLUGIN_EXPORT int
 nixl_hip_prep_xfer_indexed(nixlBackendEngine *engine,
                            int operation,
-                           const nixlStrideDesc *local_run,
+                           const nixlStrideDesc *local_runs,
+                           size_t n_local_runs,
                            const int *local_indices,
-                           const nixlStrideDesc *remote_run,
+                           const nixlStrideDesc *remote_runs,
+                           size_t n_remote_runs,
                            const int *remote_indices,
                            size_t count,
                            const char *remote_agent,
                            nixlBackendReqH **handle) {
-    if (!engine || !local_run || !remote_run || !remote_agent || !handle) return NIXL_ERR_INVALID_PARAM;
+    if (!engine || !local_runs || !remote_runs || !remote_agent || !handle) return NIXL_ERR_INVALID_PARAM;
     try {
-        return static_cast<nixlHipEngine *>(engine)->prepXferIndexed(static_cast<nixl_xfer_op_t>(operation), *local_run,
-                                                                     local_indices, *remote_run, remote_indices, count,
-                                                                     remote_agent, *handle);
+        return static_cast<nixlHipEngine *>(engine)->prepXferIndexed(static_cast<nixl_xfer_op_t>(operation), local_runs,
+                                                                     n_local_runs, local_indices, remote_runs, n_remote_runs,
+                                                                     remote_indices, count, remote_agent, *handle);
     } catch (const std::exception &e) {
         NIXL_ERROR << "HIP backend: " << e.what();
         return NIXL_ERR_BACKEND;

@@ -165,19 +165,22 @@ public:
     nixl_status_t
     releaseReqH(nixlBackendReqH *handle) const override;
 
-    // prepXfer for a request given as two index vectors into two prepared lists that are one
-    // run each (local_run, remote_run: address, block length, stride, block count): the
-    // descriptors are never written out on the host; the records of the copy plan are built
-    // on the device from the index vectors.  No reference counterpart: the reference's agent
+    // prepXfer for a request given as two index vectors into two prepared lists, each list
+    // given as its stride runs (address, block length, stride, block count, first index; at
+    // most 256 runs a list, one block length throughout): the descriptors are never written
+    // out on the host; the records of the copy plan are built on the device from the index
+    // vectors and the run tables.  No reference counterpart: the reference's agent
     // expands the indices on the host (src/core/nixl_agent.cpp:799-857) before any backend sees
     // them.  NIXL_ERR_NOT_SUPPORTED means "take the ordinary path" (alignment, direction or
     // shape outside what the device lowering handles).  Reached through the C symbol
     // nixl_hip_prep_xfer_indexed, which an agent looks up in the plugin library.
     nixl_status_t
     prepXferIndexed(const nixl_xfer_op_t &operation,
-                    const nixlStrideDesc &local_run,
+                    const nixlStrideDesc *local_runs,
+                    size_t n_local_runs,
                     const int *local_indices,
-                    const nixlStrideDesc &remote_run,
+                    const nixlStrideDesc *remote_runs,
+                    size_t n_remote_runs,
                     const int *remote_indices,
                     size_t count,
                     const std::string &remote_agent,

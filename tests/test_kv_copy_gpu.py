@@ -259,6 +259,111 @@ def test_index_vectors_into_single_run_lists(hip_agent, cuda, op):
         h.release()
 
 
+def test_index_vectors_into_lists_of_several_runs(hip_agent, cuda):
+    """A pool registered as four separate allocations (what a pool must be for peers in other
+    processes, whose mappings stay under 2 GiB each) prepared as one list of several runs, and
+    a list whose second half has another stride (two runs in one region): requests are still
+    lowered on the device, now through the run tables.  Indices cross every run boundary;
+    checked against a per-block restatement in both directions; an index past the list is
+    refused."""
+    import torch
+    a = hip_agent
+    blk, per = 4096, 700
+    n_pool, half = 4 * per, 2 * per
+    rng = np.random.default_rng(11)
+    parts = [torch.from_numpy(rng.integers(0, 256, per * blk, dtype=np.uint8)).to(cuda) for _ in range(4)]
+    other = torch.from_numpy(rng.integers(0, 256, 3 * n_pool * blk, dtype=np.uint8)).to(cuda)
+    a.register_memory(parts + [other])
+    pool_descs = np.concatenate([_descs(p, np.arange(per) * blk, [blk] * per) for p in parts])
+    other_offs = np.concatenate([np.arange(half) * blk, half * blk + np.arange(n_pool - half) * 2 * blk])
+    h_local = a.prep_xfer_dlist("", pool_descs, "VRAM")
+    h_remote = a.prep_xfer_dlist("agent", _descs(other, other_offs, [blk] * n_pool), "VRAM")
+    assert 2 <= h_local.run_count() <= 4 and h_remote.run_count() == 2
+    # distinct blocks on both sides, so that the order of the copies does not matter
+    li = rng.permutation(n_pool)[:2500].astype(np.int32)
+    ri = rng.permutation(n_pool)[:2500].astype(np.int32)
+    edge = np.array([per - 1, per, 2 * per, n_pool - 1], dtype=np.int32)  # both sides of run boundaries, the last block
+    li = np.concatenate([edge, li[~np.isin(li, edge)]])[:2400]
+    ri = np.concatenate([edge[::-1], ri[~np.isin(ri, edge)]])[:2400]
+
+    for op in ("WRITE", "READ"):
+        pool_was = [p.cpu().numpy() for p in parts]
+        other_was = other.cpu().numpy()
+        req = a.make_prepped_xfer(op, h_local, li, h_remote, ri)
+        assert req.desc_count() == (len(li), len(li) * blk)
+        _wait(a, req)
+        for l, r in zip(li.tolist(), ri.tolist()):
+            part, off, ro = l // per, (l % per) * blk, int(other_offs[r])
+            if op == "WRITE":
+                other_was[ro:ro + blk] = pool_was[part][off:off + blk]
+            else:
+                pool_was[part][off:off + blk] = other_was[ro:ro + blk]
+        for p, w in zip(parts, pool_was):
+            assert np.array_equal(p.cpu().numpy(), w)
+        assert np.array_equal(other.cpu().numpy(), other_was)
+        req.release()
+    bad = ri.copy()
+    bad[3] = n_pool
+    with pytest.raises(Exception):
+        a.make_prepped_xfer("WRITE", h_local, li, h_remote, bad)
+    for h in (h_local, h_remote):
+        h.release()
+
+
+def test_run_tables_through_the_kernel_library(cuda):
+    """nixl_amd_copy_plan_create_indexed_runs called directly: three source runs with
+    different strides, two destination runs, 5000 random blocks (more than one bisection
+    depth, several sorting windows), against the descriptor oracle; run tables that do not
+    follow each other are refused."""
+    import torch
+    lib = _lib.kernels()
+    blk = 2048
+    rng = np.random.default_rng(12)
+    src_counts, src_strides = [1000, 1, 3000], [blk, blk, 2 * blk]
+    dst_counts, dst_strides = [2500, 2500], [blk, 3 * blk]
+    n_src, n_dst = sum(src_counts), sum(dst_counts)
+
+    def layout(counts, strides, at):
+        offs, table, first = [], [], 0
+        for c, st in zip(counts, strides):
+            table.append((at, st, first, c))
+            offs.extend(at + np.arange(c) * st)
+            at += c * st + 4096  # a gap between runs
+            first += c
+        return np.array(offs, dtype=np.int64), table, at
+
+    src_offs, src_table, end = layout(src_counts, src_strides, 0)
+    dst_offs, dst_table, end = layout(dst_counts, dst_strides, end)
+    host = rng.integers(0, 256, end, dtype=np.uint8)
+    mem = torch.from_numpy(host.copy()).to(cuda)
+    base = mem.data_ptr()
+    assert base % 128 == 0
+    n = 5000
+    si = rng.integers(0, n_src, n).astype(np.int32)  # a source block may be read twice
+    di = rng.permutation(n_dst)[:n].astype(np.int32)
+    si[:3] = [999, 1000, 1001]
+
+    def c_table(table):
+        arr = (_lib.CopyRun * len(table))()
+        for r, (at, st, first, c) in enumerate(table):
+            arr[r] = _lib.CopyRun(base + at, st, first, c)
+        return arr
+
+    plan = ctypes.c_void_p()
+    rc = lib.nixl_amd_copy_plan_create_indexed_runs(c_table(src_table), len(src_table), si.ctypes.data, c_table(dst_table),
+                                                    len(dst_table), di.ctypes.data, n, blk, 0, None, ctypes.byref(plan))
+    assert rc == 0, _lib.kernels_error()
+    _run_plan(torch, plan)
+    assert lib.nixl_amd_copy_plan_destroy(plan) == 0
+    want = ko.copy_descs(host, src_offs[si], dst_offs[di], [blk] * n)
+    assert np.array_equal(mem.cpu().numpy(), want)
+    broken = list(dst_table)
+    broken[1] = (broken[1][0], broken[1][1], broken[1][2] + 1, broken[1][3])
+    rc = lib.nixl_amd_copy_plan_create_indexed_runs(c_table(src_table), len(src_table), si.ctypes.data, c_table(broken),
+                                                    len(broken), di.ctypes.data, n, blk, 0, None, ctypes.byref(plan))
+    assert rc != 0 and "follow" in _lib.kernels_error()
+
+
 def test_write_zero_read_roundtrip_and_repost(hip_agent, cuda):
     # transfer_handler round trip (test/gtest/plugins/transfer_handler.h:182-209 with
     # memory_handler.h:42-58): WRITE, clear the source, READ back, expect the increasing
