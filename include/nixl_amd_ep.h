@@ -140,6 +140,56 @@ int
 nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status);
 
 /*
+ * Low-latency dispatch in two phases, with the receive side's bounded wait.  Arguments and
+ * results are those of nixl_amd_ep_ll_dispatch, plus:
+ *   phases   1: send phase only (the selections are published; `x` is not read yet)
+ *            2: receive phase only, for the send phase issued last on this workspace (same
+ *               arguments): rows, scales and metadata are produced
+ *            3: both.  This is the split behind return_recv_hook (csrc/nixl_ep.cpp:1125-1136).
+ *   timeout_us > 0: before it places anything, the receive phase waits for each source rank's
+ *            selections, at most that long per rank; a rank whose selections have not come is
+ *            taken as having sent nothing and mask_buffer[dst][rank] is set for every dst, as
+ *            the reference's receivers do (kernels/nixl_ep_ll.cu:316-340; the budget there is
+ *            in clock cycles, csrc/nixl_ep.cpp:49-52).  Needs mask_buffer.
+ *   dispatch_wait_recv_cost_stats  [R] int64 or NULL: ticks of the GPU's constant-rate wall
+ *            clock spent waiting for each source rank, accumulated (kernels/nixl_ep_ll.cu:349).
+ *   withhold_rank  -1, or a rank whose send phase leaves out the word its receivers wait for:
+ *            the way to make a time-out happen on one GPU, where every rank's selections are
+ *            otherwise there before the receive phase starts.  The wait then lasts the whole
+ *            time-out, which must be at most one second.
+ * On a stream, the kernels of the send phase are complete before the receive phase looks, so
+ * without a withheld rank the wait costs one small kernel and never spins.
+ */
+int
+nixl_amd_ep_ll_dispatch_phased(void *packed_recv_x,
+                               void *packed_recv_x_scales,
+                               int *packed_recv_src_info,
+                               int64_t *packed_recv_layout_range,
+                               int *packed_recv_count,
+                               int *mask_buffer,
+                               int *cumulative_local_expert_recv_stats,
+                               int64_t *dispatch_wait_recv_cost_stats,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const int *num_tokens_per_rank,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_fp8,
+                               int round_scale,
+                               int use_ue8m0,
+                               int *row_map,
+                               void *workspace,
+                               size_t workspace_bytes,
+                               int phases,
+                               uint64_t timeout_us,
+                               int withhold_rank,
+                               void *stream);
+
+/*
  * Low-latency dispatch that allocates nothing.  No counterpart in the reference; it is for
  * callers that cannot allocate device memory: code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc.  Arguments and results are those of
@@ -207,6 +257,38 @@ nixl_amd_ep_ll_combine(void *combined_x,
                        int num_experts,
                        int use_logfmt,
                        void *stream);
+
+/*
+ * Low-latency combine behind a bounded wait for the ranks whose expert outputs it reads
+ * (the receive side of kernels/nixl_ep_ll.cu:846-866).  rank_ready is [R] int32 in device or
+ * pinned host memory: word j is set (nonzero) by whoever produces `x` once the rows of rank j's
+ * experts are complete, e.g. by the last kernel of that rank's expert step on another stream.
+ * A rank whose word is still zero after timeout_us (1 us .. 1 s) is entered in
+ * mask_buffer[dst][j] for every dst and its experts drop out of the sums, here and in later
+ * calls, exactly as for a rank masked by hand.  combine_wait_recv_cost_stats: [R] int64 or
+ * NULL, wall-clock ticks waited per rank, accumulated.  The caller clears rank_ready.
+ */
+int
+nixl_amd_ep_ll_combine_elastic(void *combined_x,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const float *topk_weights,
+                               const int *src_info,
+                               const int64_t *layout_range,
+                               int *mask_buffer,
+                               const int *rank_ready,
+                               int64_t *combine_wait_recv_cost_stats,
+                               const int *num_tokens_per_rank,
+                               const int *row_map,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_logfmt,
+                               uint64_t timeout_us,
+                               void *stream);
 
 /*
  * Token counts per rank and per expert and the token-in-rank matrix, for all source ranks.

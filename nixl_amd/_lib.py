@@ -92,6 +92,9 @@ _EP_SIGS = {
     "nixl_amd_ep_ll_dispatch": [c_void_p] * 10 + [c_int] * 9 + [c_void_p, c_void_p, c_size_t, c_void_p],
     "nixl_amd_ep_ll_route_dispatch": [c_void_p] * 12 + [c_int] * 9 + [c_void_p, c_void_p, c_size_t, c_void_p],
     "nixl_amd_ep_ll_dispatch_status": [c_void_p, c_void_p, POINTER(c_int)],
+    "nixl_amd_ep_ll_dispatch_phased": [c_void_p] * 11 + [c_int] * 9 + [c_void_p, c_void_p, c_size_t, c_int, c_uint64, c_int,
+                                                                      c_void_p],
+    "nixl_amd_ep_ll_combine_elastic": [c_void_p] * 11 + [c_int] * 7 + [c_uint64, c_void_p],
     "nixl_amd_ep_ll_dispatch_static": [c_void_p] * 10 + [c_int] * 9 + [c_void_p, c_void_p],
     "nixl_amd_ep_ll_combine": [c_void_p] * 9 + [c_int] * 7 + [c_void_p],
     "nixl_amd_ep_get_dispatch_layout": [c_void_p] * 4 + [c_int] * 4 + [c_void_p],

@@ -3,25 +3,28 @@
 //
 // What the reference does per rank with three passes over the payload (cast into a send
 // buffer, K message copies into per-(expert, source rank) receive slots, repack into the
-// per-expert contiguous output; kernels/nixl_ep_ll.cu:134-393) is done here in two
-// launches that touch the payload once, because every "remote" slot is an address in the
-// same HBM:
+// per-expert contiguous output; kernels/nixl_ep_ll.cu:134-393) is done here in launches
+// that touch the payload once, because every "remote" slot is an address in the same HBM:
 //   1. ll_bits_kernel      one workgroup per 64 consecutive tokens of a rank builds, in LDS,
 //                          one 64-bit word per expert (bit j: token j of the group selected the
 //                          expert) and writes it to bits[e][rank][group]: every word has one
 //                          writer, so nothing is cleared beforehand and nothing is atomic in
 //                          global memory.  With logits instead of top-k indices the same
-//                          kernel does the routing first (a wave per token, four tokens per
-//                          wave) and writes the indices and weights out as well.
+//                          kernel does the routing first (a wave per token) and writes the
+//                          indices and weights out as well.  This is the send phase.
+//   1b. ll_arrival_kernel  only for calls with a time-out: the receive side's bounded wait for
+//                          each source rank's bits; a late rank loses its bits and is masked.
 //   2. ll_dispatch_kernel  one workgroup per token reads its bf16 row once and, while the row
 //                          travels, counts for each of its K experts the bits in front of its
 //                          own (tokens of lower ranks, then lower tokens of its rank): that is
 //                          its row inside the expert.  It quantises the row in registers and
 //                          writes it straight to its K final rows of packed_recv_x, plus
-//                          src_info and the scales in their column-major place.  Workgroup e
+//                          src_info and one row of inverse scales per token.  Workgroup e
 //                          also turns expert e's bits into layout_range, recv_count and the
 //                          statistics.
-// Step 1 moves 0.3 MB; step 2 moves the payload.
+//   3. ll_scales_kernel    fp8 only: moves the per-token scales into their column-major place
+//                          per expert, 64 rows at a time through LDS.
+// Step 1 moves 0.3 MB, step 3 the scales (twice 16 MB at 32 x 128 x 7168, top-8); step 2 moves the payload.
 // The order this produces is the canonical one among those the reference's atomics allow:
 // segments by source rank ascending, tokens ascending inside a segment.
 //
@@ -71,7 +74,8 @@ wave_sum(int v) {
 
 struct BitsArgs {
     unsigned long long *bits; // [E][R][Wr]
-    int *group_status; // [R][Wr]: 1 if a token of the group names an expert twice
+    int *group_status; // [R][Wr]: bit 0: a token of the group names an expert twice; bits 1..: arrival stamp
+    int *header; // workspace header; [1] receives the arrival stamp of this call
     int32_t *topk_idx; // [R][T][K]; written when routing, read otherwise
     float *topk_weights; // [R][T][K], routing only
     const float *logits; // [R][T][E], routing only
@@ -79,6 +83,8 @@ struct BitsArgs {
     const int *mask;
     LlDims d;
     int Wr; // words (groups of 64 tokens) per rank
+    int stamp; // arrival stamp of this call (0 when nobody checks arrivals)
+    int withhold_rank; // this rank's groups leave their stamp out (its counts "never arrive"), or -1
 };
 
 // Index path: grid = R * Wr workgroups, one per word (64 tokens).  Routing path: grid =
@@ -159,8 +165,74 @@ ll_bits_kernel(BitsArgs a) {
     } else {
         for (int e = tid; e < d.E; e += n_threads)
             a.bits[e * W + blockIdx.x] = words[e];
-        if (tid == 0) a.group_status[blockIdx.x] = dup;
+        // The stamp goes out with the flag, after this group's words: what a receiver that
+        // checks arrivals (ll_arrival_kernel) waits for.
+        if (tid == 0 && r != a.withhold_rank) a.group_status[blockIdx.x] = dup | (a.stamp << 1);
+        if (tid == 0 && blockIdx.x == 0) a.header[1] = a.stamp;
     }
+}
+
+// ---- 1b. arrival check (the receive side's bounded wait) -----------------------------------------
+//
+// The reference's receivers spin on each source rank's count with a cycle budget; when it
+// runs out they set mask_buffer[src] and take the rank as having sent nothing
+// (kernels/nixl_ep_ll.cu:316-340).  Here the counts are the selection bits, and a group's bits
+// have arrived when its flag word carries this call's stamp.  One workgroup, a lane per source
+// rank: wait (at most `timeout` ticks of the constant-rate wall clock) until every group of the
+// rank is stamped; a rank that is not loses its bits (so the kernels behind this one place and
+// count nothing of it) and is masked for every destination.  Ranks whose stamps are there,
+// which is every rank unless the send side was told to withhold one, cost one pass over their
+// flags.
+struct ArrivalArgs {
+    unsigned long long *bits; // [E][R][Wr]
+    int *group_status; // [R][Wr]
+    const int *header; // [1]: the stamp to wait for
+    int *mask; // [R][R]
+    long long *wait_stats; // [R] ticks waited per source rank, accumulated; may be null
+    long long timeout; // wall-clock ticks
+    long long max_polls; // second bound of the wait, should the clock not advance
+    int R, E, Wr;
+};
+
+constexpr int kArrivalThreads = 256;
+
+__global__ void __launch_bounds__(kArrivalThreads)
+ll_arrival_kernel(ArrivalArgs a) {
+    extern __shared__ int late[]; // [R]
+    const int stamp = a.header[1];
+    int any_late = 0;
+    for (int r = threadIdx.x; r < a.R; r += kArrivalThreads) {
+        const int *flags = a.group_status + r * a.Wr;
+        // the usual case first: everything is there, one pass of independent loads and no clock
+        bool here = true;
+        for (int w = 0; w < a.Wr; ++w)
+            here &= (__hip_atomic_load(flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 1) == stamp;
+        long long waited = 0;
+        if (!here) {
+            const long long start = wall_clock64();
+            long long polls = 0;
+            do {
+                here = true;
+                for (int w = 0; w < a.Wr; ++w)
+                    here &= (__hip_atomic_load(flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 1) == stamp;
+                waited = wall_clock64() - start;
+            } while (!here && waited <= a.timeout && ++polls < a.max_polls);
+        }
+        late[r] = here ? 0 : 1;
+        if (a.wait_stats && waited) a.wait_stats[r] += waited;
+        if (!here) {
+            any_late = 1;
+            for (int dst = 0; dst < a.R; ++dst)
+                a.mask[dst * a.R + r] = 1;
+            for (int w = 0; w < a.Wr; ++w)
+                a.group_status[r * a.Wr + w] = 0;
+        }
+    }
+    if (!__syncthreads_or(any_late)) return;
+    // bits of the late ranks: every thread takes words of every expert
+    const int words = a.R * a.Wr;
+    for (int i = threadIdx.x; i < a.E * words; i += kArrivalThreads)
+        if (late[(i % words) / a.Wr]) a.bits[i] = 0ull;
 }
 
 // ---- 2. cast + scatter ----------------------------------------------------------------------------
@@ -221,7 +293,7 @@ __device__ __forceinline__ void
 reduce_status(const DispatchArgs &a, int lane) {
     int any = 0;
     for (int g = lane; g < a.n_flags; g += kWaveSize)
-        any |= a.group_status[g];
+        any |= a.group_status[g] & 1;
     any = wave_sum(any);
     if (lane == 0) a.status[0] = any ? NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT : 0;
 }
@@ -590,6 +662,36 @@ ll_combine_kernel(CombineArgs a) {
     st16_nt(reinterpret_cast<uint4 *>(a.combined + (static_cast<size_t>(r) * d.T + t) * d.H) + col, out);
 }
 
+// The combine side of the bounded wait (kernels/nixl_ep_ll.cu:846-866): a receiver waits for
+// the flag of each rank whose experts' rows it is about to read and masks a rank whose flag
+// does not come.  Here a flag is a word the caller's expert step sets when the rank's rows
+// are complete; one workgroup, a lane per rank.
+struct ReadyArgs {
+    const int *ready; // [R], nonzero: the rank's expert outputs are there
+    int *mask; // [R][R]
+    long long *wait_stats; // [R], may be null
+    long long timeout; // wall-clock ticks
+    long long max_polls; // second bound of the wait, should the clock not advance
+    int R;
+};
+
+__global__ void __launch_bounds__(kArrivalThreads)
+ll_ready_kernel(ReadyArgs a) {
+    for (int r = threadIdx.x; r < a.R; r += kArrivalThreads) {
+        const long long start = wall_clock64();
+        long long waited = 0, polls = 0;
+        bool here;
+        do {
+            here = __hip_atomic_load(a.ready + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0;
+            waited = wall_clock64() - start;
+        } while (!here && waited <= a.timeout && ++polls < a.max_polls);
+        if (a.wait_stats) a.wait_stats[r] += waited;
+        if (!here)
+            for (int dst = 0; dst < a.R; ++dst)
+                a.mask[dst * a.R + r] = 1;
+    }
+}
+
 // Four values per thread through the same routine as the dispatch kernel, so that a NaN's
 // neighbours are covered too; the last thread pads with zeros.
 __global__ void
@@ -708,7 +810,16 @@ struct LlDispatchCall {
     void *workspace;
     size_t workspace_bytes;
     void *stream;
+    // phased / elastic calls only
+    int phases = 3; // bit 0: send (selection bits and their arrival stamps), bit 1: receive (everything else)
+    uint64_t timeout_us = 0; // > 0: the receive phase checks arrivals first
+    int withhold_rank = -1;
+    int64_t *wait_stats = nullptr;
+    int *mask_rw = nullptr; // the mask buffer again, writable: late ranks are entered here
 };
+
+// Stamps of calls that check arrivals: 1 .. 2^30 - 1, never 0 (the stamp of calls that do not).
+std::atomic<uint32_t> g_arrival_stamp{0};
 
 template<bool ROUTE>
 void
@@ -751,6 +862,13 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
     if (static_cast<size_t>(d.R) * sizeof(int) > 32 * 1024) return bad(NIXL_AMD_ERR_TOO_LARGE, "more than 8192 ranks");
     if (c.logits && (d.E > kRouterMaxPerLane * kWaveSize || d.K > d.E))
         return bad(NIXL_AMD_ERR_INVALID, "routing needs num_experts <= 1024 and num_topk <= num_experts");
+    if (c.phases < 1 || c.phases > 3) return bad(NIXL_AMD_ERR_INVALID, "phases must be 1 (send), 2 (receive) or 3 (both)");
+    if (c.withhold_rank < -1 || c.withhold_rank >= d.R) return bad(NIXL_AMD_ERR_INVALID, "withhold_rank is not a rank");
+    if (c.timeout_us > 0 && !c.mask_rw) // the reference traps when a wait runs out without a mask buffer
+        return bad(NIXL_AMD_ERR_INVALID, "a time-out needs a mask buffer to record late ranks in");
+    if (c.withhold_rank >= 0 && (c.timeout_us == 0 || c.timeout_us > 1000000))
+        return bad(NIXL_AMD_ERR_INVALID, "a withheld rank is waited for: the time-out must be between 1 us and 1 s");
+    if (c.timeout_us > (1ull << 40)) return bad(NIXL_AMD_ERR_INVALID, "time-out too long");
 
     hipStream_t s = static_cast<hipStream_t>(c.stream);
     const int Wr = (d.T + kGroupTokens - 1) / kGroupTokens;
@@ -763,10 +881,16 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
     auto *token_scales =
         reinterpret_cast<float *>(base + off_bits + (static_cast<size_t>(d.E) * groups * sizeof(unsigned long long) + 255) / 256 * 256);
 
-    if (groups > 0) {
+    if (groups > 0 && (c.phases & 1)) {
         BitsArgs b{};
         b.bits = bits;
         b.group_status = group_status;
+        b.header = status;
+        b.withhold_rank = c.withhold_rank;
+        if (c.timeout_us > 0) {
+            const uint32_t n = g_arrival_stamp.fetch_add(1, std::memory_order_relaxed) % 0x3fffffffu;
+            b.stamp = static_cast<int>(n + 1);
+        }
         b.topk_idx = c.topk_idx;
         b.topk_weights = c.topk_weights;
         b.logits = c.logits;
@@ -780,6 +904,28 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
                               s, b);
         else
             launch_bits<false>(1, dim3(static_cast<unsigned>(groups)), lds, s, b);
+        HIP_TRY(hipGetLastError());
+    }
+    if (!(c.phases & 2)) return NIXL_AMD_OK;
+
+    if (groups > 0 && c.timeout_us > 0) {
+        int dev = 0, khz = 0;
+        HIP_TRY(hipGetDevice(&dev));
+        HIP_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+        if (khz <= 0) return bad(NIXL_AMD_ERR_HIP, "the device reports no wall clock rate");
+        ArrivalArgs w{};
+        w.bits = bits;
+        w.group_status = group_status;
+        w.header = status;
+        w.mask = c.mask_rw;
+        w.wait_stats = reinterpret_cast<long long *>(c.wait_stats);
+        w.timeout = static_cast<long long>(c.timeout_us * static_cast<uint64_t>(khz) / 1000u);
+        // a poll is a round trip to memory (hundreds of ns): 16 a microsecond only happen if the clock stands still
+        w.max_polls = static_cast<long long>(c.timeout_us) * 16 + 1024;
+        w.R = d.R;
+        w.E = d.E;
+        w.Wr = Wr;
+        hipLaunchKernelGGL(ll_arrival_kernel, dim3(1), dim3(kArrivalThreads), static_cast<size_t>(d.R) * sizeof(int), s, w);
         HIP_TRY(hipGetLastError());
     }
 
@@ -914,6 +1060,47 @@ nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status)
 }
 
 int
+nixl_amd_ep_ll_dispatch_phased(void *packed_recv_x,
+                               void *packed_recv_x_scales,
+                               int *packed_recv_src_info,
+                               int64_t *packed_recv_layout_range,
+                               int *packed_recv_count,
+                               int *mask_buffer,
+                               int *cumulative_local_expert_recv_stats,
+                               int64_t *dispatch_wait_recv_cost_stats,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const int *num_tokens_per_rank,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_fp8,
+                               int round_scale,
+                               int use_ue8m0,
+                               int *row_map,
+                               void *workspace,
+                               size_t workspace_bytes,
+                               int phases,
+                               uint64_t timeout_us,
+                               int withhold_rank,
+                               void *stream) {
+    LlDispatchCall c{packed_recv_x, packed_recv_x_scales, packed_recv_src_info, packed_recv_layout_range,
+                     packed_recv_count, mask_buffer, cumulative_local_expert_recv_stats, x,
+                     const_cast<int32_t *>(topk_idx), nullptr, nullptr, num_tokens_per_rank, num_tokens, hidden,
+                     num_max_dispatch_tokens_per_rank, num_topk, num_ranks, num_experts, use_fp8, round_scale,
+                     use_ue8m0, row_map, workspace, workspace_bytes, stream};
+    c.phases = phases;
+    c.timeout_us = timeout_us;
+    c.withhold_rank = withhold_rank;
+    c.wait_stats = dispatch_wait_recv_cost_stats;
+    c.mask_rw = mask_buffer;
+    return ll_dispatch_impl("ll_dispatch_phased", c);
+}
+
+int
 nixl_amd_ep_ll_dispatch_static(void *packed_recv_x,
                                void *packed_recv_x_scales,
                                int *packed_recv_src_info,
@@ -999,6 +1186,50 @@ nixl_amd_ep_ll_combine(void *combined_x,
         hipLaunchKernelGGL(ll_combine_kernel<false>, grid, dim3(wg), 0, static_cast<hipStream_t>(stream), a);
     HIP_TRY(hipGetLastError());
     return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_ep_ll_combine_elastic(void *combined_x,
+                               const void *x,
+                               const int32_t *topk_idx,
+                               const float *topk_weights,
+                               const int *src_info,
+                               const int64_t *layout_range,
+                               int *mask_buffer,
+                               const int *rank_ready,
+                               int64_t *combine_wait_recv_cost_stats,
+                               const int *num_tokens_per_rank,
+                               const int *row_map,
+                               int num_tokens,
+                               int hidden,
+                               int num_max_dispatch_tokens_per_rank,
+                               int num_topk,
+                               int num_ranks,
+                               int num_experts,
+                               int use_logfmt,
+                               uint64_t timeout_us,
+                               void *stream) {
+    if (!mask_buffer || !rank_ready)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_combine_elastic: mask buffer and ready flags are required");
+    if (timeout_us == 0 || timeout_us > 1000000)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_combine_elastic: the time-out must be between 1 us and 1 s");
+    if (num_ranks <= 0 || num_ranks > 8192) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_combine_elastic: bad number of ranks");
+    int dev = 0, khz = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    if (khz <= 0) return nixl_amd_fail(NIXL_AMD_ERR_HIP, "ll_combine_elastic: the device reports no wall clock rate");
+    ReadyArgs w{};
+    w.ready = rank_ready;
+    w.mask = mask_buffer;
+    w.wait_stats = reinterpret_cast<long long *>(combine_wait_recv_cost_stats);
+    w.timeout = static_cast<long long>(timeout_us * static_cast<uint64_t>(khz) / 1000u);
+    w.max_polls = static_cast<long long>(timeout_us) * 16 + 1024;
+    w.R = num_ranks;
+    hipLaunchKernelGGL(ll_ready_kernel, dim3(1), dim3(kArrivalThreads), 0, static_cast<hipStream_t>(stream), w);
+    HIP_TRY(hipGetLastError());
+    return nixl_amd_ep_ll_combine(combined_x, x, topk_idx, topk_weights, src_info, layout_range, mask_buffer, num_tokens_per_rank,
+                                  row_map, num_tokens, hidden, num_max_dispatch_tokens_per_rank, num_topk, num_ranks, num_experts,
+                                  use_logfmt, stream);
 }
 
 int

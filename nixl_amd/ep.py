@@ -105,10 +105,18 @@ class Buffer:
         """Reference: buffer.py:249-275."""
         return Config(Buffer.num_sms)
 
-    def __init__(self, num_ranks, low_latency_mode=True, device="cuda:0"):
+    def __init__(self, num_ranks, low_latency_mode=True, device="cuda:0", timeout_ms=None):
+        """timeout_ms (reference: buffer.py:65,80-83; 30 s there): budget of the receive side's
+        bounded waits in low-latency mode.  None (the default here) leaves the waits out: on
+        one GPU every rank's data is in place before a receiver looks, so they only matter to
+        callers that exercise the time-out -> mask path."""
         self.num_ranks = int(num_ranks)
         self.low_latency_mode = low_latency_mode
         self.device = torch.device(device)
+        self.timeout_ms = timeout_ms
+        # Fault injection for tests of that path: this rank's send phase leaves out the word
+        # its receivers wait for, so that their wait runs out (one-shot knob, -1 = off).
+        self.withhold_rank = -1
         self._k = _lib.ep_kernels()
         self.mask_buffer = torch.zeros((self.num_ranks, self.num_ranks), dtype=torch.int32, device=self.device)
         self._mask_active = False
@@ -286,8 +294,11 @@ class Buffer:
         event, hook) with handle = (src_info, layout_range, num_max_dispatch_tokens_per_rank,
         hidden).  `num_tokens_per_rank` ([R] int32 device tensor) is an extension for ragged
         worlds: rank r only owns the first num_tokens_per_rank[r] rows of x[r].
-        dispatch_wait_recv_cost_stats (cycles spent waiting for each source rank's data,
-        nixl_ep_ll.cu:349-350) is left as it is: nothing here waits for another rank.
+        With a `timeout_ms` on the buffer the receive side waits (bounded) for every source
+        rank's selections and masks a rank that is late; dispatch_wait_recv_cost_stats ([R]
+        int64, nixl_ep_ll.cu:349-350) then accumulates the wall-clock ticks waited per rank.
+        return_recv_hook=True issues the send phase only; the hook issues the receive phase
+        (`x` must stay as it is until then: the rows are read by the receive phase).
         `check_duplicates` waits for the kernels and raises if a token named an expert twice
         (the reference delivers such a token twice, nixl_ep_ll.cu:186-190; here it arrives once).
         """
@@ -295,7 +306,8 @@ class Buffer:
             raise EPError("topk_idx must be a contiguous [R, T, K] int32 tensor")
         return self._ll_dispatch(x, topk_idx, None, topk_idx.shape[2], num_max_dispatch_tokens_per_rank, num_experts,
                                  cumulative_local_expert_recv_stats, use_fp8, round_scale, use_ue8m0, async_finish,
-                                 return_recv_hook, num_tokens_per_rank, check_duplicates)[2:]
+                                 return_recv_hook, num_tokens_per_rank, check_duplicates,
+                                 dispatch_wait_recv_cost_stats)[2:]
 
     def route_dispatch(self, x, logits, num_topk, num_max_dispatch_tokens_per_rank,
                        cumulative_local_expert_recv_stats=None, use_fp8=True, round_scale=False, use_ue8m0=False,
@@ -310,7 +322,8 @@ class Buffer:
                                  return_recv_hook, num_tokens_per_rank, False)
 
     def _ll_dispatch(self, x, topk_idx, logits, K, num_max_dispatch_tokens_per_rank, num_experts, stats, use_fp8,
-                     round_scale, use_ue8m0, async_finish, return_recv_hook, num_tokens_per_rank, check_duplicates):
+                     round_scale, use_ue8m0, async_finish, return_recv_hook, num_tokens_per_rank, check_duplicates,
+                     wait_stats=None):
         if not self.low_latency_mode:
             raise EPError("dispatch() requires low-latency mode (low_latency_mode=True)")
         if x.dim() != 3 or not x.is_contiguous() or x.dtype != torch.bfloat16:
@@ -343,7 +356,29 @@ class Buffer:
         tail = (_ptr(num_tokens_per_rank), T, H, num_max_dispatch_tokens_per_rank, K, R, num_experts, int(use_fp8),
                 int(round_scale), int(use_ue8m0), _ptr(row_map), _ptr(ws), ws.numel(), _stream())
         topk_weights = None
-        if logits is None:
+        hook = None
+        phased = logits is None and (self.timeout_ms is not None or return_recv_hook)
+        if phased:
+            if wait_stats is not None and (wait_stats.dtype != torch.int64 or wait_stats.numel() < R):
+                raise EPError("dispatch_wait_recv_cost_stats must hold R int64 values")
+            timeout_us = 0 if self.timeout_ms is None else max(int(self.timeout_ms * 1000), 1)
+            withhold, self.withhold_rank = self.withhold_rank, -1
+            if timeout_us:
+                self._mask_active = True  # the kernels may enter a late rank
+            mask = _ptr(self.mask_buffer) if timeout_us else self._mask_ptr()
+
+            def issue(phases):
+                return self._k.nixl_amd_ep_ll_dispatch_phased(
+                    *head[:5], mask, _ptr(stats), _ptr(wait_stats), _ptr(x), _ptr(topk_idx), *tail[:-1], phases,
+                    timeout_us, withhold, _stream())
+
+            if return_recv_hook:
+                rc = issue(1)
+                keep = (x, topk_idx, ws, stats, wait_stats, num_tokens_per_rank)  # alive until the hook has run
+                hook = lambda keep=keep: _check(issue(2), "low_latency_dispatch (receive phase)")  # noqa: E731
+            else:
+                rc = issue(3)
+        elif logits is None:
             rc = self._k.nixl_amd_ep_ll_dispatch(*head, _ptr(topk_idx), *tail)
         else:
             topk_idx = torch.empty((R, T, K), dtype=topk_idx_t, device=dev)
@@ -362,7 +397,8 @@ class Buffer:
         handle = DispatchHandle((packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, H))
         handle.row_map = row_map
         recv = (packed_recv_x, scales.transpose(2, 3)) if use_fp8 else packed_recv_x
-        hook = (lambda: None) if return_recv_hook else None
+        if return_recv_hook and hook is None:
+            hook = lambda: None  # noqa: E731  (routing dispatch: issued whole)
         return topk_idx, topk_weights, recv, packed_recv_count, handle, EventOverlap(event), hook
 
     def dispatch(self, *args, **kwargs):
@@ -370,11 +406,15 @@ class Buffer:
 
     def low_latency_combine(self, x, topk_idx, topk_weights, handle, use_logfmt=False, zero_copy=False,
                             async_finish=False, return_recv_hook=False, out=None,
-                            combine_wait_recv_cost_stats=None, num_tokens_per_rank=None):
+                            combine_wait_recv_cost_stats=None, num_tokens_per_rank=None, rank_ready=None):
         """Reference: buffer.py:443-520, csrc/nixl_ep.cpp:1145-1246.
 
         x [R, El, N, H] bf16 expert outputs, topk_idx / topk_weights [R, T, K].  Returns
-        (combined_x [R, T, H] bf16, event, hook)."""
+        (combined_x [R, T, H] bf16, event, hook).  rank_ready ([R] int32, an extension; needs a
+        `timeout_ms` on the buffer): word j is set by the producer of `x` when rank j's rows are
+        complete; combine waits for it (bounded) and masks a rank whose word stays zero, as the
+        reference's receivers do with a rank whose flag never comes (nixl_ep_ll.cu:846-866);
+        combine_wait_recv_cost_stats ([R] int64) accumulates the ticks waited."""
         if not self.low_latency_mode:
             raise EPError("combine() requires low-latency mode (low_latency_mode=True)")
         src_info, layout_range, max_tok, hidden = handle
@@ -389,10 +429,25 @@ class Buffer:
         R, T, K = topk_idx.shape
         num_experts = x.shape[1] * R
         combined = out if out is not None else torch.empty((R, T, hidden), dtype=torch.bfloat16, device=x.device)
-        rc = self._k.nixl_amd_ep_ll_combine(
-            _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
-            self._mask_ptr(), _ptr(num_tokens_per_rank), _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K,
-            R, num_experts, int(use_logfmt), _stream())
+        if rank_ready is not None:
+            if self.timeout_ms is None:
+                raise EPError("rank_ready needs a buffer created with timeout_ms")
+            if rank_ready.dtype != torch.int32 or rank_ready.numel() < R:
+                raise EPError("rank_ready must hold R int32 values")
+            stats = combine_wait_recv_cost_stats
+            if stats is not None and (stats.dtype != torch.int64 or stats.numel() < R):
+                raise EPError("combine_wait_recv_cost_stats must hold R int64 values")
+            self._mask_active = True
+            rc = self._k.nixl_amd_ep_ll_combine_elastic(
+                _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
+                _ptr(self.mask_buffer), _ptr(rank_ready), _ptr(stats), _ptr(num_tokens_per_rank),
+                _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K, R, num_experts, int(use_logfmt),
+                max(int(self.timeout_ms * 1000), 1), _stream())
+        else:
+            rc = self._k.nixl_amd_ep_ll_combine(
+                _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
+                self._mask_ptr(), _ptr(num_tokens_per_rank), _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K,
+                R, num_experts, int(use_logfmt), _stream())
         _check(rc, "low_latency_combine")
         event = None
         if async_finish:

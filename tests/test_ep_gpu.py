@@ -721,6 +721,152 @@ def test_ll_dispatch_without_tokens(cuda):
     assert (got["recv_x"] == 0x55).all()
 
 
+# ---- the receive side's bounded wait: time-out -> mask (kernels/nixl_ep_ll.cu:316-340, 846-866) -----
+
+def raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, phases=(3,), timeout_us=0, withhold=-1, wait=None, fill=0x55):
+    """nixl_amd_ep_ll_dispatch_phased through the C ABI on buffers pre-filled with `fill`; one
+    call per entry of `phases`, on the same buffers and workspace."""
+    k = _lib.ep_kernels()
+    R, T, H = x.shape
+    K = topk.shape[2]
+    El, N = E // R, R * M
+    xd, td = x.to(cuda), torch.from_numpy(np.ascontiguousarray(topk, dtype=np.int32)).to(cuda)
+    recv_x = torch.full((R, El, N, H * (1 if use_fp8 else 2)), fill, dtype=torch.uint8, device=cuda)
+    scales = torch.full((R, El, H // 128, N, 4), fill, dtype=torch.uint8, device=cuda) if use_fp8 else None
+    src_info = torch.full((R, El, N, 4), fill, dtype=torch.uint8, device=cuda)
+    layout = torch.zeros((R, El, R), dtype=torch.int64, device=cuda)
+    count = torch.zeros((R, El), dtype=torch.int32, device=cuda)
+    ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K, H), dtype=torch.uint8, device=cuda)
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    rcs = []
+    for ph in phases:
+        rcs.append(k.nixl_amd_ep_ll_dispatch_phased(p(recv_x), p(scales), p(src_info), p(layout), p(count), p(mask), None, p(wait),
+                                                    p(xd), p(td), None, T, H, M, K, R, E, int(use_fp8), 0, 0, None, p(ws),
+                                                    ws.numel(), ph, timeout_us, withhold, None))
+    torch.cuda.synchronize()
+    status = ctypes.c_int(-1)
+    assert k.nixl_amd_ep_ll_dispatch_status(p(ws), None, ctypes.byref(status)) == 0
+    return rcs, status.value, dict(recv_x=recv_x.cpu().numpy(), scales=None if scales is None else scales.cpu().numpy(),
+                                   src_info=src_info.cpu().numpy(), layout_range=layout.cpu().numpy(),
+                                   recv_count=count.cpu().numpy())
+
+
+@pytest.mark.parametrize("use_fp8", [False, True])
+def test_ll_dispatch_time_out_masks_the_late_rank(cuda, use_fp8):
+    """A rank whose selections never arrive (its send phase is told to leave out the word the
+    receivers wait for) costs the receive side its time-out, is entered in every receiver's
+    mask and counts as having sent nothing: the outputs are those of a world in which that
+    rank has no tokens, the others' waits are short, and the next dispatch treats it as
+    masked.  T = 80: two groups of selections per rank, the second partly filled."""
+    R, T, H, K, E, M = 4, 80, 512, 4, 16, 80
+    x, topk, _ = make_world(21, R, T, H, K, E, drop=0.05)
+    xb = bits16(x).reshape(R, T, H)
+    mask = torch.zeros((R, R), dtype=torch.int32, device=cuda)
+    wait = torch.zeros(R, dtype=torch.int64, device=cuda)
+    timeout_us = 300
+    rcs, status, got = raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, timeout_us=timeout_us, withhold=2, wait=wait)
+    assert rcs == [0], _lib.kernels_error()
+    nt = np.array([T, T, 0, T], np.int32)
+    assert_dispatch_equal(got, eo.ll_dispatch(xb, topk, E, M, use_fp8, num_tokens=nt, fill=0x55), use_fp8)
+    assert status == 0
+    want_mask = np.zeros((R, R), np.int32)
+    want_mask[:, 2] = 1
+    assert np.array_equal(mask.cpu().numpy(), want_mask)
+    ticks = wait.cpu().numpy()
+    budget = timeout_us * 100  # the wall clock of these GPUs runs at 100 MHz
+    assert ticks[2] > budget and all(0 <= ticks[r] < budget for r in (0, 1, 3))
+    # the mask now does what a mask set by hand does
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, use_fp8, mask=mask.cpu().numpy())
+    assert rc == 0
+    assert_dispatch_equal(got, eo.ll_dispatch(xb, topk, E, M, use_fp8, mask=want_mask, fill=0x55), use_fp8)
+    # nobody late: the plain result, nothing masked, nearly nothing waited
+    mask.zero_()
+    wait.zero_()
+    rcs, status, got = raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, timeout_us=timeout_us, wait=wait)
+    assert rcs == [0] and status == 0
+    assert_dispatch_equal(got, eo.ll_dispatch(xb, topk, E, M, use_fp8, fill=0x55), use_fp8)
+    assert not mask.any() and int(wait.max()) < budget
+
+
+def test_ll_dispatch_in_two_phases(cuda):
+    """Send phase and receive phase issued apart give the bytes of the single call, with and
+    without the arrival check; a repeated expert is still reported when arrivals are stamped;
+    arguments that make no sense are refused before anything is launched."""
+    R, T, H, K, E, M = 3, 70, 1024, 4, 12, 70
+    x, topk, _ = make_world(22, R, T, H, K, E, drop=0.1)
+    want = eo.ll_dispatch(bits16(x).reshape(R, T, H), topk, E, M, True, fill=0x55)
+    mask = torch.zeros((R, R), dtype=torch.int32, device=cuda)
+    for timeout_us in (0, 500):
+        rcs, status, got = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, mask, phases=(1, 2), timeout_us=timeout_us)
+        assert rcs == [0, 0] and status == 0, _lib.kernels_error()
+        assert_dispatch_equal(got, want, True)
+    assert not mask.any()
+    bad = topk.copy()
+    bad[2, 69, 1] = bad[2, 69, 0] = 5
+    _, status, _ = raw_ll_dispatch_phased(cuda, x, bad, E, M, True, mask, timeout_us=500)
+    assert status == 1
+    for kwargs in (dict(phases=(0,)), dict(phases=(4,)), dict(withhold=1), dict(withhold=R, timeout_us=10),
+                   dict(withhold=1, timeout_us=2_000_000)):
+        rcs, _, _ = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, mask, **kwargs)
+        assert rcs == [-1], kwargs
+    rcs, _, _ = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, None, timeout_us=10)  # a time-out needs a mask buffer
+    assert rcs == [-1]
+
+
+def test_buffer_time_out_hooks_and_ready_flags(cuda):
+    """The same through Buffer: a buffer with timeout_ms checks arrivals; the recv hook issues
+    the receive phase; combine waits for the ready word of each rank and masks the one whose
+    word never comes (its experts then drop out of the sums, as for a rank masked by hand,
+    examples/device/ep/tests/elastic/elastic.py:359-383)."""
+    R, T, H, K, E, M = 4, 16, 512, 4, 16, 16
+    El = E // R
+    x, topk, w = make_world(31, R, T, H, K, E, drop=0.0)
+    xd, td, wd = x.to(cuda), torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    buf = Buffer(R, device=cuda, timeout_ms=0.3)
+    status = torch.zeros(R, dtype=torch.int32, device=cuda)
+    # dispatch in two halves: nothing of the payload exists before the hook has run
+    rx, cnt, handle, _, hook = buf.dispatch(xd, td, M, E, use_fp8=False, return_recv_hook=True)
+    cnt.fill_(-7)
+    torch.cuda.synchronize()
+    assert int(cnt[0, 0]) == -7
+    hook()
+    torch.cuda.synchronize()
+    plain = Buffer(R, device=cuda)
+    rx0, cnt0, handle0, _, _ = plain.dispatch(xd, td, M, E, use_fp8=False)
+    torch.cuda.synchronize()
+    assert torch.equal(cnt, cnt0) and torch.equal(handle[1], handle0[1]) and torch.equal(handle.row_map, handle0.row_map)
+    buf.query_mask_buffer(status)
+    assert status.sum().item() == 0
+    # combine: rank 3's expert outputs are never reported ready
+    y = torch.where(torch.isfinite(rx.float()), rx, torch.zeros_like(rx))
+    ready = torch.tensor([1, 1, 1, 0], dtype=torch.int32, device=cuda)
+    waited = torch.zeros(R, dtype=torch.int64, device=cuda)
+    out, _, _ = buf.combine(y, td, wd, handle, rank_ready=ready, combine_wait_recv_cost_stats=waited)
+    torch.cuda.synchronize()
+    buf.query_mask_buffer(status)
+    assert status.tolist() == [0, 0, 0, 1]
+    assert int(waited[3]) > 300 * 100 and int(waited[:3].max()) < 300 * 100
+    keep = torch.from_numpy((topk // El != 3) & (topk >= 0))
+    wsum = (torch.from_numpy(w) * keep).sum(2)
+    for r in (0, 1, 2):
+        assert calc_diff(x[r].float() * wsum[r].unsqueeze(1), out[r].float().cpu()) < 1e-5
+    mask = np.zeros((R, R), np.int32)
+    mask[:, 3] = 1
+    want = eo.ll_combine(bits16(y).reshape(R, El, R * M, H), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(), E, M,
+                         mask=mask)
+    assert np.array_equal(bits16(out).reshape(R, T, H)[:3], want[:3])
+    # a withheld rank in dispatch, through the one-shot knob
+    buf.clean_mask_buffer()
+    buf.withhold_rank = 1
+    _, cnt, _, _, _ = buf.dispatch(xd, td, M, E, use_fp8=False)
+    torch.cuda.synchronize()
+    buf.query_mask_buffer(status)
+    assert status.tolist() == [0, 1, 0, 0] and buf.withhold_rank == -1
+    alive = torch.tensor([0, 2, 3])
+    for e in range(E):
+        assert int(cnt[e // El, e % El]) == int((torch.from_numpy(topk)[alive] == e).sum())
+
+
 # ---- committed golden vectors (tests/golden, independent of the oracle) ---------------------------
 
 def _golden(name):
