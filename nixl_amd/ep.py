@@ -429,31 +429,40 @@ class Buffer:
         R, T, K = topk_idx.shape
         num_experts = x.shape[1] * R
         combined = out if out is not None else torch.empty((R, T, hidden), dtype=torch.bfloat16, device=x.device)
+        stats = combine_wait_recv_cost_stats
         if rank_ready is not None:
             if self.timeout_ms is None:
                 raise EPError("rank_ready needs a buffer created with timeout_ms")
             if rank_ready.dtype != torch.int32 or rank_ready.numel() < R:
                 raise EPError("rank_ready must hold R int32 values")
-            stats = combine_wait_recv_cost_stats
             if stats is not None and (stats.dtype != torch.int64 or stats.numel() < R):
                 raise EPError("combine_wait_recv_cost_stats must hold R int64 values")
             self._mask_active = True
-            rc = self._k.nixl_amd_ep_ll_combine_elastic(
+        row_map = getattr(handle, "row_map", None)
+
+        def issue():
+            if rank_ready is not None:
+                return self._k.nixl_amd_ep_ll_combine_elastic(
+                    _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
+                    _ptr(self.mask_buffer), _ptr(rank_ready), _ptr(stats), _ptr(num_tokens_per_rank), _ptr(row_map), T,
+                    hidden, max_tok, K, R, num_experts, int(use_logfmt), max(int(self.timeout_ms * 1000), 1), _stream())
+            return self._k.nixl_amd_ep_ll_combine(
                 _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
-                _ptr(self.mask_buffer), _ptr(rank_ready), _ptr(stats), _ptr(num_tokens_per_rank),
-                _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K, R, num_experts, int(use_logfmt),
-                max(int(self.timeout_ms * 1000), 1), _stream())
+                self._mask_ptr(), _ptr(num_tokens_per_rank), _ptr(row_map), T, hidden, max_tok, K, R, num_experts,
+                int(use_logfmt), _stream())
+
+        # The send phase of the reference moves the expert outputs to their readers; here they
+        # are read where they lie, so with a hook the whole reduction is the receive phase and
+        # combined_x is valid once the hook has run (as in the reference).
+        hook = None
+        if return_recv_hook:
+            hook = lambda: _check(issue(), "low_latency_combine (receive phase)")  # noqa: E731
         else:
-            rc = self._k.nixl_amd_ep_ll_combine(
-                _ptr(combined), _ptr(x), _ptr(topk_idx), _ptr(topk_weights), _ptr(src_info), _ptr(layout_range),
-                self._mask_ptr(), _ptr(num_tokens_per_rank), _ptr(getattr(handle, "row_map", None)), T, hidden, max_tok, K,
-                R, num_experts, int(use_logfmt), _stream())
-        _check(rc, "low_latency_combine")
+            _check(issue(), "low_latency_combine")
         event = None
         if async_finish:
             event = torch.cuda.Event()
             event.record()
-        hook = (lambda: None) if return_recv_hook else None
         return combined, EventOverlap(event), hook
 
     def combine(self, *args, **kwargs):

@@ -837,8 +837,17 @@ def test_buffer_time_out_hooks_and_ready_flags(cuda):
     assert torch.equal(cnt, cnt0) and torch.equal(handle[1], handle0[1]) and torch.equal(handle.row_map, handle0.row_map)
     buf.query_mask_buffer(status)
     assert status.sum().item() == 0
-    # combine: rank 3's expert outputs are never reported ready
     y = torch.where(torch.isfinite(rx.float()), rx, torch.zeros_like(rx))
+    # combine with a hook: the reduction is the receive phase, nothing is written before it
+    canvas = torch.full((R, T, H), 7.0, dtype=torch.bfloat16, device=cuda)
+    out, _, hook = buf.combine(y, td, wd, handle, out=canvas, return_recv_hook=True)
+    torch.cuda.synchronize()
+    assert bool((canvas == 7.0).all())
+    hook()
+    whole, _, _ = plain.combine(y, td, wd, handle0)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), whole.view(torch.int16))
+    # combine: rank 3's expert outputs are never reported ready
     ready = torch.tensor([1, 1, 1, 0], dtype=torch.int32, device=cuda)
     waited = torch.zeros(R, dtype=torch.int64, device=cuda)
     out, _, _ = buf.combine(y, td, wd, handle, rank_ready=ready, combine_wait_recv_cost_stats=waited)
