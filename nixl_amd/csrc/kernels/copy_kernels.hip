@@ -163,19 +163,27 @@ copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) { // recs,
     const uint32_t p = uniform(blockIdx.x * WAVES + threadIdx.x / kWaveSize);
     if (p >= n_recs) return;
     const PieceRec rec = recs[p]; // same address in every lane of the wave: a scalar load
-    const uint64_t d = rec.dst + lane * 16u;
     const uint32_t units = rec.units; // >= 1
-    // Loads are unconditional (a lane past the end re-reads the piece's last unit) so that
-    // all of them are in flight together; only the stores are predicated.
+    // Lane 0 of every instruction sits on a 128-byte line of the destination: the piece's
+    // units are shifted up by the destination's offset inside its line (the plan cuts pieces
+    // so that shift + units <= kPieceUnits), and each store instruction then writes whole
+    // lines except at the two ends of the piece.  A line written half by one instruction
+    // and half by the next would go out as two partial writes.
+    const uint32_t shift = static_cast<uint32_t>(rec.dst >> 4) & 7u;
+    // Loads are unconditional (a lane outside the piece re-reads its first or last unit) so
+    // that all of them are in flight together; only the stores are predicated.
     v4u v[LOADS];
 #pragma unroll
     for (int k = 0; k < LOADS; ++k) {
-        const uint32_t u = min(k * kWaveSize + lane, units - 1);
+        const uint32_t at = k * kWaveSize + lane;
+        const uint32_t u = min(at < shift ? 0u : at - shift, units - 1);
         v[k] = load16<POL>(rec.src + u * 16ull);
     }
 #pragma unroll
-    for (int k = 0; k < LOADS; ++k)
-        if (k * kWaveSize + lane < units) store16<POL>(d + k * (kWaveSize * 16u), v[k]);
+    for (int k = 0; k < LOADS; ++k) {
+        const uint32_t at = k * kWaveSize + lane;
+        if (at >= shift && at - shift < units) store16<POL>(rec.dst + (at - shift) * 16ull, v[k]);
+    }
 }
 
 // One wavefront per chunk that crosses descriptor boundaries or is short.
