@@ -314,7 +314,9 @@ class Buffer:
                        async_finish=False, return_recv_hook=False, num_tokens_per_rank=None):
         """Routing and dispatch in one call (no reference counterpart: its callers bring
         their own top-k).  logits [R, T, E] float32.  Returns (topk_idx, topk_weights) followed
-        by what low_latency_dispatch returns; the selection is that of route()."""
+        by what low_latency_dispatch returns; the selection is that of route().  Issued whole:
+        a `timeout_ms` on the buffer and return_recv_hook do not split or guard this call (its
+        first kernel routes and publishes the selections in one go)."""
         if logits.dim() != 3 or not logits.is_contiguous() or logits.dtype != torch.float32:
             raise EPError("logits must be a contiguous [R, T, E] float32 tensor")
         return self._ll_dispatch(x, None, logits, num_topk, num_max_dispatch_tokens_per_rank, logits.shape[2],
