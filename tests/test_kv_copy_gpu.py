@@ -643,6 +643,34 @@ def test_descriptors_longer_than_4_gib(cuda):
     assert bool((dst[:d0] == 0x5A).all()) and bool((dst[d0 + big:d1] == 0x5A).all()) and bool((dst[d1 + odd:] == 0x5A).all())
 
 
+def test_more_pieces_than_one_launch_takes(cuda):
+    """2^21 + 4097 descriptors of 256 bytes whose destinations start 16 bytes into a line: one
+    piece (one wavefront) each, more than the largest grid of one launch, so the plan goes out
+    as two launches.  Every destination row must hold its source row and the 16 bytes in front
+    of it must keep the canary."""
+    import torch
+    n, blk, pitch = (1 << 21) + 4097, 256, 272
+    g = torch.Generator(device=cuda).manual_seed(7)
+    src = torch.randint(0, 256, (n, blk), dtype=torch.uint8, device=cuda, generator=g)
+    dst = torch.full((n, pitch), 0xC3, dtype=torch.uint8, device=cuda)
+    perm = torch.randperm(n, device=cuda, generator=g)
+    descs = np.empty((n, 3), dtype=np.uint64)
+    descs[:, 0] = np.uint64(src.data_ptr()) + np.arange(n, dtype=np.uint64) * np.uint64(blk)
+    descs[:, 1] = np.uint64(dst.data_ptr()) + perm.cpu().numpy().astype(np.uint64) * np.uint64(pitch) + np.uint64(16)
+    descs[:, 2] = blk
+    lib = _lib.kernels()
+    plan = ctypes.c_void_p()
+    rc = lib.nixl_amd_copy_plan_create(ctypes.cast(descs.ctypes.data, ctypes.POINTER(_lib.CopyDesc)), n, 0, None, ctypes.byref(plan))
+    assert rc == 0, _lib.kernels_error()
+    info = _lib.CopyPlanInfo()
+    lib.nixl_amd_copy_plan_query(plan, ctypes.byref(info))
+    assert info.piece_items == n
+    _run_plan(torch, plan)
+    assert lib.nixl_amd_copy_plan_destroy(plan) == 0
+    assert torch.equal(dst[perm, 16:], src)
+    assert bool((dst[:, :16] == 0xC3).all())
+
+
 def test_golden_descriptor_list(cuda):
     """Committed vector (tests/golden/kv_descs.npz): mixed aligned / unaligned / empty
     descriptors, destination pre-filled with a canary byte."""
