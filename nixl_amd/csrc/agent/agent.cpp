@@ -678,6 +678,112 @@ nixlAgent::prepXferDlist(const nixl_xfer_dlist_t &descs,
     return prepXferDlist(NIXL_INIT_AGENT, descs, dlist_hndl, extra_params);
 }
 
+namespace {
+
+// First position of `indices` that does not name an entry of a list of `flat` entries, or
+// indices.size().  The scan has no early exit in its inner loop so that it vectorises; it is
+// the only place the index vectors are checked.
+size_t
+firstIndexOutside(const std::vector<int> &indices, size_t flat) {
+    constexpr size_t kBlock = 4096;
+    const unsigned limit = flat > static_cast<size_t>(INT32_MAX) ? static_cast<unsigned>(INT32_MAX) + 1u : static_cast<unsigned>(flat);
+    for (size_t b0 = 0; b0 < indices.size(); b0 += kBlock) {
+        const size_t b1 = std::min(indices.size(), b0 + kBlock);
+        unsigned bad = 0;
+        for (size_t i = b0; i < b1; ++i)
+            bad |= static_cast<unsigned>(static_cast<unsigned>(indices[i]) >= limit); // a negative index wraps to a large one
+        if (bad)
+            for (size_t i = b0; i < b1; ++i)
+                if (static_cast<unsigned>(indices[i]) >= limit) return i;
+    }
+    return indices.size();
+}
+
+// Walks a prepared list by flat index; consecutive look-ups usually stay inside one run.
+class runCursor {
+public:
+    explicit runCursor(const nixl_stride_dlist_t &runs)
+        : runs_(runs),
+          // ceiling division keeps find()'s first probe inside the run array
+          guess_((runs.flatSize() + static_cast<size_t>(runs.descCount()) - 1) / static_cast<size_t>(runs.descCount())) {}
+
+    const nixlStrideDesc &
+    at(size_t index) {
+        if (!run_ || index - run_->start_idx >= run_->count) run_ = &runs_.find(index, guess_);
+        return *run_;
+    }
+
+private:
+    const nixl_stride_dlist_t &runs_;
+    const size_t guess_;
+    const nixlStrideDesc *run_ = nullptr;
+};
+
+// First backend that prepared both handles, in the caller's order of preference if one was given.
+nixlBackendEngine *
+commonBackend(const nixlDlistH &local_side, const nixlDlistH &remote_side, const nixl_opt_args_t *extra_params) {
+    const auto both = [&](nixlBackendEngine *b) { return local_side.descs.count(b) && remote_side.descs.count(b); };
+    if (extra_params && !extra_params->backends.empty()) {
+        for (nixlBackendH *h : extra_params->backends)
+            if (both(h->engine)) return h->engine;
+        return nullptr;
+    }
+    for (const auto &kv : local_side.descs)
+        if (both(kv.first)) return kv.first;
+    return nullptr;
+}
+
+// Index pairs -> descriptor pairs (the result of src/core/nixl_agent.cpp:799-857).  With
+// `merge`, a stretch of pairs becomes one descriptor pair when it advances by one on both
+// sides inside one run each and the two runs are dense with the same pitch: only then are
+// the blocks adjacent in memory on both sides.
+nixl_status_t
+expandIndexPairs(const nixl_stride_dlist_t &lruns,
+                 const nixl_stride_dlist_t &rruns,
+                 const std::vector<int> &local_indices,
+                 const std::vector<int> &remote_indices,
+                 bool merge,
+                 nixl_meta_dlist_t &initiator,
+                 nixl_meta_dlist_t &target,
+                 size_t &total_bytes) {
+    const size_t count = local_indices.size();
+    if (const size_t at = firstIndexOutside(local_indices, lruns.flatSize()); at != count) {
+        NIXL_ERROR << "makeXferReq: local index " << local_indices[at] << " (position " << at << ") is outside its list of "
+                   << lruns.flatSize() << " entries";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    if (const size_t at = firstIndexOutside(remote_indices, rruns.flatSize()); at != count) {
+        NIXL_ERROR << "makeXferReq: remote index " << remote_indices[at] << " (position " << at << ") is outside its list of "
+                   << rruns.flatSize() << " entries";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+    initiator.reserve(count);
+    target.reserve(count);
+    runCursor lcur(lruns), rcur(rruns);
+    total_bytes = 0;
+    for (size_t i = 0, step = 1; i < count; i += step) {
+        const size_t li = static_cast<size_t>(local_indices[i]), ri = static_cast<size_t>(remote_indices[i]);
+        const nixlStrideDesc &lrun = lcur.at(li), &rrun = rcur.at(ri);
+        if (lrun.len != rrun.len) {
+            NIXL_ERROR << "makeXferReq: pair " << i << " joins a block of " << lrun.len << " bytes (local index " << li
+                       << ") with one of " << rrun.len << " bytes (remote index " << ri << ")";
+            return NIXL_ERR_INVALID_PARAM;
+        }
+        step = 1;
+        if (merge && lrun.stride == lrun.len && lrun.stride == rrun.stride) {
+            const size_t room = std::min({lrun.start_idx + lrun.count - li, rrun.start_idx + rrun.count - ri, count - i});
+            while (step < room && static_cast<size_t>(local_indices[i + step]) == li + step &&
+                   static_cast<size_t>(remote_indices[i + step]) == ri + step)
+                ++step;
+        }
+        total_bytes += initiator.emplace(lrun.getMetaDesc(li, step)).len;
+        target.emplace(rrun.getMetaDesc(ri, step));
+    }
+    return NIXL_SUCCESS;
+}
+
+} // namespace
+
 // reference: src/core/nixl_agent.cpp:696-887
 nixl_status_t
 nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
@@ -703,23 +809,9 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
         return NIXL_ERR_INVALID_PARAM;
     }
 
-    // First backend that prepared both sides, in the caller's order if one was given.
-    nixlBackendEngine *backend = nullptr;
-    if (extra_params && !extra_params->backends.empty()) {
-        for (nixlBackendH *h : extra_params->backends)
-            if (local_side->descs.count(h->engine) && remote_side->descs.count(h->engine)) {
-                backend = h->engine;
-                break;
-            }
-    } else {
-        for (const auto &kv : local_side->descs)
-            if (remote_side->descs.count(kv.first)) {
-                backend = kv.first;
-                break;
-            }
-    }
+    nixlBackendEngine *backend = commonBackend(*local_side, *remote_side, extra_params);
     if (!backend) {
-        NIXL_ERROR_FUNC << "could not find a common backend for the prepped Dlists";
+        NIXL_ERROR_FUNC << "no backend has prepared both descriptor list handles";
         return NIXL_ERR_INVALID_PARAM;
     }
 
@@ -765,52 +857,11 @@ nixlAgent::makeXferReq(const nixl_xfer_op_t &operation,
             }
         }
     }
-    req->initiatorDescs.reserve(count);
-    req->targetDescs.reserve(count);
-
-    const bool no_merge = extra_params && extra_params->skipDescMerge;
-    const size_t lflat = lruns.flatSize(), rflat = rruns.flatSize();
-    // Ceiling division keeps find()'s first probe inside the run array.
-    const size_t lguess = (lflat + lruns.descCount() - 1) / lruns.descCount();
-    const size_t rguess = (rflat + rruns.descCount() - 1) / rruns.descCount();
-
     size_t total = 0;
-    const nixlStrideDesc *lrun_p = nullptr, *rrun_p = nullptr;
-    for (size_t i = 0, step = 1; i < count; i += step) {
-        if (local_indices[i] < 0 || static_cast<size_t>(local_indices[i]) >= lflat) {
-            NIXL_ERROR_FUNC << "local index out of range at index " << i << " with value " << local_indices[i];
-            return NIXL_ERR_INVALID_PARAM;
-        }
-        if (remote_indices[i] < 0 || static_cast<size_t>(remote_indices[i]) >= rflat) {
-            NIXL_ERROR_FUNC << "remote index out of range at index " << i << " with value " << remote_indices[i];
-            return NIXL_ERR_INVALID_PARAM;
-        }
-        const size_t li = static_cast<size_t>(local_indices[i]);
-        const size_t ri = static_cast<size_t>(remote_indices[i]);
-        // the run of the previous index usually holds this one as well
-        if (!lrun_p || li - lrun_p->start_idx >= lrun_p->count) lrun_p = &lruns.find(li, lguess);
-        if (!rrun_p || ri - rrun_p->start_idx >= rrun_p->count) rrun_p = &rruns.find(ri, rguess);
-        const nixlStrideDesc &lrun = *lrun_p, &rrun = *rrun_p;
-        if (lrun.len != rrun.len) {
-            NIXL_ERROR_FUNC << "length mismatch at index " << i << " with local index " << li
-                            << " and remote index " << ri;
-            return NIXL_ERR_INVALID_PARAM;
-        }
-
-        // Consecutive indices collapse into one descriptor only when the local run is
-        // dense (stride == len), the remote run has the same stride, both index
-        // sequences advance by one, and neither run ends.
-        step = 1;
-        if (!no_merge && lrun.stride == lrun.len && lrun.stride == rrun.stride) {
-            const size_t room = std::min({lrun.start_idx + lrun.count - li, rrun.start_idx + rrun.count - ri, count - i});
-            while (step < room && static_cast<size_t>(local_indices[i + step]) == li + step &&
-                   static_cast<size_t>(remote_indices[i + step]) == ri + step)
-                ++step;
-        }
-        const nixlMetaDesc &ld = req->initiatorDescs.emplace(lrun.getMetaDesc(li, step));
-        req->targetDescs.emplace(rrun.getMetaDesc(ri, step));
-        total += ld.len;
-    }
+    const nixl_status_t expanded = expandIndexPairs(lruns, rruns, local_indices, remote_indices,
+                                                    !(extra_params && extra_params->skipDescMerge), req->initiatorDescs,
+                                                    req->targetDescs, total);
+    if (expanded != NIXL_SUCCESS) return expanded;
     NIXL_DEBUG << "merged " << count << " indices into " << req->initiatorDescs.descCount() << " descriptors";
 
     req->engine = backend;

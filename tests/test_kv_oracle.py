@@ -195,6 +195,15 @@ def test_agent_argument_errors(cpu_agent):
         with pytest.raises(NixlError) as e:
             a.make_prepped_xfer("WRITE", *args)
         assert e.value.status == ag.NIXL_ERR_INVALID_PARAM
+    # one bad entry deep inside long index vectors, on either side: the whole request is refused
+    long_ok = np.tile(np.arange(3, dtype=np.int32), 4000)
+    for pos, value in ((4096 + 17, 3), (11999, -2**31), (0, 2**31 - 1)):
+        for side in (0, 1):
+            li, ri = long_ok.copy(), long_ok.copy()
+            (li if side == 0 else ri)[pos] = value
+            with pytest.raises(NixlError) as e:
+                a.make_prepped_xfer("WRITE", hl, li, hr, ri)
+            assert e.value.status == ag.NIXL_ERR_INVALID_PARAM
     # notifications are refused for a backend without them (:771-775)
     with pytest.raises(NixlError) as e:
         a.make_prepped_xfer("WRITE", hl, [0], hr, [1], notif_msg=b"x")
