@@ -1029,26 +1029,31 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
     if (e != hipSuccess)
         return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
     auto *up_src = static_cast<int32_t *>(staging), *up_dst = up_src + n;
-    uint64_t regular = 0, src_follows = 0;
-    const int64_t dst_dense = dst_all_dense ? 1 : INT64_MIN, src_dense = src_all_dense ? 1 : INT64_MIN;
-    int64_t prev_step = 0;
-    for (size_t i = 0; i < n; ++i) {
-        up_src[i] = src_index[i];
-        up_dst[i] = dst_index[i];
-        if (i > 0) {
-            const int64_t step = static_cast<int64_t>(dst_index[i]) - dst_index[i - 1];
-            regular += (step == dst_dense) | ((i > 1) & (step == prev_step));
-            prev_step = step;
-            src_follows += (static_cast<int64_t>(src_index[i]) - src_index[i - 1] == src_dense);
-        }
+    std::memcpy(up_src, src_index, index_bytes);
+    std::memcpy(up_dst, dst_index, index_bytes);
+    // How many destination steps are regular (one block on in dense lists, or the same step as
+    // the one before) and how many source steps go one block on: differences taken modulo 2^32
+    // and without a value carried from one iteration to the next, so that the loop vectorises.
+    uint32_t regular = 0, src_follows = 0; // n < 2^31
+    const uint32_t dst_dense = dst_all_dense ? 1u : 0u, src_dense = src_all_dense ? 1u : 0u;
+    const auto *sv = reinterpret_cast<const uint32_t *>(src_index);
+    const auto *dv = reinterpret_cast<const uint32_t *>(dst_index);
+    if (n > 1) {
+        regular += ((dv[1] - dv[0]) == 1u) & dst_dense;
+        src_follows += ((sv[1] - sv[0]) == 1u) & src_dense;
+    }
+    for (size_t i = 2; i < n; ++i) {
+        const uint32_t step = dv[i] - dv[i - 1], before = dv[i - 1] - dv[i - 2];
+        regular += (static_cast<uint32_t>(step == 1u) & dst_dense) | static_cast<uint32_t>(step == before);
+        src_follows += static_cast<uint32_t>((sv[i] - sv[i - 1]) == 1u) & src_dense;
     }
     if (tables) {
         auto *up_runs = reinterpret_cast<nixl_amd_copy_run_t *>(static_cast<uint8_t *>(staging) + table_at);
         std::memcpy(up_runs, src_runs, n_src_runs * sizeof(nixl_amd_copy_run_t));
         std::memcpy(up_runs + n_src_runs, dst_runs, n_dst_runs * sizeof(nixl_amd_copy_run_t));
     }
-    const bool scattered = !(n == 1 || 2 * regular >= n - 1);
-    const bool sort = scattered && sort_scatter != 2 && 2 * src_follows >= n - 1 && n >= kSortWindow;
+    const bool scattered = !(n == 1 || 2 * static_cast<uint64_t>(regular) >= n - 1);
+    const bool sort = scattered && sort_scatter != 2 && 2 * static_cast<uint64_t>(src_follows) >= n - 1 && n >= kSortWindow;
 
     auto *plan = new nixl_amd_copy_plan();
     plan->device = device;
