@@ -115,14 +115,18 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
     prep_dlist_ms = (time.perf_counter() - t0) * 1e3
     stg_idx = np.arange(n_desc, dtype=np.int32)
 
-    def make(rng):
+    def block_list(rng):
+        """What a scheduler hands over: which blocks to send and where they go, as indices
+        into the prepared lists."""
         sel = rng.choice(pool_blocks, n_sel, replace=False)
         dst_ids = rng.permutation(pool_blocks)[:n_sel]
-        src_idx, dst_idx = _kv_indices(lk, pool_blocks, sel, order), _kv_indices(lk, pool_blocks, dst_ids, order)
+        return sel, dst_ids, _kv_indices(lk, pool_blocks, sel, order), _kv_indices(lk, pool_blocks, dst_ids, order)
+
+    def make(src_idx, dst_idx):
         t = time.perf_counter()
         gather = agent.make_prepped_xfer("WRITE", h_src, src_idx, h_stg_r, stg_idx)
         scatter = agent.make_prepped_xfer("WRITE", h_stg_l, stg_idx, h_dst, dst_idx)
-        return gather, scatter, sel, dst_ids, (time.perf_counter() - t) * 1e3
+        return gather, scatter, (time.perf_counter() - t) * 1e3
 
     def run(req):
         state = agent.transfer(req)
@@ -136,26 +140,32 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
         if not torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16)):
             raise RuntimeError("scattered blocks differ from the source blocks")
 
-    # (b) a new block list per request pair: make + post + wait, wall clock
+    # (b) a new block list per request pair, as a serving loop sees it: make + post + wait, wall
+    # clock, the pair released when it is done (its plan memory goes back to the engine's pool).
     rng = np.random.default_rng(99)
-    make_ms, fresh_ms, pairs = [], [], []
-    for i in range(max(fresh_requests, 1) + 1):
+    make_ms, fresh_ms = [], []
+    for i in range(max(fresh_requests, 1) + 2):
+        sel, dst_ids, src_idx, dst_idx = block_list(rng)
         torch.cuda.synchronize()
         w0 = time.perf_counter()
-        gather, scatter, sel, dst_ids, m = make(rng)
+        gather, scatter, m = make(src_idx, dst_idx)
         run(gather)
         run(scatter)
         w = (time.perf_counter() - w0) * 1e3
         check(sel, dst_ids)
-        if i == 0:  # the first pair also pays one-off allocations: not counted, not kept
-            gather.release()
-            scatter.release()
-            continue
-        make_ms.append(m)
-        fresh_ms.append(w)
-        pairs.append((gather, scatter, sel, dst_ids))
         n_g, bytes_g = gather.desc_count()
         assert bytes_g == n_desc * blk and n_g <= n_desc  # neighbouring blocks may have been merged
+        gather.release()
+        scatter.release()
+        if i >= 2:  # the first pairs also pay one-off allocations
+            make_ms.append(m)
+            fresh_ms.append(w)
+    # the pairs of the steady-state measurement below, over different block sets
+    pairs = []
+    for i in range(max(fresh_requests, 1)):
+        sel, dst_ids, src_idx, dst_idx = block_list(rng)
+        gather, scatter, _ = make(src_idx, dst_idx)
+        pairs.append((gather, scatter, sel, dst_ids))
 
     # (a) steady state: the prepared pairs re-posted in turn.  Which blocks a pair names moves
     # its time by several per cent (placement in DRAM), so the figure is the mean over the pairs.

@@ -89,7 +89,9 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
  * expands such indices into descriptors on the host, one by one): only the two index vectors
  * go to the device, where a kernel writes the records.  Bases and strides must be multiples
  * of 128 and `len` a whole number of chunks (1 KiB at the default tuning); the caller checks
- * the indices against the lists they index.  The index arrays may be freed on return. */
+ * the indices against the lists they index.  The index arrays may be freed on return.  The
+ * call does not wait for the device: the records are written by kernels queued on a stream of
+ * the library's, and nixl_amd_copy_plan_launch makes its stream wait for them. */
 int
 nixl_amd_copy_plan_create_indexed(uint64_t src_base,
                                   uint64_t src_stride,

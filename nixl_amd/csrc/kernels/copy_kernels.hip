@@ -32,6 +32,7 @@
 // overlap each other's destination ranges (the reference's puts are unordered too).
 #include <algorithm>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -593,7 +594,71 @@ struct nixl_amd_copy_plan {
     uint32_t generic_wgs = 0;
     nixl_amd_copy_plan_info_t info{};
     hipEvent_t ev0 = nullptr, ev1 = nullptr; // timing events, created on first use
+    // A plan built from index vectors returns before its records exist: they are written by
+    // kernels queued on the upload stream, `uploaded` is recorded behind them, and the first
+    // launches wait for it on their own stream.
+    hipEvent_t uploaded = nullptr;
 };
+
+// Pinned buffers whose contents are still travelling to the device: each goes back to the
+// upload cache once the event recorded behind its copy has completed, which the next plan
+// creation on the device looks for.
+struct PendingUpload {
+    hipEvent_t done;
+    void *staging;
+    size_t cap;
+};
+static std::mutex g_pending_mutex;
+static std::map<int, std::vector<PendingUpload>> g_pending; // by device
+
+static void
+reap_uploads(int device) {
+    std::lock_guard<std::mutex> lock(g_pending_mutex);
+    auto &list = g_pending[device];
+    for (size_t i = 0; i < list.size();) {
+        const hipError_t e = hipEventQuery(list[i].done);
+        if (e == hipErrorNotReady) {
+            (void)hipGetLastError();
+            ++i;
+            continue;
+        }
+        (void)hipEventDestroy(list[i].done);
+        upload_cache().put(device, list[i].staging, list[i].cap);
+        list[i] = list.back();
+        list.pop_back();
+    }
+}
+
+// Hands `staging` over: recycled when everything queued on `up` so far has run.  Without an
+// event to watch, the stream is waited for instead.
+static void
+recycle_after(int device, hipStream_t up, void *staging, size_t cap) {
+    hipEvent_t done = nullptr;
+    if (hipEventCreateWithFlags(&done, hipEventDisableTiming) == hipSuccess && hipEventRecord(done, up) == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_pending_mutex);
+        g_pending[device].push_back(PendingUpload{done, staging, cap});
+        return;
+    }
+    (void)hipGetLastError();
+    if (done) (void)hipEventDestroy(done);
+    (void)hipStreamSynchronize(up);
+    upload_cache().put(device, staging, cap);
+}
+
+// The plan's records are in place (or `wait` and they are not yet: block until they are).
+// Returns hipErrorNotReady when they are still being written and `wait` is false.
+static hipError_t
+settle_upload(nixl_amd_copy_plan *plan, bool wait) {
+    if (!plan->uploaded) return hipSuccess;
+    hipError_t e = wait ? hipEventSynchronize(plan->uploaded) : hipEventQuery(plan->uploaded);
+    if (e == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return e;
+    }
+    (void)hipEventDestroy(plan->uploaded);
+    plan->uploaded = nullptr;
+    return e;
+}
 
 extern "C" {
 
@@ -1025,6 +1090,7 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
     const size_t table_at = (2 * index_bytes + 15) & ~size_t(15); // the run tables follow the index vectors
     const size_t table_bytes = tables ? (n_src_runs + n_dst_runs) * sizeof(nixl_amd_copy_run_t) : 0;
     const size_t upload_bytes = tables ? table_at + table_bytes : 2 * index_bytes;
+    reap_uploads(device);
     hipError_t e = upload_cache().get(device, upload_bytes, &staging, &staging_cap);
     if (e != hipSuccess)
         return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
@@ -1089,13 +1155,18 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
                            dim3(kSortWindow / 2), 0, up, recs, static_cast<uint32_t>(n));
         e = hipGetLastError();
     }
-    if (e == hipSuccess) e = hipStreamSynchronize(up);
-    upload_cache().put(device, staging, staging_cap);
+    // No wait here: the event goes behind the kernels, launches wait for it on their stream.
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
     if (e != hipSuccess) {
+        if (up) (void)hipStreamSynchronize(up); // whatever was queued reads the buffers given back below
+        if (plan->uploaded) (void)hipEventDestroy(plan->uploaded);
+        upload_cache().put(device, staging, staging_cap);
         if (plan->arena) arena_cache().put(device, plan->arena, plan->arena_cap);
         delete plan;
         return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan upload: ") + hipGetErrorString(e));
     }
+    recycle_after(device, up, staging, staging_cap);
     plan->arena_bytes = rec_bytes + upload_bytes;
     plan->uniform_recs = recs;
     plan->chunks_per_rec = static_cast<uint32_t>(len / chunk_bytes);
@@ -1134,6 +1205,17 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
     const DeviceScope on_device(plan->device);
     HIP_TRY(on_device.status());
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (plan->uploaded) {
+        hipError_t e = settle_upload(plan, false);
+        if (e == hipErrorNotReady) {
+            e = hipStreamWaitEvent(s, plan->uploaded, 0);
+            if (e != hipSuccess) { // a stream that cannot take the dependency (e.g. under capture): wait here instead
+                (void)hipGetLastError();
+                e = settle_upload(plan, true);
+            }
+        }
+        HIP_TRY(e);
+    }
     if (plan->uniform_wgs) {
         // One launch per kMaxGrid workgroups.  With the die swizzle each launch's grid is
         // rounded up to a multiple of 8 so that every die owns an equally long slice; surplus
@@ -1180,6 +1262,7 @@ int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan) {
     if (!plan) return NIXL_AMD_OK;
     const DeviceScope on_device(plan->device);
+    (void)settle_upload(plan, true); // the arena and the upload buffer go back only when nothing writes or reads them
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     if (plan->arena) arena_cache().put(plan->device, plan->arena, plan->arena_cap);

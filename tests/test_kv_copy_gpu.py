@@ -364,6 +364,42 @@ def test_run_tables_through_the_kernel_library(cuda):
     assert rc != 0 and "follow" in _lib.kernels_error()
 
 
+def test_indexed_plans_launched_and_dropped_at_once(cuda):
+    """Plan creation from index vectors returns before the records exist on the device.  A
+    launch issued at once (no synchronisation in between, on the default stream and on
+    another one) must still see them; plans dropped unused, and many plans in a row, must
+    neither leak nor confuse the pinned buffers their indices travel through."""
+    import torch
+    lib = _lib.kernels()
+    blk, n_pool, n = 4096, 3000, 2048
+    rng = np.random.default_rng(17)
+    host = rng.integers(0, 256, 2 * n_pool * blk, dtype=np.uint8)
+    mem = torch.from_numpy(host.copy()).to(cuda)
+    base = mem.data_ptr()
+    other = torch.cuda.Stream(device=cuda)
+    want = host.copy()
+    plans = []
+    for round_ in range(12):
+        si = rng.permutation(n_pool)[:n].astype(np.int32)
+        di = rng.permutation(n_pool)[:n].astype(np.int32)
+        plan = ctypes.c_void_p()
+        rc = lib.nixl_amd_copy_plan_create_indexed(base, blk, si.ctypes.data, base + n_pool * blk, blk, di.ctypes.data, n, blk, 0,
+                                                   None, ctypes.byref(plan))
+        assert rc == 0, _lib.kernels_error()
+        if round_ % 3 == 2:  # dropped without a launch
+            assert lib.nixl_amd_copy_plan_destroy(plan) == 0
+            continue
+        stream = other if round_ % 2 else torch.cuda.default_stream(cuda)
+        torch.cuda.synchronize()  # earlier rounds' copies are over; this plan's upload may still be on its way
+        assert lib.nixl_amd_copy_plan_launch(plan, ctypes.c_void_p(stream.cuda_stream)) == 0, _lib.kernels_error()
+        plans.append(plan)
+        ko.copy_descs(want, si.astype(np.int64) * blk, (n_pool + di.astype(np.int64)) * blk, [blk] * n)
+    torch.cuda.synchronize()
+    assert np.array_equal(mem.cpu().numpy(), want)
+    for plan in plans:
+        assert lib.nixl_amd_copy_plan_destroy(plan) == 0
+
+
 def test_write_zero_read_roundtrip_and_repost(hip_agent, cuda):
     # transfer_handler round trip (test/gtest/plugins/transfer_handler.h:182-209 with
     # memory_handler.h:42-58): WRITE, clear the source, READ back, expect the increasing
