@@ -859,6 +859,24 @@ nixlHipEngine::loadRemoteMD(const nixlBlobDesc &input,
             }
             it = ipcMaps_.emplace(key, ipcMapping{base, region.device, 0}).first;
         }
+        // What the peer says about its allocation is checked against what got mapped: the
+        // region must lie inside the mapping as this process sees it.
+        void *seen_base = nullptr;
+        size_t seen_size = 0;
+        const uint64_t offset = region.addr - region.alloc_base;
+        if (hipMemGetAddressRange(reinterpret_cast<hipDeviceptr_t *>(&seen_base), &seen_size,
+                                  reinterpret_cast<hipDeviceptr_t>(it->second.base)) != hipSuccess ||
+            seen_base != it->second.base || region.len > seen_size || offset > seen_size - region.len) {
+            (void)hipGetLastError();
+            NIXL_ERROR << "HIP backend: region published by agent '" << remote_agent << "' (process " << region.pid
+                       << ") does not fit the allocation it names (" << seen_size << " bytes as mapped here)";
+            if (it->second.refs == 0) {
+                const DeviceScope on_device(it->second.device);
+                (void)hipIpcCloseMemHandle(it->second.base);
+                ipcMaps_.erase(it);
+            }
+            return NIXL_ERR_INVALID_PARAM;
+        }
         ++it->second.refs;
         mapped = it->second.base;
     }

@@ -28,4 +28,6 @@ def test_write_read_and_notify_between_two_processes(cuda, tmp_path):
             if p.poll() is None:
                 p.kill()
     assert initiator.returncode == 0 and "initiator OK" in out_i, out_i
+    # the forged blob was turned down for the right reason (the backend's own error line)
+    assert "forged blob refused" in out_i and "does not fit the allocation it names" in out_i, out_i
     assert target.returncode == 0 and "target OK" in out_t, out_t

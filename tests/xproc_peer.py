@@ -77,10 +77,26 @@ def initiator(workdir):
     agent = nixl_agent("I", nixl_agent_config(backends=("HIP",)))
     agent.register_memory([local])
     with open(md_path, "rb") as f:
-        name = agent.add_remote_agent(f.read())
-    assert name == "T", name
+        blob = f.read()
     with open(os.path.join(workdir, "target.addr")) as f:
         remote_base = int(f.read())
+    # A blob that claims a region (and an allocation) far longer than what the target shares is
+    # refused when it is loaded: the region is checked against the mapping as seen here.
+    import struct
+    honest = struct.pack("<QQ", remote_base, 2 * HALF)
+    at = blob.find(b"HIPREGN2")
+    if at < 0 or blob.count(honest) < 2:
+        raise SystemExit("initiator: the metadata blob does not look as expected")
+    forged = bytearray(blob.replace(honest, struct.pack("<QQ", remote_base, 1 << 30)))
+    forged[at + 48:at + 56] = struct.pack("<Q", (1 << 30) + (512 << 20))  # alloc_size
+    try:
+        agent.add_remote_agent(bytes(forged))
+    except Exception as e:
+        print("initiator: forged blob refused:", e, flush=True)
+    else:
+        raise SystemExit("initiator: a region longer than the target's allocation was accepted")
+    name = agent.add_remote_agent(blob)
+    assert name == "T", name
     triple = lambda a: np.array([[a, HALF, 0]], dtype=np.uint64)
     # WRITE local first half -> target first half, with a notification that must not overtake the bytes
     w = agent.initialize_xfer("WRITE", agent.get_xfer_descs(triple(local.data_ptr()), "VRAM"),
