@@ -95,102 +95,19 @@ constexpr const char *kConnMailbox = ";mbox=";
 // been seen not to return.
 constexpr size_t kMaxIpcAllocation = (size_t{2} << 30) - 1;
 
-constexpr uint32_t kMailboxSlots = 256;
-constexpr uint32_t kMailboxSlotBytes = 4096 - 16;
-constexpr uint32_t kMailboxMagic = 0x584f424du; // "MBOX"
+using nixl_amd_hip::kMailboxSlotBytes;
 std::atomic<unsigned> g_mailboxCounter{0};
 
 } // namespace
 
-// A bounded multi-producer, single-consumer ring in POSIX shared memory (cell sequence numbers
-// as in Vyukov's bounded queue): producers are the engines of other processes, the consumer is
-// the engine that created it.  A message is the sender's agent name followed by the payload.
-struct nixlHipEngine::Mailbox {
-    struct Cell {
-        std::atomic<uint64_t> sequence;
-        uint32_t senderLen;
-        uint32_t msgLen;
-        char data[kMailboxSlotBytes];
-    };
-    std::atomic<uint32_t> magic;
-    std::atomic<uint64_t> head; // next position to write
-    std::atomic<uint64_t> tail; // next position to read
-    Cell cells[kMailboxSlots];
-
-    bool
-    push(const std::string &sender, const std::string &msg) {
-        if (sender.size() + msg.size() > kMailboxSlotBytes) return false;
-        uint64_t pos = head.load(std::memory_order_relaxed);
-        for (;;) {
-            Cell &c = cells[pos % kMailboxSlots];
-            const uint64_t seq = c.sequence.load(std::memory_order_acquire);
-            const int64_t dif = static_cast<int64_t>(seq) - static_cast<int64_t>(pos);
-            if (dif == 0) {
-                if (head.compare_exchange_weak(pos, pos + 1, std::memory_order_relaxed)) {
-                    c.senderLen = static_cast<uint32_t>(sender.size());
-                    c.msgLen = static_cast<uint32_t>(msg.size());
-                    std::memcpy(c.data, sender.data(), sender.size());
-                    std::memcpy(c.data + sender.size(), msg.data(), msg.size());
-                    c.sequence.store(pos + 1, std::memory_order_release);
-                    return true;
-                }
-            } else if (dif < 0) {
-                return false; // full: the owner has not drained it
-            } else {
-                pos = head.load(std::memory_order_relaxed);
-            }
-        }
-    }
-
-    bool
-    pop(std::string &sender, std::string &msg) {
-        const uint64_t pos = tail.load(std::memory_order_relaxed);
-        Cell &c = cells[pos % kMailboxSlots];
-        if (c.sequence.load(std::memory_order_acquire) != pos + 1) return false; // empty
-        const uint32_t sl = std::min(c.senderLen, kMailboxSlotBytes), ml = std::min(c.msgLen, kMailboxSlotBytes - sl);
-        sender.assign(c.data, sl);
-        msg.assign(c.data + sl, ml);
-        tail.store(pos + 1, std::memory_order_relaxed);
-        c.sequence.store(pos + kMailboxSlots, std::memory_order_release);
-        return true;
-    }
-};
-
 nixlHipEngine::Mailbox *
 nixlHipEngine::mapMailbox(const std::string &name, bool create) {
-    static_assert(std::atomic<uint64_t>::is_always_lock_free, "the mailbox needs lock-free 64-bit atomics");
-    const int fd = shm_open(name.c_str(), create ? (O_RDWR | O_CREAT | O_EXCL) : O_RDWR, 0600);
-    if (fd < 0) return nullptr;
-    if (create && ftruncate(fd, sizeof(Mailbox)) != 0) {
-        close(fd);
-        shm_unlink(name.c_str());
-        return nullptr;
-    }
-    struct stat st {};
-    if (fstat(fd, &st) != 0 || static_cast<size_t>(st.st_size) < sizeof(Mailbox)) {
-        close(fd);
-        return nullptr;
-    }
-    void *mem = mmap(nullptr, sizeof(Mailbox), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
-    close(fd);
-    if (mem == MAP_FAILED) return nullptr;
-    auto *m = static_cast<Mailbox *>(mem);
-    if (create) {
-        for (uint32_t i = 0; i < kMailboxSlots; ++i)
-            m->cells[i].sequence.store(i, std::memory_order_relaxed);
-        m->head.store(0, std::memory_order_relaxed);
-        m->tail.store(0, std::memory_order_relaxed);
-        m->magic.store(kMailboxMagic, std::memory_order_release);
-    } else if (m->magic.load(std::memory_order_acquire) != kMailboxMagic) {
-        munmap(mem, sizeof(Mailbox));
-        return nullptr;
-    }
-    return m;
+    return nixl_amd_hip::mapMailbox(name, create);
 }
 
 void
 nixlHipEngine::unmapMailbox(Mailbox *m) {
-    if (m) munmap(m, sizeof(Mailbox));
+    nixl_amd_hip::unmapMailbox(m);
 }
 
 nixlHipReqH::~nixlHipReqH() {

@@ -23,6 +23,7 @@
 
 #include "backend/backend_engine.h"
 #include "nixl_amd_hip.h"
+#include "mailbox.h"
 
 // Registration record returned by registerMem and handed back in nixlMetaDesc::metadataP.
 // `addr` is the region's address in its OWNER's address space, which is the space the
@@ -261,7 +262,7 @@ private:
     std::thread progress_;
     // Peers whose connection info was loaded: agents of this process (no mailbox: their
     // engine is found in the process-wide registry) or of another one.
-    struct Mailbox; // shared-memory ring of notifications, defined with its users
+    using Mailbox = nixl_amd_hip::Mailbox; // shared-memory ring of notifications
     struct peerInfo {
         long long pid = 0;
         std::string mailboxName;

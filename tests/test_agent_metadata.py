@@ -321,6 +321,20 @@ def test_agents_used_from_several_threads(oracle_plugin_dir):
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
 
 
+def test_notification_ring_of_the_hip_backend_on_the_cpu():
+    """tests/cpp/mailbox_check.cpp: the shared-memory ring that carries notifications between
+    processes (nixl_amd/csrc/plugin/mailbox.h), fed by four threads and a child process at
+    once: every message arrives once, in each producer's order, bytes intact; full ring,
+    oversize message, taken name and foreign object are refused."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "mailbox_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
 def test_list_and_option_helpers_of_the_c_wrapper(two_agents):
     """The descriptor-list, option and stub helpers of the reference's C wrapper
     (src/bindings/rust/wrapper.h:193-201,297-326,457) behave as their names say; the metadata
