@@ -713,6 +713,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         const size_t cap = 2 * n;
         void *staging = nullptr;
         size_t staging_cap = 0;
+        reap_uploads(device);
         hipError_t e = upload_cache().get(device, cap * sizeof(UniformRec), &staging, &staging_cap);
         if (e != hipSuccess)
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
@@ -758,13 +759,18 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
                                    static_cast<uint32_t>(n_recs));
                 e = hipGetLastError();
             }
-            if (e == hipSuccess) e = hipStreamSynchronize(up);
-            upload_cache().put(device, staging, staging_cap);
+            // No wait here: the event goes behind the copy, launches wait for it on their stream.
+            if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
+            if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
             if (e != hipSuccess) {
+                if (up) (void)hipStreamSynchronize(up); // whatever was queued reads the buffers given back below
+                if (plan->uploaded) (void)hipEventDestroy(plan->uploaded);
+                upload_cache().put(device, staging, staging_cap);
                 if (plan->arena) arena_cache().put(device, plan->arena, plan->arena_cap);
                 delete plan;
                 return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan upload: ") + hipGetErrorString(e));
             }
+            recycle_after(device, up, staging, staging_cap);
             plan->arena_bytes = bytes;
             plan->uniform_recs = static_cast<const UniformRec *>(plan->arena);
             plan->chunks_per_rec = static_cast<uint32_t>(len0 / (chunk_units * 16u));
