@@ -1214,8 +1214,12 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
     if (plan->uploaded) {
         hipError_t e = settle_upload(plan, false);
         if (e == hipErrorNotReady) {
-            e = hipStreamWaitEvent(s, plan->uploaded, 0);
-            if (e != hipSuccess) { // a stream that cannot take the dependency (e.g. under capture): wait here instead
+            // A stream under graph capture must not be made to depend on work outside the
+            // graph: the host waits instead, and the graph holds the launch alone.
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            if (s && hipStreamIsCapturing(s, &capture) != hipSuccess) (void)hipGetLastError();
+            e = capture == hipStreamCaptureStatusNone ? hipStreamWaitEvent(s, plan->uploaded, 0) : hipErrorNotReady;
+            if (e != hipSuccess) {
                 (void)hipGetLastError();
                 e = settle_upload(plan, true);
             }
