@@ -143,6 +143,47 @@ def test_unaligned_brute_force(cuda):
     assert info.generic_descs > 0
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_mixture_of_every_descriptor_class(cuda, seed):
+    """One request that mixes everything the planner tells apart: lengths log-uniform from
+    1 byte to 200 KiB; addresses byte-aligned, 16-byte aligned, line-aligned or 4 KiB-aligned at
+    random and independently on the two sides; a sprinkling of zero lengths, exact chunk
+    multiples and lengths one unit off them.  All classes must land in one plan and every
+    byte must match the per-descriptor oracle, including the gaps between destinations."""
+    import torch
+    rng = np.random.default_rng(1000 + seed)
+    n = 3000
+    lens = np.exp(rng.uniform(0, np.log(200 << 10), n)).astype(np.int64)
+    special = rng.integers(0, n, 300)
+    lens[special[:60]] = 0
+    lens[special[60:140]] = rng.choice([1024, 2048, 4096, 8192, 16384, 65536], 80)
+    lens[special[140:220]] = rng.choice([1024, 4096, 8192, 16384], 80) + rng.choice([-16, 16, -1, 1], 80)
+    lens[special[220:]] = (lens[special[220:]] // 16) * 16
+    grain = rng.choice([1, 16, 128, 4096], n, p=[0.3, 0.3, 0.25, 0.15])
+    lens = np.where(grain >= 16, (lens // 16) * 16, lens)  # aligned addresses mostly carry aligned lengths
+    lens[rng.integers(0, n, 40)] += 3  # ... but not always
+    half = int(lens.sum() + n * (4096 + 256) + (1 << 20))
+    half = (half + 4095) // 4096 * 4096
+
+    def place(grains):
+        order = rng.permutation(n)
+        offs = np.empty(n, dtype=np.int64)
+        at = 0
+        for i in order:
+            g = int(grains[i])
+            at = (at + g - 1) // g * g
+            offs[i] = at
+            at += int(lens[i]) + int(rng.integers(0, 200))
+        assert at <= half
+        return offs
+
+    so = place(grain)
+    do = place(rng.permutation(grain)) + half
+    info = _check_against_oracle(torch, cuda, 2 * half, so, do, lens, seed=seed)
+    assert info.payload_bytes == int(lens.sum())
+    assert info.generic_descs > 0 and info.piece_items > 0 and info.vec_descs > 0
+
+
 def test_zero_length_and_empty(cuda):
     import torch
     dev = torch.zeros(4096, dtype=torch.uint8, device=cuda)
