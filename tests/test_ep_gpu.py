@@ -115,6 +115,30 @@ def test_ll_dispatch_matches_oracle(cuda, shape, use_fp8, round_scale, use_ue8m0
     assert_dispatch_equal(got, want, use_fp8, use_ue8m0)
 
 
+@pytest.mark.parametrize("hidden", [2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192])
+def test_ll_every_hidden_size_of_the_reference(cuda, hidden):
+    """The hidden sizes the reference's low-latency kernels are built for
+    (kernels/launch.cuh:100-112): dispatch (fp8 where hidden % 512 == 0, as csrc/nixl_ep.cpp:1091
+    demands, else bf16) and combine against the oracle, bit for bit."""
+    R, T, K, E, M = 2, 19, 3, 8, 24
+    El = E // R
+    x, topk, w = make_world(hidden, R, T, hidden, K, E, scale=2.0)
+    use_fp8 = hidden % 512 == 0
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, use_fp8)
+    assert rc == 0, _lib.kernels_error()
+    xb = bits16(x).reshape(R, T, hidden)
+    assert_dispatch_equal(got, eo.ll_dispatch(xb, topk, E, M, use_fp8, fill=0x55), use_fp8)
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, rx, torch.zeros_like(rx))
+    out, _, _ = buf.combine(y, td, wd, handle)
+    torch.cuda.synchronize()
+    want = eo.ll_combine(bits16(y).reshape(R, El, R * M, hidden), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(), E, M)
+    assert np.array_equal(bits16(out).reshape(R, T, hidden), want)
+
+
 def test_ll_dispatch_extreme_values(cuda):
     # zeros (amax floor 1e-4), huge and tiny magnitudes, a constant row, negative zero
     R, T, H, K, E, M = 2, 8, 512, 2, 4, 8
