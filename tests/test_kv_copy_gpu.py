@@ -441,6 +441,47 @@ def test_indexed_plans_launched_and_dropped_at_once(cuda):
         assert lib.nixl_amd_copy_plan_destroy(plan) == 0
 
 
+def test_many_requests_leave_memory_where_it_was(hip_agent, cuda):
+    """A serving loop: thousands of requests made from fresh index vectors, posted, waited for
+    and released.  Plan arenas, pinned upload buffers and events are recycled, so device memory
+    and the process's resident set stay where they were after a warm-up."""
+    import psutil
+    import torch
+    a = hip_agent
+    blk, n_pool, n = 4096, 4096, 1500
+    mem = torch.zeros(2 * n_pool * blk, dtype=torch.uint8, device=cuda)
+    a.register_memory([mem])
+    h_l = a.prep_xfer_dlist("", _descs(mem, np.arange(n_pool) * blk, [blk] * n_pool), "VRAM")
+    h_r = a.prep_xfer_dlist("agent", _descs(mem, (n_pool + np.arange(n_pool)) * blk, [blk] * n_pool), "VRAM")
+    rng = np.random.default_rng(23)
+    proc = psutil.Process()
+
+    def burst(count):
+        for i in range(count):
+            li = rng.permutation(n_pool)[:n].astype(np.int32)
+            ri = rng.permutation(n_pool)[:n].astype(np.int32)
+            if i % 3 == 0:  # every third through explicit descriptors
+                req = a.initialize_xfer("WRITE", a.get_xfer_descs(_descs(mem, li.astype(np.int64) * blk, [blk] * n), "VRAM"),
+                                        a.get_xfer_descs(_descs(mem, (n_pool + ri.astype(np.int64)) * blk, [blk] * n), "VRAM"),
+                                        "agent")
+            else:
+                req = a.make_prepped_xfer("WRITE", h_l, li, h_r, ri)
+            if i % 7 != 6:  # some are released without ever being posted
+                _wait(a, req)
+            req.release()
+
+    burst(200)
+    torch.cuda.synchronize()
+    free0, rss0 = torch.cuda.mem_get_info()[0], proc.memory_info().rss
+    burst(2500)
+    torch.cuda.synchronize()
+    free1, rss1 = torch.cuda.mem_get_info()[0], proc.memory_info().rss
+    assert free0 - free1 < (64 << 20), f"device memory shrank by {(free0 - free1) >> 20} MiB"
+    assert rss1 - rss0 < (96 << 20), f"resident set grew by {(rss1 - rss0) >> 20} MiB"
+    for h in (h_l, h_r):
+        h.release()
+
+
 def test_write_zero_read_roundtrip_and_repost(hip_agent, cuda):
     # transfer_handler round trip (test/gtest/plugins/transfer_handler.h:182-209 with
     # memory_handler.h:42-58): WRITE, clear the source, READ back, expect the increasing
