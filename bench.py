@@ -76,7 +76,7 @@ def _triples(addrs, blk):
     return np.stack([addrs, np.full(n, blk, np.uint64), np.zeros(n, np.uint64)], 1)
 
 
-def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
+def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False):
     """Gather + scatter of config 2's shape with `blk`-byte descriptors.  The pools and the
     staging buffer are prepared ONCE as descriptor lists (prep_xfer_dlist); every request is
     made from index vectors into those lists (make_prepped_xfer), the call pattern of the
@@ -119,6 +119,8 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4):
         """What a scheduler hands over: which blocks to send and where they go, as indices
         into the prepared lists."""
         sel = rng.choice(pool_blocks, n_sel, replace=False)
+        if sorted_ids:  # a scheduler that hands its block list over in ascending order of the source blocks
+            sel = np.sort(sel)
         dst_ids = rng.permutation(pool_blocks)[:n_sel]
         return sel, dst_ids, _kv_indices(lk, pool_blocks, sel, order), _kv_indices(lk, pool_blocks, dst_ids, order)
 
@@ -557,6 +559,11 @@ def main():
                 "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
                 "make_request_pair_ms": r["kv"]["make_request_pair_ms"],
                 "value_including_prepare": r["kv"]["value_including_prepare"]}
+        r = run_kv(args, blk, args.order, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2, sorted_ids=True)
+        others[f"{blk // 1024}KiB_{args.order}_order_source_blocks_ascending"] = {
+            "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
+            "note": "the same random block sets and random destinations, the request listing its source blocks in "
+                    "ascending order: the gather then reads the pool monotonically"}
         line["kv"]["other_points"] = others
     if not args.no_small:
         line["kv"]["small_descriptor_stress"] = run_small_descriptors()
