@@ -292,6 +292,12 @@ nixlHipEngine::registerMem(const nixlBlobDesc &mem, const nixl_mem_t &nixl_mem, 
         have_range = true;
     } else {
         (void)hipGetLastError();
+        // Device memory whose allocation the runtime cannot name is not registered: nothing
+        // would bound the region, and a descriptor beyond the allocation is a GPU fault.
+        if (nixl_mem == VRAM_SEG) {
+            NIXL_ERROR << "HIP backend: the allocation behind address " << mem.addr << " cannot be queried";
+            return NIXL_ERR_INVALID_PARAM;
+        }
     }
 
     auto *md = new nixlHipMD(mem.addr, mem.len, device, nixl_mem);
@@ -440,7 +446,11 @@ nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
             if (run.count == 0 || run.start_idx != flat[side]) return NIXL_ERR_NOT_SUPPORTED;
             if (run.len != len) return NIXL_ERR_NOT_SUPPORTED; // mixed lengths: the descriptor path judges them
             const auto *md = static_cast<const nixlHipMD *>(run.metadataP);
-            if (!md || !md->contains(run.addr, (run.count - 1) * run.stride + run.len)) {
+            // bytes from the run's first block to the end of its last, without wrapping around
+            size_t span = 0;
+            const bool fits = md && !__builtin_mul_overflow(run.count - 1, run.stride, &span) &&
+                !__builtin_add_overflow(span, run.len, &span) && md->contains(run.addr, span);
+            if (!fits) {
                 NIXL_ERROR << "HIP backend: a prepared list reaches outside its registered region";
                 return NIXL_ERR_INVALID_PARAM;
             }
