@@ -32,11 +32,13 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 
 # HBM bytes per launch of the dominant kernel from hardware counters.  Counters cannot be read
-# from inside this process: these figures come from rocprofv3 --pmc runs of this same file
-# (FETCH_SIZE and WRITE_SIZE, one run each, scaled by a plain 1 GiB element-wise kernel in the
-# same run); the summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks,
-# descriptor bytes) - the two descriptor orders move the same bytes; a shape without a counter
-# run reports null.
+# from inside this process.  The headline's figure is measured by measure_traffic_live below
+# (child runs under the profiler); the other points, and the headline when the profiler cannot
+# be run, take the figures of earlier rocprofv3 --pmc runs of this same file (FETCH_SIZE and
+# WRITE_SIZE, one run each, scaled by a plain 1 GiB element-wise kernel in the same run); the
+# summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks, descriptor
+# bytes) - the two descriptor orders move the same bytes; a shape without a counter run
+# reports null.
 _KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, not this run)"
 MEASURED_TRAFFIC = {
     (1024, 8192, 16384): {"bytes": 2164231731, "source": _KV_PROFILE},
@@ -45,6 +47,74 @@ MEASURED_TRAFFIC = {
                         "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
                                   "this file, not this run)"},
 }
+
+
+def measure_traffic_live(args, blk):
+    """HBM bytes per launch of the headline kernel from hardware counters, measured now: the
+    headline leg of this file is run twice more as a child process under `rocprofv3 --pmc`
+    (FETCH_SIZE, then WRITE_SIZE: one counter a run), each with one plain element-wise kernel
+    of known size (1 GiB read, 1 GiB written) as the yardstick the counter is scaled by.
+    Returns {"bytes", "source", ...}, or {"error": why} when the profiler is not there or a run
+    fails; the caller then falls back to the figures of profiles/."""
+    import csv
+    import glob
+    import shutil
+    import signal
+    import statistics
+    import subprocess
+    import tempfile
+    prof = shutil.which("rocprofv3")
+    if not prof:
+        return {"error": "rocprofv3 not found"}
+    if any("rocprof" in os.environ.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB")):
+        return {"error": "this process already runs under a profiler"}
+    child = [sys.executable, os.path.abspath(__file__), "--quick", "--no-ep", "--no-small", "--no-cpu-baseline",
+             "--no-live-traffic", "--calibrate-copy", "--steps", "3", "--warmup", "1", "--fresh-requests", "1",
+             "--block-bytes", str(blk), "--order", args.order, "--blocks", str(args.blocks),
+             "--pool-blocks", str(args.pool_blocks)]
+    for kv in args.backend_param:
+        child += ["--backend-param", kv]
+    got = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        out_dir = tempfile.mkdtemp(prefix="nixl_amd_pmc_", dir="/tmp")
+        try:
+            cmd = [prof, "--pmc", counter, "--output-format", "csv", "-d", out_dir, "-o", "t", "--"] + child
+            proc = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, stdout=subprocess.DEVNULL,
+                                    stderr=subprocess.DEVNULL, start_new_session=True)
+            try:
+                rc = proc.wait(timeout=150)
+            except subprocess.TimeoutExpired:
+                os.killpg(proc.pid, signal.SIGKILL)
+                proc.wait()
+                return {"error": f"the {counter} run did not finish in 150 s"}
+            if rc != 0:
+                return {"error": f"the {counter} run ended with status {rc}"}
+            files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+            if not files:
+                return {"error": f"the {counter} run left no counter file"}
+            kernel, yard = [], []
+            with open(files[0], newline="") as f:
+                for row in csv.DictReader(f):
+                    if row.get("Counter_Name") != counter:
+                        continue
+                    name = row.get("Kernel_Name", "")
+                    if "copy_uniform_kernel" in name:
+                        kernel.append(float(row["Counter_Value"]))
+                    elif "CUDAFunctorOnSelf_add<int>" in name:
+                        yard.append(float(row["Counter_Value"]))
+            if not kernel or not yard or max(yard) <= 0:
+                return {"error": f"the {counter} run has no samples of the copy kernel or of the yardstick"}
+            factor = (1 << 20) / max(yard)  # the yardstick moves exactly 2^20 KiB each way
+            got[counter] = (statistics.median(kernel) * factor * 1024.0, factor, len(kernel))
+        finally:
+            shutil.rmtree(out_dir, ignore_errors=True)
+    read, written = got["FETCH_SIZE"][0], got["WRITE_SIZE"][0]
+    return {"bytes": int(round(read + written)), "read_bytes": int(round(read)), "written_bytes": int(round(written)),
+            "counter_scale": {"FETCH_SIZE": round(got["FETCH_SIZE"][1], 4), "WRITE_SIZE": round(got["WRITE_SIZE"][1], 4)},
+            "launches_sampled": got["FETCH_SIZE"][2],
+            "source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over two child runs of this bench invocation's "
+                      "headline leg (median over the copy kernel's launches, KiB per dispatch scaled by a 1 GiB "
+                      "element-wise kernel in the same run)"}
 
 
 def _kv_layout():
@@ -547,6 +617,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain element-wise kernel that reads 1 GiB and writes 1 GiB, as the "
                          "known-size yardstick for hardware counter runs")
+    ap.add_argument("--no-live-traffic", action="store_true",
+                    help="do not run the headline leg under rocprofv3 --pmc first; roofline.traffic then comes from "
+                         "the counter runs summarised under profiles/")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (virtual ranks are regions of one "
@@ -555,10 +628,18 @@ def main():
     import __graft_entry__ as entry
     entry._ensure_built()
 
+    blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
+    # before this process touches the GPU: the counter runs are processes of their own
+    live = None if args.no_live_traffic else measure_traffic_live(args, blk)
     if args.calibrate_copy:
         run_calibration_copy()
-    blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
     kv = run_kv(args, blk, args.order, args.steps, args.warmup, fresh_requests=args.fresh_requests)
+    if live and "bytes" in live:
+        kv["roofline"]["traffic"] = live["bytes"]
+        kv["roofline"]["traffic_source"] = live["source"]
+        kv["roofline"]["traffic_detail"] = {k: live[k] for k in ("read_bytes", "written_bytes", "counter_scale", "launches_sampled")}
+    elif live:
+        kv["roofline"]["traffic_live_error"] = live["error"]
     tokens_per_block = blk // (_kv_layout().bytes_per_sub_block // 16)
     line = {
         "metric": "KV xfer GB/s (% HBM peak) @16KB blocks; EP dispatch+combine µs @7168 top-8",
