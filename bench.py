@@ -629,17 +629,9 @@ def main():
     entry._ensure_built()
 
     blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
-    # before this process touches the GPU: the counter runs are processes of their own
-    live = None if args.no_live_traffic else measure_traffic_live(args, blk)
     if args.calibrate_copy:
         run_calibration_copy()
     kv = run_kv(args, blk, args.order, args.steps, args.warmup, fresh_requests=args.fresh_requests)
-    if live and "bytes" in live:
-        kv["roofline"]["traffic"] = live["bytes"]
-        kv["roofline"]["traffic_source"] = live["source"]
-        kv["roofline"]["traffic_detail"] = {k: live[k] for k in ("read_bytes", "written_bytes", "counter_scale", "launches_sampled")}
-    elif live:
-        kv["roofline"]["traffic_live_error"] = live["error"]
     tokens_per_block = blk // (_kv_layout().bytes_per_sub_block // 16)
     line = {
         "metric": "KV xfer GB/s (% HBM peak) @16KB blocks; EP dispatch+combine µs @7168 top-8",
@@ -700,6 +692,16 @@ def main():
         # the reference's own loopback needs libucp, which this image does not ship
         import ctypes.util
         line["cpu_baseline"]["libucp"] = ctypes.util.find_library("ucp") or "absent"
+    # Last, when everything timed is over: the counter runs are processes of their own.  With
+    # them ahead of the timed legs this process's wall-clock figures came out at half (its
+    # kernel times unchanged); behind them they disturb nothing.
+    live = None if args.no_live_traffic else measure_traffic_live(args, blk)
+    if live and "bytes" in live:
+        line["roofline"]["traffic"] = live["bytes"]
+        line["roofline"]["traffic_source"] = live["source"]
+        line["roofline"]["traffic_detail"] = {k: live[k] for k in ("read_bytes", "written_bytes", "counter_scale", "launches_sampled")}
+    elif live:
+        line["roofline"]["traffic_live_error"] = live["error"]
     print(json.dumps(line))
 
 
