@@ -410,6 +410,63 @@ def run_small_descriptors(steps=20, warmup=3, backend_params=None):
             "kernel": "copy_piece_kernel<policy,4,1>"}
 
 
+def run_ceilings(iters=20):
+    """What this GPU gives a plain copy of 1 GiB, as context for the roofline fractions: the
+    runtime's own device-to-device copy (torch's copy_, i.e. hipMemcpyAsync) and this
+    backend's kernel on ONE contiguous 1 GiB descriptor.  HBM traffic (read + write) per
+    second, HIP events on the launch stream, caches flushed before every launch."""
+    import torch
+    from nixl_amd import nixl_agent, nixl_agent_config
+    dev = torch.device("cuda:0")
+    n = 1 << 30
+    src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=dev)
+    dst = torch.zeros(n, dtype=torch.uint8, device=dev)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.Stream(device=dev)
+    agent = nixl_agent("ceiling", nixl_agent_config(backends=()))
+    agent.create_backend("HIP", {"stream": str(stream.cuda_stream)})
+    agent.register_memory([src, dst])
+    req = agent.initialize_xfer("WRITE", agent.get_xfer_descs(src), agent.get_xfer_descs(dst), "ceiling")
+
+    def plugin():
+        state = agent.transfer(req)
+        while state == "PROC":
+            state = agent.check_xfer_state(req)
+        if state != "DONE":
+            raise RuntimeError(f"transfer ended in state {state}")
+
+    def runtime():
+        with torch.cuda.stream(stream):
+            dst.copy_(src)
+
+    out = {}
+    for name, fn in (("runtime_copy_1GiB", runtime), ("this_backend_one_1GiB_descriptor", plugin)):
+        times = []
+        for i in range(iters + 3):
+            with torch.cuda.stream(stream):
+                flush.fill_(i & 1)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            fn()
+            e1.record(stream)
+            e1.synchronize()
+            if i >= 3:
+                times.append(e0.elapsed_time(e1) * 1e-3)
+        if not torch.equal(dst, src):
+            raise RuntimeError(f"{name}: copy differs from its source")
+        dst.zero_()
+        gbps = 2 * n / float(np.mean(times)) / 1e9
+        out[name] = {"traffic_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "avg_us": round(float(np.mean(times)) * 1e6, 1)}
+    req.release()
+    agent.close()
+    del src, dst, flush
+    torch.cuda.empty_cache()
+    out["note"] = ("a plain copy of 1 GiB on this GPU, read + write per second: the runtime's device-to-device copy and this "
+                   "backend's kernel on one contiguous descriptor; context for the fractions above, not a target")
+    return out
+
+
 def run_calibration_copy():
     """One launch of torch's element-wise add over 2^28 int32: reads exactly 1 GiB, writes 1 GiB."""
     import torch
@@ -674,6 +731,8 @@ def main():
         line["kv"]["other_points"] = others
     if not args.no_small:
         line["kv"]["small_descriptor_stress"] = run_small_descriptors()
+    if not args.quick:
+        line["kv"]["plain_copy_ceilings"] = run_ceilings()
     many = min(16, os.cpu_count() or 1)
     if not args.no_ep:
         from nixl_amd import ep_bench
