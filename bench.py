@@ -41,9 +41,9 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 # reports null.
 _KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, not this run)"
 MEASURED_TRAFFIC = {
-    (1024, 8192, 16384): {"bytes": 2164231731, "source": _KV_PROFILE},
-    (1024, 8192, 32768): {"bytes": 4311687860, "source": _KV_PROFILE},
-    ("small", 262144): {"bytes": 977089988,
+    (1024, 8192, 16384): {"bytes": 2164231147, "source": _KV_PROFILE},
+    (1024, 8192, 32768): {"bytes": 4311673261, "source": _KV_PROFILE},
+    ("small", 262144): {"bytes": 977133961,
                         "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
                                   "this file, not this run)"},
 }
