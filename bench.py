@@ -649,6 +649,17 @@ def run_cpu_baseline(seconds=12.0, threads=1, blk=16384):
             "host_cpus": os.cpu_count()}
 
 
+def _leg(fn, *a, **kw):
+    """Runs one of the legs beside the headline; a leg that fails is reported in its place (and
+    on stderr) instead of taking the line, and the legs that did run, with it."""
+    try:
+        return fn(*a, **kw)
+    except Exception as e:  # noqa: BLE001 - whatever it was, the line still goes out
+        import traceback
+        traceback.print_exc()
+        return {"error": f"{type(e).__name__}: {e}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -713,41 +724,44 @@ def main():
         "kv": kv["kv"],
     }
     if not args.block_bytes and not args.quick:
-        # beside the headline: config 2 as BASELINE words it (16 tokens per block, 32 KiB), and
-        # both sizes with the descriptors listed the other way round; each with its own roofline
-        others = {}
-        other_order = "block" if args.order == "layer" else "layer"
-        for b, o in ((32768, args.order), (16384, other_order), (32768, other_order)):
-            r = run_kv(args, b, o, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2)
-            others[f"{b // 1024}KiB_{o}_order"] = {
+        def other_points():
+            # beside the headline: config 2 as BASELINE words it (16 tokens per block, 32 KiB), and
+            # both sizes with the descriptors listed the other way round; each with its own roofline
+            others = {}
+            other_order = "block" if args.order == "layer" else "layer"
+            for b, o in ((32768, args.order), (16384, other_order), (32768, other_order)):
+                r = run_kv(args, b, o, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2)
+                others[f"{b // 1024}KiB_{o}_order"] = {
+                    "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
+                    "make_request_pair_ms": r["kv"]["make_request_pair_ms"],
+                    "value_including_prepare": r["kv"]["value_including_prepare"]}
+            r = run_kv(args, blk, args.order, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2, sorted_ids=True)
+            others[f"{blk // 1024}KiB_{args.order}_order_source_blocks_ascending"] = {
                 "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
-                "make_request_pair_ms": r["kv"]["make_request_pair_ms"],
-                "value_including_prepare": r["kv"]["value_including_prepare"]}
-        r = run_kv(args, blk, args.order, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2, sorted_ids=True)
-        others[f"{blk // 1024}KiB_{args.order}_order_source_blocks_ascending"] = {
-            "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
-            "note": "the same random block sets and random destinations, the request listing its source blocks in "
-                    "ascending order: the gather then reads the pool monotonically"}
-        line["kv"]["other_points"] = others
+                "note": "the same random block sets and random destinations, the request listing its source blocks in "
+                        "ascending order: the gather then reads the pool monotonically"}
+            return others
+
+        line["kv"]["other_points"] = _leg(other_points)
     if not args.no_small:
-        line["kv"]["small_descriptor_stress"] = run_small_descriptors()
+        line["kv"]["small_descriptor_stress"] = _leg(run_small_descriptors)
     if not args.quick:
-        line["kv"]["plain_copy_ceilings"] = run_ceilings()
+        line["kv"]["plain_copy_ceilings"] = _leg(run_ceilings)
     many = min(16, os.cpu_count() or 1)
     if not args.no_ep:
         from nixl_amd import ep_bench
-        line["ep"] = ep_bench.run(args)
+        line["ep"] = _leg(ep_bench.run, args)
         if not args.no_cpu_baseline:
-            line["ep"]["cpu_baseline"] = run_ep_cpu_baseline(seconds=6.0)
+            line["ep"]["cpu_baseline"] = _leg(run_ep_cpu_baseline, seconds=6.0)
             if many > 1:
-                line["ep"]["cpu_baseline"]["all_cores_full_size"] = run_ep_cpu_baseline(threads=many, full=True)
+                line["ep"]["cpu_baseline"]["all_cores_full_size"] = _leg(run_ep_cpu_baseline, threads=many, full=True)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = run_cpu_baseline(blk=blk)
+        line["cpu_baseline"] = _leg(run_cpu_baseline, blk=blk)
         # the same path with the descriptor list split over the box's CPU share, reported beside
         if many > 1:
-            line["cpu_baseline"]["all_cores"] = run_cpu_baseline(seconds=5.0, threads=many, blk=blk)
-        line["cpu_baseline"]["config1"] = run_config1()
-        line["cpu_baseline"]["posix_path_analogue"] = run_posix_analogue()
+            line["cpu_baseline"]["all_cores"] = _leg(run_cpu_baseline, seconds=5.0, threads=many, blk=blk)
+        line["cpu_baseline"]["config1"] = _leg(run_config1)
+        line["cpu_baseline"]["posix_path_analogue"] = _leg(run_posix_analogue)
         # the reference's own loopback needs libucp, which this image does not ship
         import ctypes.util
         line["cpu_baseline"]["libucp"] = ctypes.util.find_library("ucp") or "absent"
