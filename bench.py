@@ -34,16 +34,16 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 # HBM bytes per launch of the dominant kernel from hardware counters.  Counters cannot be read
 # from inside this process.  The headline's figure is measured by measure_traffic_live below
 # (child runs under the profiler); the other points, and the headline when the profiler cannot
-# be run, take the figures of earlier rocprofv3 --pmc runs of this same file (FETCH_SIZE and
-# WRITE_SIZE, one run each, scaled by a plain 1 GiB element-wise kernel in the same run); the
-# summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks, descriptor
+# be run, take the figures of earlier rocprofv3 --pmc runs of this same file (read requests by
+# size class in one run, WRITE_SIZE in another, checked against a plain 1 GiB element-wise
+# kernel in the same run); the summaries under profiles/ name the commands.  Keyed by (blocks, pool blocks, descriptor
 # bytes) - the two descriptor orders move the same bytes; a shape without a counter run
 # reports null.
-_KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, not this run)"
+_KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc runs of this file, not this run)"
 MEASURED_TRAFFIC = {
-    (1024, 8192, 16384): {"bytes": 2164231147, "source": _KV_PROFILE},
-    (1024, 8192, 32768): {"bytes": 4311673261, "source": _KV_PROFILE},
-    ("small", 262144): {"bytes": 977133961,
+    (1024, 8192, 16384): {"bytes": 2155883520, "source": _KV_PROFILE},
+    (1024, 8192, 32768): {"bytes": 4303367840, "source": _KV_PROFILE},
+    ("small", 262144): {"bytes": 938610880,
                         "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
                                   "this file, not this run)"},
 }
@@ -51,9 +51,12 @@ MEASURED_TRAFFIC = {
 
 def measure_traffic_live(args, blk):
     """HBM bytes per launch of the headline kernel from hardware counters, measured now: the
-    headline leg of this file is run twice more as a child process under `rocprofv3 --pmc`
-    (FETCH_SIZE, then WRITE_SIZE: one counter a run), each with one plain element-wise kernel
-    of known size (1 GiB read, 1 GiB written) as the yardstick the counter is scaled by.
+    headline leg of this file is run twice more as a child process under `rocprofv3 --pmc`.
+    Reads: the L2's requests to memory by size class (TCC_EA0_RDREQ_128B / _64B / _32B, one
+    run), bytes = 128 a + 64 b + 32 c.  Writes: WRITE_SIZE (KiB per dispatch, second run).
+    Each run also holds one plain element-wise kernel of known size (1 GiB read, 1 GiB
+    written): the write counter is scaled by what it shows for that kernel, and the read
+    classes must reproduce its 1 GiB (reported as `yardstick`).
     Returns {"bytes", "source", ...}, or {"error": why} when the profiler is not there or a run
     fails; the caller then falls back to the figures of profiles/."""
     import csv
@@ -74,11 +77,12 @@ def measure_traffic_live(args, blk):
              "--pool-blocks", str(args.pool_blocks)]
     for kv in args.backend_param:
         child += ["--backend-param", kv]
+    read_classes = {"TCC_EA0_RDREQ_128B_sum": 128, "TCC_EA0_RDREQ_64B_sum": 64, "TCC_EA0_RDREQ_32B_sum": 32}
     got = {}
-    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+    for run, counters in (("read", list(read_classes)), ("write", ["WRITE_SIZE"])):
         out_dir = tempfile.mkdtemp(prefix="nixl_amd_pmc_", dir="/tmp")
         try:
-            cmd = [prof, "--pmc", counter, "--output-format", "csv", "-d", out_dir, "-o", "t", "--"] + child
+            cmd = [prof, "--pmc", *counters, "--output-format", "csv", "-d", out_dir, "-o", "t", "--"] + child
             proc = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, stdout=subprocess.DEVNULL,
                                     stderr=subprocess.DEVNULL, start_new_session=True)
             try:
@@ -86,35 +90,42 @@ def measure_traffic_live(args, blk):
             except subprocess.TimeoutExpired:
                 os.killpg(proc.pid, signal.SIGKILL)
                 proc.wait()
-                return {"error": f"the {counter} run did not finish in 150 s"}
+                return {"error": f"the {run} counter run did not finish in 150 s"}
             if rc != 0:
-                return {"error": f"the {counter} run ended with status {rc}"}
+                return {"error": f"the {run} counter run ended with status {rc}"}
             files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
             if not files:
-                return {"error": f"the {counter} run left no counter file"}
-            kernel, yard = [], []
+                return {"error": f"the {run} counter run left no counter file"}
+            kernel = {c: [] for c in counters}
+            yard = {c: [] for c in counters}
             with open(files[0], newline="") as f:
                 for row in csv.DictReader(f):
-                    if row.get("Counter_Name") != counter:
+                    c, name = row.get("Counter_Name"), row.get("Kernel_Name", "")
+                    if c not in kernel:
                         continue
-                    name = row.get("Kernel_Name", "")
                     if "copy_uniform_kernel" in name:
-                        kernel.append(float(row["Counter_Value"]))
+                        kernel[c].append(float(row["Counter_Value"]))
                     elif "CUDAFunctorOnSelf_add<int>" in name:
-                        yard.append(float(row["Counter_Value"]))
-            if not kernel or not yard or max(yard) <= 0:
-                return {"error": f"the {counter} run has no samples of the copy kernel or of the yardstick"}
-            factor = (1 << 20) / max(yard)  # the yardstick moves exactly 2^20 KiB each way
-            got[counter] = (statistics.median(kernel) * factor * 1024.0, factor, len(kernel))
+                        yard[c].append(float(row["Counter_Value"]))
+            if any(not kernel[c] or not yard[c] for c in counters):
+                return {"error": f"the {run} counter run has no samples of the copy kernel or of the yardstick"}
+            got[run] = ({c: statistics.median(kernel[c]) for c in counters}, {c: max(yard[c]) for c in counters},
+                        len(kernel[counters[0]]))
         finally:
             shutil.rmtree(out_dir, ignore_errors=True)
-    read, written = got["FETCH_SIZE"][0], got["WRITE_SIZE"][0]
+    read = sum(got["read"][0][c] * size for c, size in read_classes.items())
+    yard_read = sum(got["read"][1][c] * size for c, size in read_classes.items())
+    if got["write"][1]["WRITE_SIZE"] <= 0:
+        return {"error": "the write counter shows nothing for the yardstick"}
+    write_scale = (1 << 20) / got["write"][1]["WRITE_SIZE"]  # the yardstick writes exactly 2^20 KiB
+    written = got["write"][0]["WRITE_SIZE"] * write_scale * 1024.0
     return {"bytes": int(round(read + written)), "read_bytes": int(round(read)), "written_bytes": int(round(written)),
-            "counter_scale": {"FETCH_SIZE": round(got["FETCH_SIZE"][1], 4), "WRITE_SIZE": round(got["WRITE_SIZE"][1], 4)},
-            "launches_sampled": got["FETCH_SIZE"][2],
-            "source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over two child runs of this bench invocation's "
-                      "headline leg (median over the copy kernel's launches, KiB per dispatch scaled by a 1 GiB "
-                      "element-wise kernel in the same run)"}
+            "read_requests": {c[len("TCC_EA0_RDREQ_"):-len("_sum")]: int(got["read"][0][c]) for c in read_classes},
+            "yardstick": {"read_bytes_counted_for_1GiB": int(round(yard_read)), "write_scale": round(write_scale, 4)},
+            "launches_sampled": got["read"][2],
+            "source": "rocprofv3 --pmc over two child runs of this bench invocation's headline leg, median over the copy "
+                      "kernel's launches: reads = the L2's requests to memory by size class (TCC_EA0_RDREQ_128B/64B/32B), "
+                      "writes = WRITE_SIZE scaled by a 1 GiB element-wise kernel in the same run"}
 
 
 def _kv_layout():
@@ -772,7 +783,8 @@ def main():
     if live and "bytes" in live:
         line["roofline"]["traffic"] = live["bytes"]
         line["roofline"]["traffic_source"] = live["source"]
-        line["roofline"]["traffic_detail"] = {k: live[k] for k in ("read_bytes", "written_bytes", "counter_scale", "launches_sampled")}
+        line["roofline"]["traffic_detail"] = {k: live[k] for k in ("read_bytes", "written_bytes", "read_requests", "yardstick",
+                                                                   "launches_sampled")}
     elif live:
         line["roofline"]["traffic_live_error"] = live["error"]
     print(json.dumps(line))

@@ -61,13 +61,14 @@ struct MixedArgs {
     uint32_t n_mixed;
 };
 
-// A piece of a small descriptor: at most kPieceUnits 16-byte units, one wavefront's work.
+// A piece of a small descriptor: at most kPieceUnits (256) 16-byte units, one wavefront's work.
+// 16 bytes a record: the unit count, less one, rides in the top byte of the destination
+// address (device and pinned host addresses stay far below 2^56; the host checks it).
 struct PieceRec {
     uint64_t src;
-    uint64_t dst;
-    uint32_t units;
-    uint32_t pad;
+    uint64_t dst_units; // dst | (units - 1) << 56
 };
+constexpr int kPieceUnitsShift = 56;
 
 struct GenericItem {
     uint64_t src;
@@ -157,14 +158,22 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t first_chunk, uint32_t n_chu
 constexpr int kPieceLoads = 4;
 constexpr uint32_t kPieceUnits = kWaveSize * kPieceLoads; // 4 KiB
 
+// Workgroups are handed to the 8 dies round-robin; die x takes the x-th eighth of the records
+// (grid = a multiple of 8 workgroups, `per_die` of them a die), so that a line of records is
+// fetched into one die's cache instead of into several: with records dealt out round-robin the
+// record lines were read 3.3 times over.
 template<int POL, int LOADS, int WAVES>
 __global__ void __launch_bounds__(kWaveSize *WAVES)
-copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs) { // recs, n_recs: of this launch
+copy_piece_kernel(const PieceRec *__restrict__ recs, uint32_t n_recs, uint32_t per_die) { // recs, n_recs: of this launch
     const uint32_t lane = threadIdx.x & (kWaveSize - 1);
-    const uint32_t p = uniform(blockIdx.x * WAVES + threadIdx.x / kWaveSize);
+    const uint32_t wg = (blockIdx.x % kNumXcd) * per_die + blockIdx.x / kNumXcd;
+    const uint32_t p = uniform(wg * WAVES + threadIdx.x / kWaveSize);
     if (p >= n_recs) return;
-    const PieceRec rec = recs[p]; // same address in every lane of the wave: a scalar load
-    const uint32_t units = rec.units; // >= 1
+    const PieceRec packed = recs[p]; // same address in every lane of the wave: a scalar load
+    struct {
+        uint64_t src, dst;
+    } rec{packed.src, packed.dst_units & ((1ull << kPieceUnitsShift) - 1ull)};
+    const uint32_t units = static_cast<uint32_t>(packed.dst_units >> kPieceUnitsShift) + 1u; // >= 1
     // Lane 0 of every instruction sits on a 128-byte line of the destination: the piece's
     // units are shifted up by the destination's offset inside its line (the plan cuts pieces
     // so that shift + units <= kPieceUnits), and each store instruction then writes whole
@@ -453,14 +462,16 @@ launch_mixed_upl(int upl, dim3 grid, hipStream_t s, const MixedArgs &a) {
 
 template<int POL>
 void
-launch_pieces(uint32_t w, dim3 grid, hipStream_t s, const PieceRec *recs, uint32_t n) {
+launch_pieces(uint32_t w, uint32_t n_wgs, hipStream_t s, const PieceRec *recs, uint32_t n) {
     const dim3 block(kWaveSize * w);
+    const uint32_t per_die = (n_wgs + kNumXcd - 1) / kNumXcd;
+    const dim3 grid(per_die * kNumXcd); // surplus workgroups exit at once
     if (w == 1)
-        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 1>), grid, block, 0, s, recs, n);
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 1>), grid, block, 0, s, recs, n, per_die);
     else if (w == 2)
-        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 2>), grid, block, 0, s, recs, n);
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 2>), grid, block, 0, s, recs, n, per_die);
     else
-        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 4>), grid, block, 0, s, recs, n);
+        hipLaunchKernelGGL((copy_piece_kernel<POL, kPieceLoads, 4>), grid, block, 0, s, recs, n, per_die);
 }
 
 // Calls f.template operator()<POL>() for the plan's policy.
@@ -815,10 +826,12 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             // Pieces of at most kPieceUnits units, one wavefront each.  The first piece is
             // cut so that every later one starts on a 128-byte line of the destination: no
             // line is then written by two wavefronts.
+            if ((d.dst + d.len) >> kPieceUnitsShift)
+                return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: destination address beyond 2^56");
             const uint64_t head = kPieceUnits - ((d.dst >> 4) & 7u);
             for (uint64_t first = 0; first < du;) {
                 const uint64_t n_units = std::min<uint64_t>(first == 0 ? head : kPieceUnits, du - first);
-                pieces.push_back(PieceRec{d.src + first * 16u, d.dst + first * 16u, static_cast<uint32_t>(n_units), 0u});
+                pieces.push_back(PieceRec{d.src + first * 16u, (d.dst + first * 16u) | ((n_units - 1) << kPieceUnitsShift)});
                 first += n_units;
             }
             ++n_piece_descs;
@@ -1252,7 +1265,7 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
         for (uint32_t p0 = 0; p0 < plan->n_pieces; p0 += per_launch) {
             const uint32_t n = std::min(per_launch, plan->n_pieces - p0);
             with_policy(plan->piece_policy,
-                        [&]<int POL>() { launch_pieces<POL>(w, dim3((n + w - 1) / w), s, plan->piece_recs + p0, n); });
+                        [&]<int POL>() { launch_pieces<POL>(w, (n + w - 1) / w, s, plan->piece_recs + p0, n); });
             HIP_TRY(hipGetLastError());
         }
     }
