@@ -49,6 +49,30 @@ MEASURED_TRAFFIC = {
 }
 
 
+def counter_samples(csv_path, counters, kernel_tag="copy_uniform_kernel", yardstick_tag="CUDAFunctorOnSelf_add<int>"):
+    """Reads a rocprofv3 counter_collection.csv (one row per dispatch and counter: Kernel_Name,
+    Counter_Name, Counter_Value).  Returns ({counter: median over the kernel's dispatches},
+    {counter: largest value over the yardstick's dispatches}, number of kernel dispatches), or
+    None when either has no sample of some counter."""
+    import csv
+    import statistics
+    kernel = {c: [] for c in counters}
+    yard = {c: [] for c in counters}
+    with open(csv_path, newline="") as f:
+        for row in csv.DictReader(f):
+            c, name = row.get("Counter_Name"), row.get("Kernel_Name", "")
+            if c not in kernel:
+                continue
+            if kernel_tag in name:
+                kernel[c].append(float(row["Counter_Value"]))
+            elif yardstick_tag in name:
+                yard[c].append(float(row["Counter_Value"]))
+    if any(not kernel[c] or not yard[c] for c in counters):
+        return None
+    return ({c: statistics.median(kernel[c]) for c in counters}, {c: max(yard[c]) for c in counters},
+            len(kernel[counters[0]]))
+
+
 def measure_traffic_live(args, blk):
     """HBM bytes per launch of the headline kernel from hardware counters, measured now: the
     headline leg of this file is run twice more as a child process under `rocprofv3 --pmc`.
@@ -59,11 +83,9 @@ def measure_traffic_live(args, blk):
     classes must reproduce its 1 GiB (reported as `yardstick`).
     Returns {"bytes", "source", ...}, or {"error": why} when the profiler is not there or a run
     fails; the caller then falls back to the figures of profiles/."""
-    import csv
     import glob
     import shutil
     import signal
-    import statistics
     import subprocess
     import tempfile
     prof = shutil.which("rocprofv3")
@@ -96,21 +118,10 @@ def measure_traffic_live(args, blk):
             files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
             if not files:
                 return {"error": f"the {run} counter run left no counter file"}
-            kernel = {c: [] for c in counters}
-            yard = {c: [] for c in counters}
-            with open(files[0], newline="") as f:
-                for row in csv.DictReader(f):
-                    c, name = row.get("Counter_Name"), row.get("Kernel_Name", "")
-                    if c not in kernel:
-                        continue
-                    if "copy_uniform_kernel" in name:
-                        kernel[c].append(float(row["Counter_Value"]))
-                    elif "CUDAFunctorOnSelf_add<int>" in name:
-                        yard[c].append(float(row["Counter_Value"]))
-            if any(not kernel[c] or not yard[c] for c in counters):
+            parsed = counter_samples(files[0], counters)
+            if parsed is None:
                 return {"error": f"the {run} counter run has no samples of the copy kernel or of the yardstick"}
-            got[run] = ({c: statistics.median(kernel[c]) for c in counters}, {c: max(yard[c]) for c in counters},
-                        len(kernel[counters[0]]))
+            got[run] = parsed
         finally:
             shutil.rmtree(out_dir, ignore_errors=True)
     read = sum(got["read"][0][c] * size for c, size in read_classes.items())

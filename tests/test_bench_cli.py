@@ -11,3 +11,24 @@ def test_more_than_one_gpu_is_refused_with_a_message():
                           timeout=120)
     assert proc.returncode != 0
     assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_counter_file_of_the_profiler_is_read_per_kernel(tmp_path):
+    """bench.py takes its live traffic figure from rocprofv3's counter_collection.csv: median over the copy
+    kernel's dispatches, the yardstick kernel apart, other kernels and counters ignored."""
+    sys.path.insert(0, ROOT)
+    import bench
+    rows = [("copy_uniform_kernel<1, 4, 1>(x)", "A", 10.0), ("copy_uniform_kernel<1, 4, 1>(x)", "A", 30.0),
+            ("copy_uniform_kernel<1, 4, 1>(x)", "A", 20.0), ("copy_uniform_kernel<1, 4, 1>(x)", "B", 7.0),
+            ("void at::native::vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<int>, a>(b)", "A", 5.0),
+            ("void at::native::vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<int>, a>(b)", "A", 6.0),
+            ("void at::native::vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<int>, a>(b)", "B", 2.0),
+            ("some_other_kernel(y)", "A", 1e9), ("copy_uniform_kernel<1, 4, 1>(x)", "C", 1e9)]
+    path = tmp_path / "t_counter_collection.csv"
+    with open(path, "w") as f:
+        f.write('"Dispatch_Id","Kernel_Name","Counter_Name","Counter_Value"\n')
+        for i, (k, c, v) in enumerate(rows):
+            f.write(f'{i},"{k}","{c}",{v}\n')
+    kernel, yard, n = bench.counter_samples(str(path), ["A", "B"])
+    assert kernel == {"A": 20.0, "B": 7.0} and yard == {"A": 6.0, "B": 2.0} and n == 3
+    assert bench.counter_samples(str(path), ["A", "D"]) is None
