@@ -14,6 +14,18 @@ from .ep import Buffer
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per call from hardware counters (read requests by size class and WRITE_SIZE, summed
+# over the call's kernels): figures of rocprofv3 --pmc runs of bench.py, summarised under
+# profiles/; counters cannot be read from inside the process.
+_LL_PROFILE = "profiles/ep_low_latency_kernels_32x128x7168_top8.txt (rocprofv3 --pmc runs of bench.py, not this run)"
+_HT_PROFILE = "profiles/ep_normal_mode_kernels_8x4096x7168_top8_zipf.txt (rocprofv3 --pmc runs of bench.py, not this run)"
+MEASURED_TRAFFIC = {
+    "ll_dispatch": {"traffic": 308_300_000, "traffic_source": _LL_PROFILE},  # bits 0.7 + dispatch 297.1 + scales 10.5 MB
+    "ll_combine": {"traffic": 530_100_000, "traffic_source": _LL_PROFILE},
+    "ht_dispatch": {"traffic": 2_969_300_000, "traffic_source": _HT_PROFILE},  # scan 1.8 + rows 2949.4 + metadata 18.1 MB
+    "ht_combine": {"traffic": 2_967_600_000, "traffic_source": _HT_PROFILE},
+}
+
 
 def _timed(fn, flush, warmup, iters):
     for _ in range(warmup):
@@ -94,8 +106,8 @@ def run_low_latency(dev, warmup=20, iters=50):
     both_us = t_dispatch["avg_us"] + t_combine["avg_us"]
     return {
         "workload": f"{R} virtual ranks x {T} tokens x hidden {H}, {E} experts, top-{K}, fp8 e4m3 dispatch, bf16 combine",
-        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"])},
-        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
+        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]), **MEASURED_TRAFFIC["ll_dispatch"]},
+        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"]), **MEASURED_TRAFFIC["ll_combine"]},
         "dispatch_plus_combine_us": round(both_us, 2),
         "dispatch_plus_combine": _rate(dispatch_bytes + combine_bytes, both_us),
         "dispatch_then_combine_one_event_pair": {**t_both, **_rate(dispatch_bytes + combine_bytes, t_both["avg_us"])},
@@ -172,12 +184,12 @@ def run_normal(dev, warmup=5, iters=20):
         "rows_received": int(rows),
         "expert_load": {"max": int(counts.max()), "mean": round(float(counts.mean()), 1), "min": int(counts.min())},
         "layout": t_layout,
-        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]),
+        "dispatch": {**t_dispatch, **_rate(dispatch_bytes, t_dispatch["avg_us"]), **MEASURED_TRAFFIC["ht_dispatch"],
                      "note": "count exchange + rows + per-row metadata; receive tensors sized for the worst case, so the "
                              "host's wait for the counts (pinned memory) overlaps the row kernel"},
         "dispatch_cached_handle": {**t_cached, **_rate(tokens * H * 2 + rows * H * 2, t_cached["avg_us"]),
                                    "note": "layout of an earlier dispatch reused: rows only, no count exchange"},
-        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"])},
+        "combine": {**t_combine, **_rate(combine_bytes, t_combine["avg_us"]), **MEASURED_TRAFFIC["ht_combine"]},
         "dispatch_fp8_rows_with_scales": {**t_fp8, **_rate(fp8_bytes, t_fp8["avg_us"]),
                                           "note": "rows of 7168 fp8 bytes plus 56 fp32 scales per token"},
     }
