@@ -65,6 +65,7 @@ def run_low_latency(dev, warmup=20, iters=50):
     def dispatch():
         state["out"] = buf.dispatch(x, topk, M, E, use_fp8=True)
 
+    t_empty = _timed(lambda: None, flush, warmup, iters)  # what an event pair behind the flush shows with nothing in it
     t_router = _timed(lambda: buf.route(logits, K), flush, warmup, iters)
     t_dispatch = _timed(dispatch, flush, warmup, iters)
     (q, sc_t), cnt, handle, _, _ = state["out"]
@@ -118,6 +119,8 @@ def run_low_latency(dev, warmup=20, iters=50):
             "note": "router (logits -> top-k + softmax) included; its logits add 4.2 MB"},
         "combine_logfmt": {**t_logfmt, "note": "rows passed through the LogFMT-10 codec before accumulation"},
         "router": {**t_router, "bytes": tokens * E * 4},
+        "empty_event_pair": {**t_empty, "note": "the same timing with no call between the two events: what every figure above "
+                                                "contains besides its kernels; not subtracted anywhere"},
     }
 
 
