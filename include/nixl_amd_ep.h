@@ -51,7 +51,9 @@ nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, i
  *                          repeated expert a row of its own (kernels/nixl_ep_ll.cu:186-190); here
  *                          the repeats share one row, and the call reports it:
  *                          nixl_amd_ep_ll_dispatch_status then returns
- *                          NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT
+ *                          NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT.  Dispatch, experts and combine
+ *                          together still give the reference's result: its two rows hold the
+ *                          same data and its combine reads one of them for both selections
  *   num_tokens_per_rank    [R] int32 tokens present on each rank (<= T), or NULL = T
  *   mask_buffer            [R][R] int32 or NULL; tokens travel a -> b only if neither
  *                          mask[a][b] nor mask[b][a] is set (kernels/nixl_ep_ll.cu:197,266,319)

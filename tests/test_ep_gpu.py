@@ -735,6 +735,44 @@ def test_ll_dispatch_reports_a_repeated_expert(cuda):
     buf.dispatch(xd, torch.from_numpy(bad).to(cuda), M, E, check_duplicates=True)
 
 
+def test_ll_repeated_expert_combines_as_in_the_reference(cuda):
+    """A token that names an expert twice: the reference gives the token two rows at that expert
+    (kernels/nixl_ep_ll.cu:186-190), both hold the same data, and its combine reads, for each of
+    the two selections, the row that was written back last into the token's slot for that
+    expert (kernels/nixl_ep_ll.cu:959-1012): w1 * y + w2 * y.  Here the two selections share one
+    row, so dispatch counts one row less, and combine must give the same bytes as the oracle's
+    pipeline with the reference's slotting."""
+    R, T, H, K, E, M = 2, 40, 512, 4, 8, 48
+    x, topk, w = make_world(31, R, T, H, K, E, drop=0.0)
+    rng = np.random.default_rng(7)
+    dups = 0
+    for r in range(R):
+        for t in rng.choice(T, 6, replace=False):
+            a, b = rng.choice(K, 2, replace=False)
+            topk[r, t, b] = topk[r, t, a]
+            dups += 1
+    El = E // R
+    buf = Buffer(R, device=cuda)
+    td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
+    rx, cnt, handle, _, _ = buf.dispatch(x.to(cuda), td, M, E, use_fp8=False)
+    factor = (1 + 0.001 * torch.arange(E, device=cuda, dtype=torch.float32)).view(R, El, 1, 1)
+    valid = (torch.arange(R * M, device=cuda).view(1, 1, -1) < cnt.unsqueeze(-1)).unsqueeze(-1)
+    y = torch.where(valid, (rx.float() * factor).to(torch.bfloat16), torch.zeros_like(rx))
+    got, _, _ = buf.combine(y, td, wd, handle)
+    searched, _, _ = buf.combine(y, td, wd, tuple(handle))  # rows found through src_info instead of the row map
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), searched.view(torch.int16))
+
+    ref = eo.ll_dispatch(bits16(x), topk, E, M, use_fp8=False)  # every (token, selection) a slot of its own
+    assert int(ref["recv_count"].sum()) == R * T * K and int(cnt.sum().item()) == R * T * K - dups
+    ref_x = torch.from_numpy(ref["recv_x"].view(np.int16)).view(torch.bfloat16)
+    ref_valid = (np.arange(R * M).reshape(1, 1, -1) < ref["recv_count"][..., None])[..., None]
+    ref_y = (ref_x.float() * factor.cpu()).to(torch.bfloat16)
+    ref_y = torch.where(torch.from_numpy(ref_valid), ref_y, torch.zeros_like(ref_y))
+    want = eo.ll_combine(bits16(ref_y).reshape(R, El, R * M, H), topk, w, ref["src_info"], ref["layout_range"], E, M, use_fma=True)
+    assert np.array_equal(bits16(got).reshape(R, T, H), want)
+
+
 def test_ll_dispatch_without_tokens(cuda):
     R, H, K, E, M = 4, 512, 2, 8, 4
     x = torch.zeros((R, 0, H), dtype=torch.bfloat16)
