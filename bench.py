@@ -168,7 +168,7 @@ def _triples(addrs, blk):
     return np.stack([addrs, np.full(n, blk, np.uint64), np.zeros(n, np.uint64)], 1)
 
 
-def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False):
+def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, descriptor_path=False):
     """Gather + scatter of config 2's shape with `blk`-byte descriptors.  The pools and the
     staging buffer are prepared ONCE as descriptor lists (prep_xfer_dlist); every request is
     made from index vectors into those lists (make_prepped_xfer), the call pattern of the
@@ -216,75 +216,127 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False):
         dst_ids = rng.permutation(pool_blocks)[:n_sel]
         return sel, dst_ids, _kv_indices(lk, pool_blocks, sel, order), _kv_indices(lk, pool_blocks, dst_ids, order)
 
-    def make(src_idx, dst_idx):
-        t = time.perf_counter()
-        gather = agent.make_prepped_xfer("WRITE", h_src, src_idx, h_stg_r, stg_idx)
-        scatter = agent.make_prepped_xfer("WRITE", h_stg_l, stg_idx, h_dst, dst_idx)
-        return gather, scatter, (time.perf_counter() - t) * 1e3
+    handles = {"src": h_src, "dst": h_dst, "stg_r": h_stg_r, "stg_l": h_stg_l}
 
-    def run(req):
-        state = agent.transfer(req)
-        while state == "PROC":
-            state = agent.check_xfer_state(req)
-        if state != "DONE":
-            raise RuntimeError(f"transfer ended in state {state}")
+    def make(src_idx, dst_idx, ag=agent, h=handles):
+        t = time.perf_counter()
+        gather = ag.make_prepped_xfer("WRITE", h["src"], src_idx, h["stg_r"], stg_idx)
+        scatter = ag.make_prepped_xfer("WRITE", h["stg_l"], stg_idx, h["dst"], dst_idx)
+        return gather, scatter, (time.perf_counter() - t) * 1e3
 
     def check(sel, dst_ids):
         sel_t, dst_t = torch.from_numpy(sel).to(dev), torch.from_numpy(dst_ids).to(dev)
         if not torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16)):
             raise RuntimeError("scattered blocks differ from the source blocks")
 
-    # (b) a new block list per request pair, as a serving loop sees it: make + post + wait, wall
-    # clock, the pair released when it is done (its plan memory goes back to the engine's pool).
-    rng = np.random.default_rng(99)
-    make_ms, fresh_ms = [], []
-    for i in range(max(fresh_requests, 1) + 2):
-        sel, dst_ids, src_idx, dst_idx = block_list(rng)
+    def fresh_pairs(ag, h, rng):
+        """Request pairs with a new block list every time, as a serving loop sees them, three
+        ways.  (b) one after the other: make both requests, post and wait for the gather, post
+        and wait for the scatter; the pair is released when it is done (its plan memory goes
+        back to the engine's pool).  (b') each request posted as soon as it is made, so that
+        the gather copies while the host makes the scatter (one stream keeps the order).
+        (c) the host's share hidden altogether: the next pair is made and posted while the
+        current one copies; a pair is waited for and released one iteration later."""
+        def wait(req):
+            state = ag.check_xfer_state(req)
+            while state == "PROC":
+                state = ag.check_xfer_state(req)
+            if state != "DONE":
+                raise RuntimeError(f"transfer ended in state {state}")
+
+        def post(req):
+            if ag.transfer(req) not in ("PROC", "DONE"):
+                raise RuntimeError("post failed")
+
+        n_pairs = max(fresh_requests, 1)
+        make_ms, fresh_ms, as_made_ms = [], [], []
+        for i in range(n_pairs + 2):
+            sel, dst_ids, src_idx, dst_idx = block_list(rng)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            gather, scatter, m = make(src_idx, dst_idx, ag, h)
+            for req in (gather, scatter):
+                post(req)
+                wait(req)
+            w = (time.perf_counter() - w0) * 1e3
+            check(sel, dst_ids)
+            n_g, bytes_g = gather.desc_count()
+            assert bytes_g == n_desc * blk and n_g <= n_desc  # neighbouring blocks may have been merged
+            gather.release()
+            scatter.release()
+            if i >= 2:  # the first pairs also pay one-off allocations
+                make_ms.append(m)
+                fresh_ms.append(w)
+        for i in range(n_pairs):
+            sel, dst_ids, src_idx, dst_idx = block_list(rng)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            gather = ag.make_prepped_xfer("WRITE", h["src"], src_idx, h["stg_r"], stg_idx)
+            post(gather)
+            scatter = ag.make_prepped_xfer("WRITE", h["stg_l"], stg_idx, h["dst"], dst_idx)
+            post(scatter)
+            wait(gather)
+            wait(scatter)
+            as_made_ms.append((time.perf_counter() - w0) * 1e3)
+            check(sel, dst_ids)
+            gather.release()
+            scatter.release()
+        lists = [block_list(rng) for _ in range(n_pairs + 4)]
         torch.cuda.synchronize()
         w0 = time.perf_counter()
-        gather, scatter, m = make(src_idx, dst_idx)
-        run(gather)
-        run(scatter)
-        w = (time.perf_counter() - w0) * 1e3
-        check(sel, dst_ids)
-        n_g, bytes_g = gather.desc_count()
-        assert bytes_g == n_desc * blk and n_g <= n_desc  # neighbouring blocks may have been merged
-        gather.release()
-        scatter.release()
-        if i >= 2:  # the first pairs also pay one-off allocations
-            make_ms.append(m)
-            fresh_ms.append(w)
-    # (c) the same serving loop with the host's share hidden: the next pair is made and posted
-    # while the current one copies (both requests of a pair and all pairs go to one stream, so
-    # they run in the order posted); a pair is waited for and released one iteration later.
-    lists = [block_list(rng) for _ in range(max(fresh_requests, 1) + 4)]
+        in_flight = None
+        for sel, dst_ids, src_idx, dst_idx in lists:
+            gather, scatter, _ = make(src_idx, dst_idx, ag, h)
+            post(gather)
+            post(scatter)
+            if in_flight is not None:
+                for req in in_flight:
+                    wait(req)
+                    req.release()
+            in_flight = (gather, scatter)
+        for req in in_flight:
+            wait(req)
+        pipelined_ms = (time.perf_counter() - w0) * 1e3 / len(lists)
+        check(*lists[-1][:2])
+        for req in in_flight:
+            req.release()
 
-    def wait(req):
-        state = agent.check_xfer_state(req)
-        while state == "PROC":
-            state = agent.check_xfer_state(req)
-        if state != "DONE":
-            raise RuntimeError(f"transfer ended in state {state}")
+        def rate(ms):
+            return round(2 * n_desc * blk / (ms * 1e-3) / 1e9, 1)
 
-    torch.cuda.synchronize()
-    w0 = time.perf_counter()
-    in_flight = None
-    for sel, dst_ids, src_idx, dst_idx in lists:
-        gather, scatter, _ = make(src_idx, dst_idx)
-        for req in (gather, scatter):
-            if agent.transfer(req) not in ("PROC", "DONE"):
-                raise RuntimeError("post failed")
-        if in_flight is not None:
-            for req in in_flight:
-                wait(req)
-                req.release()
-        in_flight = (gather, scatter)
-    for req in in_flight:
-        wait(req)
-    pipelined_ms = (time.perf_counter() - w0) * 1e3 / len(lists)
-    check(*lists[-1][:2])
-    for req in in_flight:
-        req.release()
+        return {"make_request_pair_ms": round(float(np.mean(make_ms)), 3),
+                "value_including_prepare": rate(float(np.mean(fresh_ms))),
+                "value_including_prepare_note": f"new block list per request pair: make_prepped_xfer x2, then post + wait "
+                                                f"of each, mean of {len(fresh_ms)} pairs, wall clock",
+                "value_including_prepare_posted_as_made": rate(float(np.mean(as_made_ms))),
+                "value_including_prepare_posted_as_made_note": "the same, each request posted as soon as it is made: the gather "
+                                                               "copies while the host makes the scatter",
+                "value_including_prepare_pipelined": rate(pipelined_ms),
+                "value_including_prepare_pipelined_note": f"the same, the next pair made and posted while the current one "
+                                                          f"copies: wall clock over {len(lists)} pairs back to back"}
+
+    rng = np.random.default_rng(99)
+    fresh = fresh_pairs(agent, handles, rng)
+    # The same loops with every request written out as descriptors and passed through prepXfer:
+    # what an agent that knows nothing of this plugin's index entry does (the reference's
+    # makeXferReq, src/core/nixl_agent.cpp:799-880).  A second agent over the same memory whose
+    # backend has that entry switched off.
+    through_prepxfer = None
+    if descriptor_path:
+        agent_d = nixl_agent("bench_d", nixl_agent_config(backends=()))
+        agent_d.create_backend("HIP", {"stream": str(stream.cuda_stream), "indexed_prep": "0",
+                                       **dict(kv.split("=", 1) for kv in args.backend_param)})
+        agent_d.register_memory([src_pool, dst_pool, staging])
+        handles_d = {"src": agent_d.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM"),
+                     "dst": agent_d.prep_xfer_dlist("bench_d", _triples(np.uint64(dst_pool.data_ptr()) + pool_offsets, blk), "VRAM"),
+                     "stg_r": agent_d.prep_xfer_dlist("bench_d", _triples(stg_addrs, blk), "VRAM"),
+                     "stg_l": agent_d.prep_xfer_dlist("", _triples(stg_addrs, blk), "VRAM")}
+        through_prepxfer = fresh_pairs(agent_d, handles_d, np.random.default_rng(98))
+        through_prepxfer["entry"] = ("nixlBackendEngine::prepXfer with two lists of written-out descriptors a request "
+                                    "(backend parameter indexed_prep=0): what an unchanged libnixl calls")
+        for hd in handles_d.values():
+            hd.release()
+        agent_d.close()
     # the pairs of the steady-state measurement below, over different block sets
     pairs = []
     for i in range(max(fresh_requests, 1)):
@@ -352,13 +404,9 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False):
         "kv": {"descriptors_per_request": n_desc, "descriptor_bytes": blk, "descriptor_order": order,
                "prepared_list_descriptors": {"pool": n_pool, "staging": n_desc},
                "prep_dlist_ms_once": round(prep_dlist_ms, 2),
-               "make_request_pair_ms": round(float(np.mean(make_ms)), 3),
-               "value_including_prepare": round(payload_per_step / (float(np.mean(fresh_ms)) * 1e-3) / 1e9, 1),
-               "value_including_prepare_note": f"new block list per request pair: make_prepped_xfer x2 + post + wait, "
-                                               f"mean of {len(fresh_ms)} pairs, wall clock",
-               "value_including_prepare_pipelined": round(payload_per_step / (pipelined_ms * 1e-3) / 1e9, 1),
-               "value_including_prepare_pipelined_note": f"the same, the next pair made and posted while the current one "
-                                                         f"copies: wall clock over {len(lists)} pairs back to back",
+               **fresh,
+               "entry": "nixl_hip_prep_xfer_indexed (this plugin's own entry: index vectors lowered on the device)",
+               **({"through_prepxfer": through_prepxfer} if through_prepxfer else {}),
                "block_sets_timed": len(pairs),
                "scatter_ms_by_block_set": [round(float(np.mean(kernel_ms[2 * k + 1::2 * len(pairs)])), 4) for k in range(len(pairs))],
                "post_us": {"avg": round(float(np.mean(post_us)), 1), "p99": round(float(np.percentile(post_us, 99)), 1)},
@@ -372,6 +420,107 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False):
     agent.close()
     del src_pool, dst_pool, staging
     torch.cuda.empty_cache()
+    return out
+
+
+def run_prep_breakdown_child(args, blk):
+    """Child side of measure_prep_breakdown: requests of the headline's shape made through
+    prepXfer (indexed_prep=0), each posted, waited for and released; prints the wall time of
+    every make_prepped_xfer call.  The phase timings come out on stderr as the debug lines of
+    the agent and of the plugin (NIXL_LOG_LEVEL=DEBUG, set by the parent)."""
+    import torch
+    from nixl_amd import nixl_agent, nixl_agent_config
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    kv = _kv_layout()
+    pool_blocks, n_sel = args.pool_blocks, args.blocks
+    lk = kv.layers * kv.sub_blocks_per_layer
+    src_pool = torch.zeros((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+    dst_pool = torch.zeros((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+    staging = torch.zeros((n_sel * lk, blk // 2), dtype=torch.bfloat16, device=dev)
+    agent = nixl_agent("bench_d", nixl_agent_config(backends=()))
+    agent.create_backend("HIP", {"indexed_prep": "0", **dict(kv.split("=", 1) for kv in args.backend_param)})
+    agent.register_memory([src_pool, dst_pool, staging])
+    n_desc, n_pool = n_sel * lk, lk * pool_blocks
+    pool_offsets = np.arange(n_pool, dtype=np.uint64) * np.uint64(blk)
+    stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
+    h_src = agent.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+    h_dst = agent.prep_xfer_dlist("bench_d", _triples(np.uint64(dst_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+    h_stg_r = agent.prep_xfer_dlist("bench_d", _triples(stg_addrs, blk), "VRAM")
+    h_stg_l = agent.prep_xfer_dlist("", _triples(stg_addrs, blk), "VRAM")
+    stg_idx = np.arange(n_desc, dtype=np.int32)
+    rng = np.random.default_rng(7)
+    wall_us = []
+    for _ in range(10):
+        sel = rng.choice(pool_blocks, n_sel, replace=False)
+        dst_ids = rng.permutation(pool_blocks)[:n_sel]
+        for local, li, remote, ri in ((h_src, _kv_indices(lk, pool_blocks, sel, args.order), h_stg_r, stg_idx),
+                                      (h_stg_l, stg_idx, h_dst, _kv_indices(lk, pool_blocks, dst_ids, args.order))):
+            t0 = time.perf_counter()
+            req = agent.make_prepped_xfer("WRITE", local, li, remote, ri)
+            wall_us.append((time.perf_counter() - t0) * 1e6)
+            state = agent.transfer(req)
+            while state == "PROC":
+                state = agent.check_xfer_state(req)
+            req.release()
+    print(json.dumps({"make_prepped_xfer_wall_us": wall_us, "descriptors": n_desc}))
+    for h in (h_src, h_dst, h_stg_r, h_stg_l):
+        h.release()
+    agent.close()
+
+
+def parse_prep_debug_lines(text):
+    """The phase timings in the debug output of the agent (makeXferReq) and of the plugin
+    (prepXfer), one entry per request: lists of microseconds by phase."""
+    import re
+    phases = {"agent_expand_index_pairs": [], "plugin_block_pass": [], "plugin_plan_from_records": [], "plugin_rest": []}
+    paths = []
+    for line in text.splitlines():
+        m = re.search(r"makeXferReq: merged \d+ indices into \d+ descriptors in ([0-9.e+-]+) us", line)
+        if m:
+            phases["agent_expand_index_pairs"].append(float(m.group(1)))
+        m = re.search(r"prepXfer of \d+ descriptors \((\w+)\): block pass ([0-9.e+-]+) us, plan from records ([0-9.e+-]+) us, "
+                      r"rest \([^)]*\) ([0-9.e+-]+) us", line)
+        if m:
+            paths.append(m.group(1))
+            for key, value in zip(("plugin_block_pass", "plugin_plan_from_records", "plugin_rest"), m.groups()[1:]):
+                phases[key].append(float(value))
+    return phases, paths
+
+
+def measure_prep_breakdown(args, blk):
+    """Where the time of one request made through prepXfer goes, per phase, in microseconds
+    (median over the requests of a child run of this file with the libraries' debug lines on):
+    the agent's expansion of the index pairs into two descriptor lists, the plugin's pass over
+    those lists (checks against the registrations + records written to the pinned upload
+    buffer), the plan made from the records (arena, queued upload and sort, events), and what is
+    left of the call's wall time (C wrapper, ctypes, copies of the index vectors)."""
+    import subprocess
+    child = [sys.executable, os.path.abspath(__file__), "--prep-breakdown-child", "--block-bytes", str(blk), "--order", args.order,
+             "--blocks", str(args.blocks), "--pool-blocks", str(args.pool_blocks)]
+    for kv in args.backend_param:
+        child += ["--backend-param", kv]
+    try:
+        proc = subprocess.run(child, env={**os.environ, "NIXL_LOG_LEVEL": "DEBUG"}, capture_output=True, text=True, timeout=180)
+    except subprocess.TimeoutExpired:
+        return {"error": "the child run did not finish in 180 s"}
+    if proc.returncode != 0:
+        return {"error": f"the child run ended with status {proc.returncode}: {proc.stderr[-300:]}"}
+    phases, paths = parse_prep_debug_lines(proc.stderr)
+    try:
+        report = json.loads(proc.stdout.strip().splitlines()[-1])
+    except (ValueError, IndexError):
+        return {"error": "the child run printed no timings"}
+    wall = report["make_prepped_xfer_wall_us"][4:]  # the first requests also pay one-off allocations
+    if not wall or any(len(v) < len(report["make_prepped_xfer_wall_us"]) for v in phases.values()):
+        return {"error": "debug lines missing from the child run"}
+    out = {k: round(float(np.median(v[4:])), 1) for k, v in phases.items()}
+    out["make_prepped_xfer_wall"] = round(float(np.median(wall)), 1)
+    out["wrapper_and_other"] = round(out["make_prepped_xfer_wall"] - sum(out[k] for k in phases), 1)
+    out["plugin_prepxfer_total"] = round(out["plugin_block_pass"] + out["plugin_plan_from_records"] + out["plugin_rest"], 1)
+    out["descriptors_per_request"] = report["descriptors"]
+    out["plugin_path"] = sorted(set(paths))
+    out["source"] = "median over the requests of a child run of this file with NIXL_LOG_LEVEL=DEBUG (phase timers of agent and plugin)"
     return out
 
 
@@ -707,6 +856,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain element-wise kernel that reads 1 GiB and writes 1 GiB, as the "
                          "known-size yardstick for hardware counter runs")
+    ap.add_argument("--prep-breakdown-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-live-traffic", action="store_true",
                     help="do not run the headline leg under rocprofv3 --pmc first; roofline.traffic then comes from "
                          "the counter runs summarised under profiles/")
@@ -719,9 +869,13 @@ def main():
     entry._ensure_built()
 
     blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
+    if args.prep_breakdown_child:
+        run_prep_breakdown_child(args, blk)
+        return
     if args.calibrate_copy:
         run_calibration_copy()
-    kv = run_kv(args, blk, args.order, args.steps, args.warmup, fresh_requests=args.fresh_requests)
+    kv = run_kv(args, blk, args.order, args.steps, args.warmup, fresh_requests=args.fresh_requests,
+                descriptor_path=not args.quick)
     tokens_per_block = blk // (_kv_layout().bytes_per_sub_block // 16)
     line = {
         "metric": "KV xfer GB/s (% HBM peak) @16KB blocks; EP dispatch+combine µs @7168 top-8",
@@ -790,6 +944,8 @@ def main():
     # Last, when everything timed is over: the counter runs are processes of their own.  With
     # them ahead of the timed legs this process's wall-clock figures came out at half (its
     # kernel times unchanged); behind them they disturb nothing.
+    if not args.quick:
+        line["kv"]["through_prepxfer"]["prep_breakdown_us"] = _leg(measure_prep_breakdown, args, blk)
     live = None if args.no_live_traffic else measure_traffic_live(args, blk)
     if live and "bytes" in live:
         line["roofline"]["traffic"] = live["bytes"]

@@ -30,7 +30,7 @@ enum nixl_amd_status {
     NIXL_AMD_ERR_INVALID = -1, /* bad argument (null pointer, zero count, bad variant) */
     NIXL_AMD_ERR_HIP = -2, /* a HIP runtime call failed; see nixl_amd_last_error() */
     NIXL_AMD_ERR_NO_DEVICE = -3, /* no gfx950-class device visible */
-    NIXL_AMD_ERR_BUSY = -4, /* plan destroyed or relaunched while still running */
+    NIXL_AMD_ERR_BUSY = -4, /* plan destroyed while one of its launches has not completed */
     NIXL_AMD_ERR_TOO_LARGE = -5 /* request exceeds a documented fixed limit */
 };
 
@@ -134,6 +134,60 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
                                        const nixl_amd_copy_tuning_t *tuning,
                                        nixl_amd_copy_plan_t **out);
 
+/* A plan of equal blocks from records the CALLER writes: what a backend's prepXfer does when
+ * it checks the two nixl_meta_dlist_t of a request (src/api/cpp/backend/backend_engine.h:135-141)
+ * in one pass and every descriptor pair is the same length.  nixl_amd_copy_records_begin hands
+ * out room for `max_records` {src, dst} pairs in a pinned upload buffer of the library's
+ * (recycled between requests); the caller fills records[0 .. n) and passes the handle to
+ * nixl_amd_copy_plan_create_from_records, which checks the records (whole chunks of at least
+ * 8 KiB, every address on a 128-byte line, none null, no range that wraps:
+ * NIXL_AMD_ERR_INVALID otherwise), reads the destination and source patterns from them and
+ * queues their copy to the device without waiting for it, or to nixl_amd_copy_records_abandon.
+ * Either call consumes the handle, whatever it returns.  No reference counterpart: the
+ * reference's backends keep the descriptor lists and walk them at post time
+ * (src/plugins/ucx/ucx_backend.cpp:1216-1244). */
+typedef struct nixl_amd_copy_record {
+    uint64_t src;
+    uint64_t dst;
+} nixl_amd_copy_record_t;
+
+typedef struct nixl_amd_copy_records nixl_amd_copy_records_t;
+
+/* What a caller that looked at every record while writing it already knows, so that the
+ * library does not read them all again: the OR of every src and dst address (its low seven
+ * bits must be zero), of `steps` pairs of consecutive records (all of them, or a sample:
+ * the counts only decide cache policy and record order by majority) how many advance the
+ * destination regularly (by one block, or by the same amount as the pair before) and how many
+ * advance the source by exactly one block.  Passing it also states that every record lies in
+ * memory the device can address (not null, not wrapping): a backend knows that from its
+ * registrations.  NULL makes the library find all of this out itself. */
+typedef struct nixl_amd_copy_record_facts {
+    uint64_t address_bits;
+    uint64_t regular_dst_steps;
+    uint64_t following_src_steps;
+    uint64_t steps;
+} nixl_amd_copy_record_facts_t;
+
+int
+nixl_amd_copy_records_begin(size_t max_records, nixl_amd_copy_records_t **out, nixl_amd_copy_record_t **records);
+
+int
+nixl_amd_copy_plan_create_from_records(nixl_amd_copy_records_t *records,
+                                       size_t n,
+                                       uint64_t len,
+                                       int device,
+                                       const nixl_amd_copy_tuning_t *tuning,
+                                       const nixl_amd_copy_record_facts_t *facts,
+                                       nixl_amd_copy_plan_t **out);
+
+int
+nixl_amd_copy_records_abandon(nixl_amd_copy_records_t *records);
+
+/* 1 if equal blocks of `len` bytes can make such a plan under `tuning` (a whole number of
+ * chunks, at least 8 KiB), else 0: lets a caller decide before it writes any record. */
+int
+nixl_amd_copy_block_len_fits(uint64_t len, const nixl_amd_copy_tuning_t *tuning);
+
 /* Enqueue the whole plan on `stream`: the per-post work of
  * nixlUcxEngine::postXfer -> sendXferRange (src/plugins/ucx/ucx_backend.cpp:1183-1310).
  * Re-launching re-reads the current source bytes; nothing is cached at plan creation
@@ -141,7 +195,11 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
 int
 nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream);
 
-/* Free the plan's device arrays.  The caller must have synchronised with every launch. */
+/* Free the plan's device arrays.  While a launch of the plan has not completed the call
+ * returns NIXL_AMD_ERR_BUSY and leaves the plan as it is (its arrays would go back to a pool
+ * that the next plan's upload writes into): wait for the launch, then destroy again.  Launches
+ * recorded into a HIP graph are not tracked: their owner keeps the plan for as long as the
+ * graph may be replayed. */
 int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan);
 

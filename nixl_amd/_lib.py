@@ -44,6 +44,15 @@ class CopyRun(Structure):
     _fields_ = [("base", c_uint64), ("stride", c_uint64), ("first_index", c_uint64), ("count", c_uint64)]
 
 
+class CopyRecord(Structure):
+    _fields_ = [("src", c_uint64), ("dst", c_uint64)]
+
+
+class CopyRecordFacts(Structure):
+    _fields_ = [("address_bits", c_uint64), ("regular_dst_steps", c_uint64), ("following_src_steps", c_uint64),
+                ("steps", c_uint64)]
+
+
 class CopyPlanInfo(Structure):
     _fields_ = [("payload_bytes", c_uint64), ("vec_descs", c_uint64), ("generic_descs", c_uint64),
                 ("plan_device_bytes", c_uint64), ("vec_chunks", c_uint32),
@@ -72,6 +81,14 @@ def kernels():
                                                            c_void_p, c_size_t, c_uint64, c_int, POINTER(CopyTuning),
                                                            POINTER(c_void_p)]
     lib.nixl_amd_copy_plan_create_indexed_runs.restype = c_int
+    lib.nixl_amd_copy_records_begin.argtypes = [c_size_t, POINTER(c_void_p), POINTER(POINTER(CopyRecord))]
+    lib.nixl_amd_copy_plan_create_from_records.argtypes = [c_void_p, c_size_t, c_uint64, c_int, POINTER(CopyTuning),
+                                                           POINTER(CopyRecordFacts), POINTER(c_void_p)]
+    lib.nixl_amd_copy_records_abandon.argtypes = [c_void_p]
+    lib.nixl_amd_copy_block_len_fits.argtypes = [c_uint64, POINTER(CopyTuning)]
+    for fn in ("nixl_amd_copy_records_begin", "nixl_amd_copy_plan_create_from_records", "nixl_amd_copy_records_abandon",
+               "nixl_amd_copy_block_len_fits"):
+        getattr(lib, fn).restype = c_int
     lib.nixl_amd_copy_plan_launch.argtypes = [c_void_p, c_void_p]
     lib.nixl_amd_copy_plan_destroy.argtypes = [c_void_p]
     lib.nixl_amd_copy_plan_query.argtypes = [c_void_p, POINTER(CopyPlanInfo)]
@@ -128,7 +145,8 @@ def ep_kernels():
 
 def kernel_symbols():
     return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create", "nixl_amd_copy_plan_create_indexed",
-                   "nixl_amd_copy_plan_create_indexed_runs",
+                   "nixl_amd_copy_plan_create_indexed_runs", "nixl_amd_copy_records_begin",
+                   "nixl_amd_copy_plan_create_from_records", "nixl_amd_copy_records_abandon", "nixl_amd_copy_block_len_fits",
                    "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
                    "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
 

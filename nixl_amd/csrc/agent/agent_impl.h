@@ -143,6 +143,57 @@ public:
     const descs_t descs;
 };
 
+// Storage of the descriptor lists a request made from index vectors carries.  A paged-KV
+// request names tens of thousands of blocks, so its two lists are a few MiB that would be
+// allocated, faulted in page by page, filled and freed once per request; instead the
+// element vectors of released requests are kept (a few, up to a byte limit) and handed to
+// the next request with their pages already resident.
+class nixlDescStoragePool {
+public:
+    using storage_t = std::vector<nixlMetaDesc>;
+
+    static nixlDescStoragePool &
+    instance();
+
+    // Gives `list` element storage of exactly `count` entries, contents unspecified.
+    void
+    adopt(nixl_meta_dlist_t &list, size_t count);
+    // Takes the element storage of `list` back (the list is left empty).
+    void
+    surrender(nixl_meta_dlist_t &list);
+
+    static nixlMetaDesc *
+    data(nixl_meta_dlist_t &list) {
+        return storageOf(list).data();
+    }
+
+    static void
+    shrink(nixl_meta_dlist_t &list, size_t count) {
+        storageOf(list).resize(count);
+    }
+
+private:
+    // The element vector is a protected member of the list class (the reference's layout).
+    struct opened : nixl_meta_dlist_t {
+        static storage_t nixl_meta_dlist_t::*
+        member() {
+            return &opened::descs;
+        }
+    };
+
+    static storage_t &
+    storageOf(nixl_meta_dlist_t &list) {
+        return list.*opened::member();
+    }
+
+    static constexpr size_t kMaxKept = 8;
+    static constexpr size_t kMaxKeptBytes = size_t{64} << 20;
+    static constexpr size_t kMinPooled = 1024; // smaller lists are cheaper to allocate than to share
+    std::mutex mutex_;
+    std::vector<storage_t> kept_;
+    size_t keptBytes_ = 0;
+};
+
 class nixlXferReqH {
 public:
     nixlXferReqH(const std::string &remote_agent, nixl_xfer_op_t op, nixl_mem_t local_type, nixl_mem_t remote_type)
@@ -157,6 +208,9 @@ public:
 
     ~nixlXferReqH() {
         if (backendHandle && engine) engine->releaseReqH(backendHandle);
+        // only after the backend let go of the request: it may keep references to the lists
+        nixlDescStoragePool::instance().surrender(initiatorDescs);
+        nixlDescStoragePool::instance().surrender(targetDescs);
     }
 
     nixlBackendEngine *engine = nullptr;

@@ -4,8 +4,9 @@
 // Data layout of a plan in HBM
 //   16-byte-aligned descriptors of 256 B to 8 KiB, and longer ones whose source or
 //   destination does not start on a 128-byte line, become pieces of at most 4 KiB: a
-//   24-byte record {src, dst, units} and one wavefront each (wavefront-per-descriptor for
-//   anything up to 4 KiB); pieces after the first start on a destination line.
+//   16-byte record {src, dst | (units - 1) << 56} and one wavefront each
+//   (wavefront-per-descriptor for anything up to 4 KiB); pieces after the first start on a
+//   destination line.
 //   The other 16-byte-aligned descriptors (long and line-aligned, or tiny) are
 //   concatenated, in request order, into one virtual stream measured in 16-byte units.  The stream is cut into chunks of
 //   64*UPL units; one wavefront moves one chunk: lane l moves units k*64 + l of the chunk,
@@ -609,6 +610,11 @@ struct nixl_amd_copy_plan {
     // kernels queued on the upload stream, `uploaded` is recorded behind them, and the first
     // launches wait for it on their own stream.
     hipEvent_t uploaded = nullptr;
+    // Recorded behind the kernels of every launch (not on a capturing stream): destroying the
+    // plan while it has not completed is refused, because the arena would go back to the pool
+    // and the next plan's upload would overwrite records a running kernel still reads.
+    hipEvent_t launched = nullptr;
+    bool launched_valid = false;
 };
 
 // Pinned buffers whose contents are still travelling to the device: each goes back to the
@@ -671,6 +677,143 @@ settle_upload(nixl_amd_copy_plan *plan, bool wait) {
     return e;
 }
 
+struct Tuning {
+    int upl = 1, nt = 0, waves = 1, swizzle = 0, sort_scatter = 0;
+    uint32_t max_wgs = 0;
+};
+
+// Defaults from a sweep on MI355X: the smallest chunk (one 128-bit load and store per lane,
+// one wave per workgroup) gave the highest HBM rate; the cache policy follows the
+// destination pattern.
+static int
+parse_tuning(const nixl_amd_copy_tuning_t *tuning, Tuning &t, const char *who) {
+    if (tuning) {
+        if (tuning->units_per_lane) t.upl = tuning->units_per_lane;
+        if (tuning->nontemporal) t.nt = tuning->nontemporal;
+        if (tuning->max_workgroups > 0) t.max_wgs = static_cast<uint32_t>(tuning->max_workgroups);
+        if (tuning->waves_per_workgroup) t.waves = tuning->waves_per_workgroup;
+        if (tuning->xcd_swizzle) t.swizzle = tuning->xcd_swizzle == 1 ? 1 : 0;
+        t.sort_scatter = tuning->sort_scatter;
+    }
+    if (t.upl != 1 && t.upl != 2 && t.upl != 4 && t.upl != 8 && t.upl != 16)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, std::string(who) + ": units_per_lane must be 1, 2, 4, 8 or 16");
+    if (t.nt < 0 || t.nt > 4) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, std::string(who) + ": nontemporal must be 0 to 4");
+    if (t.waves != 1 && t.waves != 2 && t.waves != 4 && t.waves != 8 && t.waves != 16)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, std::string(who) + ": waves_per_workgroup must be 1, 2, 4, 8 or 16");
+    return NIXL_AMD_OK;
+}
+
+// Whether equal blocks of `len` bytes can be a plan of one record per block: whole chunks,
+// long enough that a record is small next to its payload.
+static bool
+block_len_fits(uint64_t len, const Tuning &t) {
+    const uint64_t chunk_bytes = static_cast<uint64_t>(kWaveSize) * t.upl * 16u;
+    return len >= 8192 && len % chunk_bytes == 0;
+}
+
+constexpr int kNotBlocks = 1; // build_block_plan: the records are not what a block plan takes (no error recorded)
+
+// A plan of `n_recs` equal blocks of `len` bytes whose {src, dst} records the host has written
+// to the start of the pinned buffer `staging`.  One vectorisable pass over the records checks
+// them (every address on a 128-byte line, none null, no range that wraps) and reads the
+// pattern of the destinations (cache policy) and of the sources (record order); the copy to the
+// device, the optional sort and the event behind them are queued on the upload stream and not
+// waited for.  `staging` is taken over in every case.  Returns kNotBlocks when the records do
+// not qualify, so that the caller can lower the request the general way.
+static int
+build_block_plan(int device, const Tuning &t, void *staging, size_t staging_cap, size_t n_recs, uint64_t len, size_t n_descs,
+                 const nixl_amd_copy_record_facts_t *facts, nixl_amd_copy_plan_t **out) {
+    const uint64_t chunk_bytes = static_cast<uint64_t>(kWaveSize) * t.upl * 16u;
+    const auto *recs = static_cast<const UniformRec *>(staging);
+    bool fits = n_recs > 0 && block_len_fits(len, t) && n_recs < (1ull << 31) && n_recs * (len / chunk_bytes) < (1ull << 32);
+    uint64_t regular = 0, src_follows = 0, steps = n_recs ? n_recs - 1 : 0;
+    if (fits && facts) {
+        // the caller looked at every record while it wrote them
+        fits = (facts->address_bits & 127u) == 0;
+        regular = facts->regular_dst_steps;
+        src_follows = facts->following_src_steps;
+        steps = facts->steps;
+    } else if (fits) {
+        uint64_t misfit = 0;
+        for (size_t i = 0; i < n_recs; ++i) {
+            const uint64_t a = recs[i].src, b = recs[i].dst;
+            misfit |= ((a | b) & 127u) | static_cast<uint64_t>(a == 0) | static_cast<uint64_t>(b == 0) |
+                static_cast<uint64_t>(a + len < a) | static_cast<uint64_t>(b + len < b);
+        }
+        fits = misfit == 0;
+        // Destination steps that are regular (one block on, or the same step as the one before)
+        // and source steps that go one block on; nothing is carried from one iteration to the
+        // next, so that the loop vectorises.
+        if (n_recs > 1) {
+            regular += (recs[1].dst - recs[0].dst) == len;
+            src_follows += (recs[1].src - recs[0].src) == len;
+        }
+        for (size_t i = 2; i < n_recs; ++i) {
+            const uint64_t step = recs[i].dst - recs[i - 1].dst, before = recs[i - 1].dst - recs[i - 2].dst;
+            regular += static_cast<uint32_t>(step == len) | static_cast<uint32_t>(step == before);
+            src_follows += static_cast<uint32_t>((recs[i].src - recs[i - 1].src) == len);
+        }
+    }
+    if (!fits) {
+        upload_cache().put(device, staging, staging_cap);
+        return kNotBlocks;
+    }
+    const size_t bytes = n_recs * sizeof(UniformRec);
+    auto *plan = new nixl_amd_copy_plan();
+    plan->device = device;
+    plan->upl = t.upl;
+    plan->waves = t.waves;
+    plan->swizzle = t.swizzle;
+    plan->max_wgs = t.max_wgs;
+    // cache policy by destination pattern, as in the general lowering
+    const bool scattered = !(steps == 0 || 2 * regular >= steps);
+    // a scatter out of consecutive memory is put into ascending destination order, window by window
+    const bool sort = scattered && t.sort_scatter != 2 && 2 * src_follows >= steps && n_recs >= kSortWindow;
+    plan->policy = t.nt ? t.nt : ((!scattered || sort) ? kPolNtSc1Nt : kPolPlainSc1Nt);
+    hipStream_t up = nullptr;
+    hipError_t e = arena_cache().get(device, bytes, &plan->arena, &plan->arena_cap);
+    if (e == hipSuccess) e = upload_stream(device, &up);
+    if (e == hipSuccess) e = hipMemcpyAsync(plan->arena, staging, bytes, hipMemcpyHostToDevice, up);
+    if (e == hipSuccess && sort) {
+        hipLaunchKernelGGL(sort_records_kernel, dim3(static_cast<uint32_t>((n_recs + kSortWindow - 1) / kSortWindow)),
+                           dim3(kSortWindow / 2), 0, up, static_cast<UniformRec *>(plan->arena), static_cast<uint32_t>(n_recs));
+        e = hipGetLastError();
+    }
+    // No wait here: the event goes behind the copy, launches wait for it on their stream.
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
+    if (e != hipSuccess) {
+        if (up) (void)hipStreamSynchronize(up); // whatever was queued reads the buffers given back below
+        if (plan->uploaded) (void)hipEventDestroy(plan->uploaded);
+        upload_cache().put(device, staging, staging_cap);
+        if (plan->arena) arena_cache().put(device, plan->arena, plan->arena_cap);
+        delete plan;
+        return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan upload: ") + hipGetErrorString(e));
+    }
+    recycle_after(device, up, staging, staging_cap);
+    plan->arena_bytes = bytes;
+    plan->uniform_recs = static_cast<const UniformRec *>(plan->arena);
+    plan->chunks_per_rec = static_cast<uint32_t>(len / chunk_bytes);
+    plan->n_uniform = static_cast<uint32_t>(n_recs * plan->chunks_per_rec);
+    plan->uniform_wgs = (plan->n_uniform + static_cast<uint32_t>(t.waves) - 1) / static_cast<uint32_t>(t.waves);
+    plan->info.payload_bytes = n_recs * len;
+    plan->info.vec_descs = n_descs;
+    plan->info.plan_device_bytes = bytes;
+    plan->info.vec_chunks = plan->n_uniform;
+    plan->info.uniform_chunks = plan->n_uniform;
+    plan->info.units_per_lane = static_cast<uint32_t>(t.upl);
+    plan->info.uniform_workgroups = plan->uniform_wgs;
+    *out = plan;
+    return NIXL_AMD_OK;
+}
+
+// A pinned upload buffer that its caller fills with block records (nixl_amd_copy_records_begin).
+struct nixl_amd_copy_records {
+    void *staging = nullptr;
+    size_t staging_cap = 0;
+    size_t max_records = 0;
+};
+
 extern "C" {
 
 int
@@ -684,24 +827,11 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     if (!descs && n) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: descs is null");
     if (n >= (1ull << 32)) return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "plan_create: more than 2^32-1 descriptors");
 
-    // Defaults from a sweep on MI355X: the smallest chunk (one 128-bit load and store per
-    // lane, one wave per workgroup) gave the highest HBM rate; the cache policy follows the
-    // destination pattern (below).
-    int upl = 1, nt = 0, waves = 1, swizzle = 0, sort_scatter = 0;
-    uint32_t max_wgs = 0;
-    if (tuning) {
-        if (tuning->units_per_lane) upl = tuning->units_per_lane;
-        if (tuning->nontemporal) nt = tuning->nontemporal;
-        if (tuning->max_workgroups > 0) max_wgs = static_cast<uint32_t>(tuning->max_workgroups);
-        if (tuning->waves_per_workgroup) waves = tuning->waves_per_workgroup;
-        if (tuning->xcd_swizzle) swizzle = tuning->xcd_swizzle == 1 ? 1 : 0;
-        sort_scatter = tuning->sort_scatter;
-    }
-    if (upl != 1 && upl != 2 && upl != 4 && upl != 8 && upl != 16)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: units_per_lane must be 1, 2, 4, 8 or 16");
-    if (nt < 0 || nt > 4) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: nontemporal must be 0 to 4");
-    if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16)
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create: waves_per_workgroup must be 1, 2, 4, 8 or 16");
+    Tuning t;
+    if (const int rc = parse_tuning(tuning, t, "plan_create")) return rc;
+    const int upl = t.upl, waves = t.waves, swizzle = t.swizzle;
+    int nt = t.nt;
+    const uint32_t max_wgs = t.max_wgs;
 
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
@@ -715,8 +845,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     // ---- fast path: equal-length, line-aligned descriptors of whole chunks (KV blocks) ----
     // One pass over the descriptors writes the {src, dst} records straight into the pinned
     // upload buffer; nothing else is built.
-    if (n > 0 && descs[0].len >= 8192 && descs[0].len % (chunk_units * 16u) == 0 &&
-        2 * n * (descs[0].len / (chunk_units * 16u)) < (1ull << 32)) {
+    if (n > 0 && block_len_fits(descs[0].len, t)) {
         // Descriptors whose length is a multiple of the first one's (neighbouring blocks that
         // the caller merged) become that many records; room for twice as many records as
         // descriptors, beyond that the general lowering takes over.
@@ -725,79 +854,36 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         void *staging = nullptr;
         size_t staging_cap = 0;
         reap_uploads(device);
-        hipError_t e = upload_cache().get(device, cap * sizeof(UniformRec), &staging, &staging_cap);
+        const hipError_t e = upload_cache().get(device, cap * sizeof(UniformRec), &staging, &staging_cap);
         if (e != hipSuccess)
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
         auto *recs = static_cast<UniformRec *>(staging);
-        uint64_t misfit = 0, regular = 0, prev_dst = 0, prev_step = 0, payload = 0, src_follows = 0, prev_src_end = 0;
+        bool misfit = false;
         size_t n_recs = 0;
-        for (size_t i = 0; i < n && !misfit; ++i) {
+        for (size_t i = 0; i < n; ++i) {
             const nixl_amd_copy_desc_t &d = descs[i];
+            if (d.len == len0) {
+                recs[n_recs++] = UniformRec{d.src, d.dst};
+                continue;
+            }
             const uint64_t k = d.len / len0;
-            misfit |= (d.len - k * len0) | ((d.src | d.dst) & 127u) | (d.src == 0) | (d.dst == 0) | (k == 0) |
-                (d.src + d.len < d.src) | (d.dst + d.len < d.dst) | (n_recs + k > cap);
-            const uint64_t step = d.dst - prev_dst;
-            regular += (i > 0) & ((step == len0) | ((i > 1) & (step == prev_step)));
-            prev_step = step;
-            prev_dst = d.dst + d.len - len0; // start of the descriptor's last block
-            src_follows += (d.src == prev_src_end);
-            prev_src_end = d.src + d.len;
-            payload += d.len;
-            if (misfit) break;
+            if (k == 0 || d.len != k * len0 || k > cap - n_recs || d.src + d.len < d.src || d.dst + d.len < d.dst) {
+                misfit = true;
+                break;
+            }
             for (uint64_t j = 0; j < k; ++j)
                 recs[n_recs++] = UniformRec{d.src + j * len0, d.dst + j * len0};
-        }
-        const size_t bytes = n_recs * sizeof(UniformRec);
-        if (!misfit) {
-            auto *plan = new nixl_amd_copy_plan();
-            plan->device = device;
-            plan->upl = upl;
-            plan->waves = waves;
-            plan->swizzle = swizzle;
-            plan->max_wgs = max_wgs;
-            // cache policy by destination pattern, as in the general lowering below
-            const bool scattered = !(n == 1 || 2 * regular >= n - 1);
-            // a scatter out of consecutive memory is put into ascending destination order, window by window
-            const bool sort = scattered && sort_scatter != 2 && 2 * src_follows >= n - 1 && n_recs >= kSortWindow;
-            plan->policy = nt ? nt : ((!scattered || sort) ? kPolNtSc1Nt : kPolPlainSc1Nt);
-            hipStream_t up = nullptr;
-            e = arena_cache().get(device, bytes, &plan->arena, &plan->arena_cap);
-            if (e == hipSuccess) e = upload_stream(device, &up);
-            if (e == hipSuccess) e = hipMemcpyAsync(plan->arena, staging, bytes, hipMemcpyHostToDevice, up);
-            if (e == hipSuccess && sort) {
-                hipLaunchKernelGGL(sort_records_kernel, dim3(static_cast<uint32_t>((n_recs + kSortWindow - 1) / kSortWindow)),
-                                   dim3(kSortWindow / 2), 0, up, static_cast<UniformRec *>(plan->arena),
-                                   static_cast<uint32_t>(n_recs));
-                e = hipGetLastError();
+            if (n_recs + (n - 1 - i) > cap) { // the rest must still fit one record each
+                misfit = true;
+                break;
             }
-            // No wait here: the event goes behind the copy, launches wait for it on their stream.
-            if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
-            if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
-            if (e != hipSuccess) {
-                if (up) (void)hipStreamSynchronize(up); // whatever was queued reads the buffers given back below
-                if (plan->uploaded) (void)hipEventDestroy(plan->uploaded);
-                upload_cache().put(device, staging, staging_cap);
-                if (plan->arena) arena_cache().put(device, plan->arena, plan->arena_cap);
-                delete plan;
-                return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan upload: ") + hipGetErrorString(e));
-            }
-            recycle_after(device, up, staging, staging_cap);
-            plan->arena_bytes = bytes;
-            plan->uniform_recs = static_cast<const UniformRec *>(plan->arena);
-            plan->chunks_per_rec = static_cast<uint32_t>(len0 / (chunk_units * 16u));
-            plan->n_uniform = static_cast<uint32_t>(n_recs * plan->chunks_per_rec);
-            plan->uniform_wgs = (plan->n_uniform + static_cast<uint32_t>(waves) - 1) / static_cast<uint32_t>(waves);
-            plan->info.payload_bytes = payload;
-            plan->info.vec_descs = n;
-            plan->info.plan_device_bytes = bytes;
-            plan->info.vec_chunks = plan->n_uniform;
-            plan->info.uniform_chunks = plan->n_uniform;
-            plan->info.units_per_lane = static_cast<uint32_t>(upl);
-            plan->info.uniform_workgroups = plan->uniform_wgs;
-            *out = plan;
-            return NIXL_AMD_OK;
         }
-        upload_cache().put(device, staging, staging_cap); // something else: the general lowering decides
+        if (misfit) {
+            upload_cache().put(device, staging, staging_cap); // something else: the general lowering decides
+        } else {
+            const int rc = build_block_plan(device, t, staging, staging_cap, n_recs, len0, n, nullptr, out);
+            if (rc != kNotBlocks) return rc;
+        }
     }
 
     // ---- host-side lowering ------------------------------------------------------
@@ -973,6 +1059,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     if (total > 0) {
         void *staging = nullptr;
         size_t staging_cap = 0;
+        reap_uploads(device);
         hipError_t e = upload_cache().get(device, total, &staging, &staging_cap);
         if (e != hipSuccess) {
             delete plan;
@@ -995,17 +1082,22 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
             delete plan;
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipMalloc(plan arena): ") + hipGetErrorString(e));
         }
-        // The copy is waited for: the pinned buffer goes back to the cache right after it.
+        // No wait here either: the event goes behind the copy, launches wait for it on their
+        // stream, and the pinned buffer is recycled once the copy has completed.
         hipStream_t up = nullptr;
         e = upload_stream(device, &up);
         if (e == hipSuccess) e = hipMemcpyAsync(plan->arena, host, total, hipMemcpyHostToDevice, up);
-        if (e == hipSuccess) e = hipStreamSynchronize(up);
-        upload_cache().put(device, staging, staging_cap);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
         if (e != hipSuccess) {
+            if (up) (void)hipStreamSynchronize(up); // a queued copy still reads the buffer given back below
+            if (plan->uploaded) (void)hipEventDestroy(plan->uploaded);
+            upload_cache().put(device, staging, staging_cap);
             arena_cache().put(device, plan->arena, plan->arena_cap);
             delete plan;
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipMemcpy(plan arena): ") + hipGetErrorString(e));
         }
+        recycle_after(device, up, staging, staging_cap);
         plan->arena_bytes = total;
         auto *base = static_cast<uint8_t *>(plan->arena);
         plan->uniform_recs = reinterpret_cast<const UniformRec *>(base + off_uni);
@@ -1050,6 +1142,79 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
 }
 
 int
+nixl_amd_copy_block_len_fits(uint64_t len, const nixl_amd_copy_tuning_t *tuning) {
+    Tuning t;
+    if (parse_tuning(tuning, t, "block_len_fits")) return 0;
+    return block_len_fits(len, t) ? 1 : 0;
+}
+
+int
+nixl_amd_copy_records_begin(size_t max_records, nixl_amd_copy_records_t **out, nixl_amd_copy_record_t **records) {
+    static_assert(sizeof(nixl_amd_copy_record_t) == sizeof(UniformRec));
+    if (!out || !records) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "records_begin: null argument");
+    *out = nullptr;
+    *records = nullptr;
+    if (max_records == 0 || max_records >= (1ull << 31))
+        return nixl_amd_fail(NIXL_AMD_ERR_TOO_LARGE, "records_begin: between 1 and 2^31-1 records");
+    auto *r = new nixl_amd_copy_records();
+    r->max_records = max_records;
+    const hipError_t e = upload_cache().get(0, max_records * sizeof(UniformRec), &r->staging, &r->staging_cap);
+    if (e != hipSuccess) {
+        delete r;
+        return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
+    }
+    *records = static_cast<nixl_amd_copy_record_t *>(r->staging);
+    *out = r;
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_copy_records_abandon(nixl_amd_copy_records_t *records) {
+    if (!records) return NIXL_AMD_OK;
+    upload_cache().put(0, records->staging, records->staging_cap);
+    delete records;
+    return NIXL_AMD_OK;
+}
+
+int
+nixl_amd_copy_plan_create_from_records(nixl_amd_copy_records_t *records,
+                                       size_t n,
+                                       uint64_t len,
+                                       int device,
+                                       const nixl_amd_copy_tuning_t *tuning,
+                                       const nixl_amd_copy_record_facts_t *facts,
+                                       nixl_amd_copy_plan_t **out) {
+    if (!records) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_from_records: records is null");
+    // the buffer is taken over whatever happens below
+    void *staging = records->staging;
+    const size_t staging_cap = records->staging_cap, max_records = records->max_records;
+    delete records;
+    const auto give_back = [&](int code, const char *why) {
+        upload_cache().put(0, staging, staging_cap);
+        return nixl_amd_fail(code, why);
+    };
+    if (!out) return give_back(NIXL_AMD_ERR_INVALID, "plan_create_from_records: out is null");
+    *out = nullptr;
+    if (n == 0 || n > max_records) return give_back(NIXL_AMD_ERR_INVALID, "plan_create_from_records: record count outside the buffer");
+    Tuning t;
+    if (const int rc = parse_tuning(tuning, t, "plan_create_from_records")) {
+        upload_cache().put(0, staging, staging_cap);
+        return rc;
+    }
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0) return give_back(NIXL_AMD_ERR_NO_DEVICE, "plan_create_from_records: no HIP device");
+    if (device < 0 || device >= ndev) return give_back(NIXL_AMD_ERR_INVALID, "plan_create_from_records: bad device index");
+    const DeviceScope on_device(device);
+    if (on_device.status() != hipSuccess) return give_back(NIXL_AMD_ERR_HIP, "plan_create_from_records: hipSetDevice failed");
+    reap_uploads(device);
+    const int rc = build_block_plan(device, t, staging, staging_cap, n, len, n, facts, out);
+    if (rc == kNotBlocks)
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID,
+                             "plan_create_from_records: blocks must be whole chunks of at least 8 KiB, start on 128-byte lines and not wrap");
+    return rc;
+}
+
+int
 nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
                                        size_t n_src_runs,
                                        const int32_t *src_index,
@@ -1064,17 +1229,9 @@ nixl_amd_copy_plan_create_indexed_runs(const nixl_amd_copy_run_t *src_runs,
     if (!out) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: out is null");
     *out = nullptr;
     if (!src_index || !dst_index || n == 0) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: no indices");
-    int upl = 1, nt = 0, waves = 1, swizzle = 0, sort_scatter = 0;
-    if (tuning) {
-        if (tuning->units_per_lane) upl = tuning->units_per_lane;
-        if (tuning->nontemporal) nt = tuning->nontemporal;
-        if (tuning->waves_per_workgroup) waves = tuning->waves_per_workgroup;
-        if (tuning->xcd_swizzle) swizzle = tuning->xcd_swizzle == 1 ? 1 : 0;
-        sort_scatter = tuning->sort_scatter;
-    }
-    if ((upl != 1 && upl != 2 && upl != 4 && upl != 8 && upl != 16) || nt < 0 || nt > 4 ||
-        (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16))
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: bad tuning value");
+    Tuning t;
+    if (const int rc = parse_tuning(tuning, t, "plan_create_indexed")) return rc;
+    const int upl = t.upl, nt = t.nt, waves = t.waves, swizzle = t.swizzle, sort_scatter = t.sort_scatter;
     const uint64_t chunk_bytes = static_cast<uint64_t>(kWaveSize) * upl * 16u;
     if (!src_runs || !dst_runs || n_src_runs == 0 || n_dst_runs == 0 || n_src_runs > kMaxIndexRuns || n_dst_runs > kMaxIndexRuns)
         return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_create_indexed: between 1 and 256 runs a side");
@@ -1278,6 +1435,15 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
                            plan->generic_items, plan->n_generic);
         HIP_TRY(hipGetLastError());
     }
+    // What nixl_amd_copy_plan_destroy looks at.  A stream under graph capture gets no event: the
+    // graph's owner keeps the plan alive for as long as the graph may be replayed.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &capture) != hipSuccess) (void)hipGetLastError();
+    if (capture == hipStreamCaptureStatusNone) {
+        if (!plan->launched) HIP_TRY(hipEventCreateWithFlags(&plan->launched, hipEventDisableTiming));
+        HIP_TRY(hipEventRecord(plan->launched, s));
+        plan->launched_valid = true;
+    }
     return NIXL_AMD_OK;
 }
 
@@ -1285,7 +1451,17 @@ int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan) {
     if (!plan) return NIXL_AMD_OK;
     const DeviceScope on_device(plan->device);
+    if (plan->launched_valid) {
+        // The arena goes back to a pool that the next plan's upload writes into: not while a
+        // launch of this plan may still read it.  The plan stays as it is; destroy it later.
+        const hipError_t state = hipEventQuery(plan->launched);
+        if (state == hipErrorNotReady) {
+            (void)hipGetLastError();
+            return nixl_amd_fail(NIXL_AMD_ERR_BUSY, "plan_destroy: a launch of this plan has not completed");
+        }
+    }
     (void)settle_upload(plan, true); // the arena and the upload buffer go back only when nothing writes or reads them
+    if (plan->launched) (void)hipEventDestroy(plan->launched);
     if (plan->ev0) (void)hipEventDestroy(plan->ev0);
     if (plan->ev1) (void)hipEventDestroy(plan->ev1);
     if (plan->arena) arena_cache().put(plan->device, plan->arena, plan->arena_cap);

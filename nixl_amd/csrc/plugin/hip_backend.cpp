@@ -125,6 +125,9 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     tuning_.max_workgroups = paramInt(p, "max_workgroups", 0);
     tuning_.waves_per_workgroup = paramInt(p, "waves_per_workgroup", 0);
     tuning_.xcd_swizzle = paramInt(p, "xcd_swizzle", 0);
+    indexedPrep_ = paramInt(p, "indexed_prep", 1) != 0;
+    prepThreads_ = paramInt(p, "prep_threads", 1);
+    if (prepThreads_ < 1 || prepThreads_ > 16) throw std::runtime_error("HIP backend: prep_threads must be in [1, 16]");
     streamsPerDevice_ = paramInt(p, "num_streams", 1);
     if (streamsPerDevice_ < 1 || streamsPerDevice_ > 16)
         throw std::runtime_error("HIP backend: num_streams must be in [1, 16]");
@@ -222,6 +225,18 @@ nixlHipEngine::pickStream(int device) const {
             streams_[idx] = nullptr;
     }
     return streams_[idx];
+}
+
+nixl_amd_hip::WorkerPool *
+nixlHipEngine::prepPool() const {
+    std::call_once(prepPoolOnce_, [this] {
+        try {
+            prepPool_ = std::make_unique<WorkerPool>(static_cast<unsigned>(prepThreads_ - 1));
+        } catch (const std::exception &e) {
+            NIXL_WARN << "HIP backend: no helper threads for prepXfer (" << e.what() << ")";
+        }
+    });
+    return prepPool_.get();
 }
 
 void
@@ -323,33 +338,16 @@ nixlHipEngine::deregisterMem(nixlBackendMD *meta) {
     return NIXL_SUCCESS;
 }
 
+// The general lowering's pass: every descriptor pair checked against its registrations and
+// written out as {src, dst, len} with the direction applied.
 nixl_status_t
-nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
-                        const nixl_meta_dlist_t &local,
-                        const nixl_meta_dlist_t &remote,
-                        const std::string &remote_agent,
-                        nixlBackendReqH *&handle,
-                        const nixl_opt_b_args_t *opt_args) const {
-    handle = nullptr;
-    reapRetired(false);
-
-    if (!knowsAgent(remote_agent)) {
-        NIXL_ERROR << "HIP backend: agent '" << remote_agent << "' is neither this agent ('" << localAgent
-                   << "') nor a peer whose connection info was loaded";
-        return NIXL_ERR_NOT_FOUND;
-    }
-    if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
+nixlHipEngine::lowerGeneral(bool write,
+                            const nixl_meta_dlist_t &local,
+                            const nixl_meta_dlist_t &remote,
+                            nixl_amd_copy_desc_t *lowered,
+                            int &device,
+                            size_t &bytes) const {
     const int n = local.descCount();
-    if (n == 0 || n != remote.descCount()) {
-        NIXL_ERROR << "HIP backend: descriptor count mismatch (local " << n << ", remote "
-                   << remote.descCount() << ")";
-        return NIXL_ERR_INVALID_PARAM;
-    }
-
-    const auto t_start = std::chrono::steady_clock::now();
-    const std::unique_ptr<nixl_amd_copy_desc_t[]> lowered(new nixl_amd_copy_desc_t[static_cast<size_t>(n)]); // not zero-filled
-    int device = -1;
-    size_t bytes = 0;
     const nixlHipMD *prev_lmd = nullptr, *prev_rmd = nullptr;
     for (int i = 0; i < n; ++i) {
         const nixlMetaDesc &l = local[i];
@@ -378,7 +376,6 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
                 return NIXL_ERR_NOT_SUPPORTED;
             }
         }
-        const bool write = (operation == NIXL_WRITE);
         const uintptr_t la = lmd->here(l.addr), ra = rmd->here(r.addr); // a peer's region may be mapped elsewhere here
         lowered[i].src = write ? la : ra;
         lowered[i].dst = write ? ra : la;
@@ -386,16 +383,262 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
         bytes += l.len;
     }
     if (device < 0) device = static_cast<const nixlHipMD *>(local[0].metadataP)->device;
+    return NIXL_SUCCESS;
+}
 
-    const auto t_lowered = std::chrono::steady_clock::now();
+// The block pass of prepXfer over descriptor pairs [begin, end): pair i becomes record i.
+// While the two registrations do not change from one pair to the next (a pool and a staging
+// buffer: never) their bounds stay in registers and the checks are accumulated without
+// branches and looked at once per stretch.  A pair of several blocks (neighbours the agent
+// merged) writes its first block and is noted in `merged`; a pair that is no whole number of
+// blocks ends the pass (`blocks` false).  The pass also gathers what the plan wants to know
+// of the records (nixl_amd_copy_record_facts_t), so that nothing reads them a second time.
+struct nixlHipEngine::blockSlice {
+    nixl_status_t status = NIXL_SUCCESS;
+    bool blocks = true;
+    int device = -1; // of the VRAM regions seen
+    size_t bytes = 0;
+    nixl_amd_copy_record_facts_t facts{};
+    std::vector<std::pair<size_t, size_t>> merged; // {pair, blocks}
+};
+
+void
+nixlHipEngine::lowerBlockSlice(bool write,
+                               const nixlMetaDesc *L,
+                               const nixlMetaDesc *R,
+                               size_t begin,
+                               size_t end,
+                               size_t len0,
+                               nixl_amd_copy_record_t *records,
+                               blockSlice &out) const {
+    uint64_t address_bits = 0;
+    size_t total = 0;
+    for (size_t i = begin; i < end;) {
+        const auto *lmd = static_cast<const nixlHipMD *>(L[i].metadataP);
+        const auto *rmd = static_cast<const nixlHipMD *>(R[i].metadataP);
+        if (!lmd || !rmd) {
+            NIXL_ERROR << "HIP backend: descriptor " << i << " carries no registration";
+            out.status = NIXL_ERR_INVALID_PARAM;
+            return;
+        }
+        // The kernel runs on the device that owns the VRAM side(s); two VRAM regions on
+        // different devices would need peer mappings, which this backend does not set up.
+        for (const nixlHipMD *md : {lmd, rmd}) {
+            if (md->mem != VRAM_SEG) continue;
+            if (out.device < 0) out.device = md->device;
+            if (md->device != out.device) {
+                NIXL_ERROR << "HIP backend: descriptors span devices " << out.device << " and " << md->device;
+                out.status = NIXL_ERR_NOT_SUPPORTED;
+                return;
+            }
+        }
+        const nixlBackendMD *const lkey = L[i].metadataP, *const rkey = R[i].metadataP;
+        const uintptr_t lbase = lmd->addr, rbase = rmd->addr;
+        const size_t lspan = lmd->len, rspan = rmd->len;
+        // a peer's region may be mapped elsewhere here; the direction decides which side is read
+        const uintptr_t to_src = static_cast<uintptr_t>(write ? lmd->delta : rmd->delta);
+        const uintptr_t to_dst = static_cast<uintptr_t>(write ? rmd->delta : lmd->delta);
+        const size_t stretch_begin = i;
+        size_t bad = 0;
+        for (; i < end; ++i) {
+            const nixlMetaDesc &l = L[i], &r = R[i];
+            if (l.metadataP != lkey || r.metadataP != rkey) break; // other registrations: hoist again
+            const size_t len = l.len;
+            // inside its region on both sides (an address below the region wraps to a huge offset)
+            bad |= static_cast<size_t>(len != r.len) | static_cast<size_t>(len > lspan) | static_cast<size_t>(len > rspan) |
+                static_cast<size_t>(l.addr - lbase > lspan - len) | static_cast<size_t>(r.addr - rbase > rspan - len);
+            const uintptr_t src = (write ? l.addr : r.addr) + to_src, dst = (write ? r.addr : l.addr) + to_dst;
+            records[i] = nixl_amd_copy_record_t{src, dst};
+            address_bits |= src | dst;
+            total += len;
+            if (len != len0) [[unlikely]] {
+                const size_t k = len / len0;
+                if (k == 0 || k * len0 != len) {
+                    out.blocks = false;
+                    return;
+                }
+                out.merged.emplace_back(i, k);
+            }
+        }
+        if (bad) {
+            // which one: walk the stretch again, this time with the words
+            out.status = NIXL_ERR_INVALID_PARAM;
+            for (size_t j = stretch_begin; j < i; ++j) {
+                if (L[j].len != R[j].len) {
+                    NIXL_ERROR << "HIP backend: length mismatch at descriptor " << j;
+                    return;
+                }
+                if (!lmd->contains(L[j].addr, L[j].len) || !rmd->contains(R[j].addr, R[j].len)) {
+                    NIXL_ERROR << "HIP backend: descriptor " << j << " is outside its registered region";
+                    return;
+                }
+            }
+            return;
+        }
+    }
+    out.bytes = total;
+    out.facts.address_bits = address_bits;
+    // How the destinations and the sources advance decides the plan's cache policy and record
+    // order by majority, so a sample answers it: the first 64 steps of every 1024 records
+    // (carrying three values from pair to pair through the loop above cost it half its time
+    // again).  A pair of several blocks shows up as one irregular step.
+    constexpr size_t kWindow = 1024, kLook = 64;
+    uint64_t regular = 0, follows = 0, steps = 0;
+    for (size_t w = begin; w + 2 < end; w += kWindow) {
+        const size_t last = std::min(end, w + kLook + 2);
+        for (size_t i = w + 2; i < last; ++i) {
+            const uintptr_t step = records[i].dst - records[i - 1].dst, before = records[i - 1].dst - records[i - 2].dst;
+            regular += static_cast<uint64_t>(step == len0) | static_cast<uint64_t>(step == before);
+            follows += static_cast<uint64_t>(records[i].src - records[i - 1].src == len0);
+        }
+        steps += last - (w + 2);
+    }
+    out.facts.regular_dst_steps = regular;
+    out.facts.following_src_steps = follows;
+    out.facts.steps = steps;
+}
+
+// Runs the block pass over the whole request: alone for short lists, with the helper threads
+// for long ones (sixteen slices that the threads take as they come).  The records of pairs of
+// several blocks beyond their first go behind the others: the order of records decides
+// nothing about the bytes that arrive.
+nixlHipEngine::blockPass
+nixlHipEngine::lowerBlocks(bool write,
+                           const nixl_meta_dlist_t &local,
+                           const nixl_meta_dlist_t &remote,
+                           nixl_amd_copy_record_t *records,
+                           size_t room,
+                           size_t &n_records,
+                           int &device,
+                           size_t &bytes,
+                           nixl_amd_copy_record_facts_t &facts) const {
+    const size_t n = static_cast<size_t>(local.descCount());
+    const nixlMetaDesc *const L = &local[0], *const R = &remote[0];
+    const size_t len0 = L[0].len;
+    constexpr size_t kParallelFrom = 16384; // pairs; below that the pass is shorter than waking a helper
+    constexpr unsigned kSlices = 16;
+    std::vector<blockSlice> slices(1);
+    bool shared = false;
+    if (n >= kParallelFrom && prepThreads_ > 1) {
+        WorkerPool *pool = prepPool();
+        if (pool) {
+            slices.assign(kSlices, blockSlice{});
+            shared = pool->run(kSlices, [&](unsigned s) {
+                lowerBlockSlice(write, L, R, n * s / kSlices, n * (s + 1) / kSlices, len0, records, slices[s]);
+            });
+            if (!shared) slices.assign(1, blockSlice{}); // the pool serves another thread's request
+        }
+    }
+    if (!shared) lowerBlockSlice(write, L, R, 0, n, len0, records, slices[0]);
+
+    device = -1;
+    bytes = 0;
+    facts = nixl_amd_copy_record_facts_t{};
+    size_t made = n;
+    for (const blockSlice &s : slices) {
+        if (s.status != NIXL_SUCCESS) return {s.status, false};
+        if (!s.blocks) return {NIXL_SUCCESS, false};
+        if (s.device >= 0) {
+            if (device < 0) device = s.device;
+            if (s.device != device) {
+                NIXL_ERROR << "HIP backend: descriptors span devices " << device << " and " << s.device;
+                return {NIXL_ERR_NOT_SUPPORTED, false};
+            }
+        }
+        bytes += s.bytes;
+        facts.address_bits |= s.facts.address_bits;
+        facts.regular_dst_steps += s.facts.regular_dst_steps;
+        facts.following_src_steps += s.facts.following_src_steps;
+        facts.steps += s.facts.steps;
+        for (const auto &[pair, blocks] : s.merged) {
+            if (blocks - 1 > room - made) return {NIXL_SUCCESS, false};
+            for (size_t j = 1; j < blocks; ++j)
+                records[made++] = nixl_amd_copy_record_t{records[pair].src + j * len0, records[pair].dst + j * len0};
+        }
+    }
+    if (device < 0) device = static_cast<const nixlHipMD *>(L[0].metadataP)->device;
+    n_records = made;
+    return {NIXL_SUCCESS, true};
+}
+
+nixl_status_t
+nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
+                        const nixl_meta_dlist_t &local,
+                        const nixl_meta_dlist_t &remote,
+                        const std::string &remote_agent,
+                        nixlBackendReqH *&handle,
+                        const nixl_opt_b_args_t *opt_args) const {
+    handle = nullptr;
+    reapRetired(false);
+
+    if (!knowsAgent(remote_agent)) {
+        NIXL_ERROR << "HIP backend: agent '" << remote_agent << "' is neither this agent ('" << localAgent
+                   << "') nor a peer whose connection info was loaded";
+        return NIXL_ERR_NOT_FOUND;
+    }
+    if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
+    const int n = local.descCount();
+    if (n == 0 || n != remote.descCount()) {
+        NIXL_ERROR << "HIP backend: descriptor count mismatch (local " << n << ", remote "
+                   << remote.descCount() << ")";
+        return NIXL_ERR_INVALID_PARAM;
+    }
+
+    const auto t_start = std::chrono::steady_clock::now();
     auto req = std::make_unique<nixlHipReqH>();
+    int device = -1;
+    size_t bytes = 0;
+    const bool write = (operation == NIXL_WRITE);
+    const char *path = "general";
+    auto t_pass = t_start;
+
+    // Equal blocks (paged KV): ONE pass checks every descriptor pair against its registrations
+    // and writes its {src, dst} record straight into the pinned buffer the plan is uploaded
+    // from.  Anything else in the lists (mixed lengths, blocks too short or not on 128-byte
+    // lines) sends the request to the general lowering below.
+    if (nixl_amd_copy_block_len_fits(local[0].len, &tuning_)) {
+        nixl_amd_copy_records_t *buffer = nullptr;
+        nixl_amd_copy_record_t *records = nullptr;
+        const size_t room = 2 * static_cast<size_t>(n); // merged neighbours become one record per block
+        if (nixl_amd_copy_records_begin(room, &buffer, &records) != NIXL_AMD_OK) {
+            NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+            return NIXL_ERR_BACKEND;
+        }
+        size_t n_records = 0;
+        nixl_amd_copy_record_facts_t facts{};
+        const blockPass pass = lowerBlocks(write, local, remote, records, room, n_records, device, bytes, facts);
+        t_pass = std::chrono::steady_clock::now();
+        if (pass.status != NIXL_SUCCESS) {
+            (void)nixl_amd_copy_records_abandon(buffer);
+            return pass.status;
+        }
+        if (!pass.blocks) {
+            (void)nixl_amd_copy_records_abandon(buffer);
+        } else {
+            const int rc = nixl_amd_copy_plan_create_from_records(buffer, n_records, local[0].len, device, &tuning_, &facts, &req->plan);
+            if (rc == NIXL_AMD_OK)
+                path = "blocks";
+            else if (rc != NIXL_AMD_ERR_INVALID) { // INVALID: not on 128-byte lines, say; the general lowering judges
+                NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+                return NIXL_ERR_BACKEND;
+            }
+        }
+    }
+    const auto t_lowered = std::chrono::steady_clock::now();
+
+    if (!req->plan) {
+        const std::unique_ptr<nixl_amd_copy_desc_t[]> lowered(new nixl_amd_copy_desc_t[static_cast<size_t>(n)]); // not zero-filled
+        device = -1;
+        bytes = 0;
+        const nixl_status_t st = lowerGeneral(write, local, remote, lowered.get(), device, bytes);
+        if (st != NIXL_SUCCESS) return st;
+        if (nixl_amd_copy_plan_create(lowered.get(), static_cast<size_t>(n), device, &tuning_, &req->plan) != NIXL_AMD_OK) {
+            NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
+            return NIXL_ERR_BACKEND;
+        }
+    }
     req->device = device;
     req->bytes = bytes;
-    if (nixl_amd_copy_plan_create(lowered.get(), static_cast<size_t>(n), device, &tuning_, &req->plan) !=
-        NIXL_AMD_OK) {
-        NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
-        return NIXL_ERR_BACKEND;
-    }
     const DeviceScope on_device(device);
     if (!on_device.ok() || !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
         return NIXL_ERR_BACKEND;
@@ -403,9 +646,10 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
     if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
 
     const auto t_done = std::chrono::steady_clock::now();
-    NIXL_DEBUG << "HIP backend: prepXfer of " << n << " descriptors: checks and lowering "
-               << std::chrono::duration<double, std::micro>(t_lowered - t_start).count() << " us, device plan and event "
-               << std::chrono::duration<double, std::micro>(t_done - t_lowered).count() << " us";
+    const auto us = [](auto from, auto to) { return std::chrono::duration<double, std::micro>(to - from).count(); };
+    NIXL_DEBUG << "HIP backend: prepXfer of " << n << " descriptors (" << path << "): block pass " << us(t_start, t_pass)
+               << " us, plan from records " << us(t_pass, t_lowered) << " us, rest (general lowering, event, stream) "
+               << us(t_lowered, t_done) << " us";
     handle = req.release();
     return NIXL_SUCCESS;
 }
@@ -422,6 +666,7 @@ nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
                                const std::string &remote_agent,
                                nixlBackendReqH *&handle) const {
     handle = nullptr;
+    if (!indexedPrep_) return NIXL_ERR_NOT_SUPPORTED; // switched off: every request comes through prepXfer
     reapRetired(false);
     if (!knowsAgent(remote_agent)) return NIXL_ERR_NOT_FOUND;
     if (operation != NIXL_READ && operation != NIXL_WRITE) return NIXL_ERR_INVALID_PARAM;
@@ -1054,6 +1299,8 @@ nixl_plugin_init() {
                                  {"waves_per_workgroup", "0"},
                                  {"xcd_swizzle", "0"},
                                  {"num_streams", "1"},
+                                 {"indexed_prep", "1"},
+                                 {"prep_threads", "1"},
                                  {"stream", ""}},
                                 {VRAM_SEG, DRAM_SEG});
 }

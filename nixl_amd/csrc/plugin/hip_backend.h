@@ -15,6 +15,7 @@
 
 #include <atomic>
 #include <condition_variable>
+#include <memory>
 #include <mutex>
 #include <thread>
 #include <string>
@@ -24,6 +25,7 @@
 #include "backend/backend_engine.h"
 #include "nixl_amd_hip.h"
 #include "mailbox.h"
+#include "worker_pool.h"
 
 // Registration record returned by registerMem and handed back in nixlMetaDesc::metadataP.
 // `addr` is the region's address in its OWNER's address space, which is the space the
@@ -219,6 +221,41 @@ public:
                      const nixl_opt_args_t *extra_params = nullptr) const override;
 
 private:
+    // The two passes of prepXfer over a request's descriptor lists (hip_backend.cpp).
+    struct blockPass {
+        nixl_status_t status;
+        bool blocks; // every pair a whole number of equal blocks and the records fit
+    };
+    struct blockSlice;
+    blockPass
+    lowerBlocks(bool write,
+                const nixl_meta_dlist_t &local,
+                const nixl_meta_dlist_t &remote,
+                nixl_amd_copy_record_t *records,
+                size_t room,
+                size_t &n_records,
+                int &device,
+                size_t &bytes,
+                nixl_amd_copy_record_facts_t &facts) const;
+    void
+    lowerBlockSlice(bool write,
+                    const nixlMetaDesc *L,
+                    const nixlMetaDesc *R,
+                    size_t begin,
+                    size_t end,
+                    size_t len0,
+                    nixl_amd_copy_record_t *records,
+                    blockSlice &out) const;
+    using WorkerPool = nixl_amd_hip::WorkerPool;
+    WorkerPool *
+    prepPool() const; // made on first use
+    nixl_status_t
+    lowerGeneral(bool write,
+                 const nixl_meta_dlist_t &local,
+                 const nixl_meta_dlist_t &remote,
+                 nixl_amd_copy_desc_t *lowered,
+                 int &device,
+                 size_t &bytes) const;
     hipStream_t
     pickStream(int device) const;
     void
@@ -239,6 +276,12 @@ private:
 
     int numDevices_ = 0;
     int streamsPerDevice_ = 1;
+    // prep_threads: threads that share the pass over a long request's descriptor lists (the
+    // caller included; 1 = the caller alone).
+    int prepThreads_ = 1;
+    mutable std::once_flag prepPoolOnce_;
+    mutable std::unique_ptr<WorkerPool> prepPool_;
+    bool indexedPrep_ = true; // backend parameter indexed_prep: 0 makes prepXferIndexed decline every request
     bool useExternalStream_ = false; // launches go to the application's stream (may be the null stream)
     hipStream_t externalStream_ = nullptr;
     nixl_amd_copy_tuning_t tuning_{};

@@ -335,6 +335,20 @@ def test_notification_ring_of_the_hip_backend_on_the_cpu():
     assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
 
 
+def test_helper_threads_of_the_hip_backend_on_the_cpu():
+    """tests/cpp/worker_pool_check.cpp: the helper threads that share prepXfer's pass over a long
+    request (nixl_amd/csrc/plugin/worker_pool.h): every slice of every job runs exactly once,
+    a second caller is turned away while the pool is busy, competing callers lose nothing, and
+    the pool shuts down with its helpers polling or asleep."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "_build", "worker_pool_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} missing: run __graft_entry__.build() first")
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0 and proc.stdout.strip().endswith("OK"), proc.stdout + proc.stderr
+
+
 def test_list_and_option_helpers_of_the_c_wrapper(two_agents):
     """The descriptor-list, option and stub helpers of the reference's C wrapper
     (src/bindings/rust/wrapper.h:193-201,297-326,457) behave as their names say; the metadata

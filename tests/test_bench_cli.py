@@ -32,3 +32,22 @@ def test_counter_file_of_the_profiler_is_read_per_kernel(tmp_path):
     kernel, yard, n = bench.counter_samples(str(path), ["A", "B"])
     assert kernel == {"A": 20.0, "B": 7.0} and yard == {"A": 6.0, "B": 2.0} and n == 3
     assert bench.counter_samples(str(path), ["A", "D"]) is None
+
+
+def test_phase_timers_are_read_from_the_debug_lines():
+    """bench.py's breakdown of a request made through prepXfer comes from the debug lines of the
+    agent and of the plugin: one entry per request and phase, other lines ignored."""
+    sys.path.insert(0, ROOT)
+    import bench
+    text = "\n".join([
+        "[nixl D] backend HIP: prepared 524288 descriptors into 1 strides",
+        "[nixl D] makeXferReq: merged 65536 indices into 65536 descriptors in 128.5 us",
+        "[nixl D] HIP backend: prepXfer of 65536 descriptors (blocks): block pass 124.525 us, plan from records 8.03 us, "
+        "rest (general lowering, event, stream) 0.611 us",
+        "[nixl D] makeXferReq: merged 65536 indices into 65472 descriptors in 1.3e+02 us",
+        "[nixl D] HIP backend: prepXfer of 65472 descriptors (general): block pass 0 us, plan from records 0 us, "
+        "rest (general lowering, event, stream) 2500.5 us"])
+    phases, paths = bench.parse_prep_debug_lines(text)
+    assert phases == {"agent_expand_index_pairs": [128.5, 130.0], "plugin_block_pass": [124.525, 0.0],
+                      "plugin_plan_from_records": [8.03, 0.0], "plugin_rest": [0.611, 2500.5]}
+    assert paths == ["blocks", "general"]
