@@ -195,6 +195,15 @@ nixl_amd_copy_block_len_fits(uint64_t len, const nixl_amd_copy_tuning_t *tuning)
 int
 nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream);
 
+/* Whether the plan's launches have completed: NIXL_AMD_OK when all have (or none was made),
+ * NIXL_AMD_ERR_BUSY while one still runs (no error text is recorded for that answer: the call
+ * is made to be polled), another negative status if a launch failed.  With `wait` non-zero the
+ * call blocks until the answer is not BUSY.  This is what nixlBackendEngine::checkXfer
+ * (src/api/cpp/backend/backend_engine.h:153) asks of a posted request.  Launches recorded
+ * into a HIP graph are not tracked. */
+int
+nixl_amd_copy_plan_status(nixl_amd_copy_plan_t *plan, int wait);
+
 /* Free the plan's device arrays.  While a launch of the plan has not completed the call
  * returns NIXL_AMD_ERR_BUSY and leaves the plan as it is (its arrays would go back to a pool
  * that the next plan's upload writes into): wait for the launch, then destroy again.  Launches

@@ -91,6 +91,8 @@ def kernels():
         getattr(lib, fn).restype = c_int
     lib.nixl_amd_copy_plan_launch.argtypes = [c_void_p, c_void_p]
     lib.nixl_amd_copy_plan_destroy.argtypes = [c_void_p]
+    lib.nixl_amd_copy_plan_status.argtypes = [c_void_p, c_int]
+    lib.nixl_amd_copy_plan_status.restype = c_int
     lib.nixl_amd_copy_plan_query.argtypes = [c_void_p, POINTER(CopyPlanInfo)]
     lib.nixl_amd_copy_plan_time.argtypes = [c_void_p, c_void_p, c_int, POINTER(c_float)]
     for fn in ("nixl_amd_copy_plan_create", "nixl_amd_copy_plan_launch",
@@ -147,8 +149,8 @@ def kernel_symbols():
     return sorted(["nixl_amd_last_error", "nixl_amd_device_count", "nixl_amd_copy_plan_create", "nixl_amd_copy_plan_create_indexed",
                    "nixl_amd_copy_plan_create_indexed_runs", "nixl_amd_copy_records_begin",
                    "nixl_amd_copy_plan_create_from_records", "nixl_amd_copy_records_abandon", "nixl_amd_copy_block_len_fits",
-                   "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_query",
-                   "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
+                   "nixl_amd_copy_plan_launch", "nixl_amd_copy_plan_destroy", "nixl_amd_copy_plan_status",
+                   "nixl_amd_copy_plan_query", "nixl_amd_copy_plan_time", "nixl_amd_ep_ll_workspace_bytes"] + list(_EP_SIGS))
 
 
 # ---------------------------------------------------------------------------------------

@@ -1448,6 +1448,20 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream) {
 }
 
 int
+nixl_amd_copy_plan_status(nixl_amd_copy_plan_t *plan, int wait) {
+    if (!plan) return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "plan_status: plan is null");
+    if (!plan->launched_valid) return NIXL_AMD_OK;
+    const DeviceScope on_device(plan->device);
+    const hipError_t state = wait ? hipEventSynchronize(plan->launched) : hipEventQuery(plan->launched);
+    if (state == hipSuccess) return NIXL_AMD_OK;
+    if (state == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return NIXL_AMD_ERR_BUSY; // polled in a loop: no message is made for it
+    }
+    return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("plan_status: ") + hipGetErrorString(state));
+}
+
+int
 nixl_amd_copy_plan_destroy(nixl_amd_copy_plan_t *plan) {
     if (!plan) return NIXL_AMD_OK;
     const DeviceScope on_device(plan->device);

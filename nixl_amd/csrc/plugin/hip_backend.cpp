@@ -113,7 +113,19 @@ nixlHipEngine::unmapMailbox(Mailbox *m) {
 nixlHipReqH::~nixlHipReqH() {
     const DeviceScope on_device(device);
     if (plan) (void)nixl_amd_copy_plan_destroy(plan);
-    if (done) (void)hipEventDestroy(done);
+}
+
+// NIXL_SUCCESS when nothing of the request is running any more, NIXL_IN_PROG while its posted
+// copy runs, NIXL_ERR_BACKEND if it failed.  The plan itself keeps the event behind its last
+// launch, so a post costs one event record, not two.
+nixl_status_t
+nixlHipReqH::state(bool wait) const {
+    if (!posted) return NIXL_SUCCESS;
+    const int rc = nixl_amd_copy_plan_status(plan, wait ? 1 : 0);
+    if (rc == NIXL_AMD_OK) return NIXL_SUCCESS;
+    if (rc == NIXL_AMD_ERR_BUSY) return NIXL_IN_PROG;
+    NIXL_ERROR << "HIP backend: transfer failed: " << nixl_amd_last_error();
+    return NIXL_ERR_BACKEND;
 }
 
 nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
@@ -244,11 +256,9 @@ nixlHipEngine::reapRetired(bool wait) const {
     std::lock_guard<std::mutex> lock(retiredMutex_);
     size_t keep = 0;
     for (nixlHipReqH *r : retired_) {
-        const DeviceScope on_device(r->device);
-        hipError_t state = hipSuccess;
-        if (r->posted) state = wait ? hipEventSynchronize(r->done) : hipEventQuery(r->done);
-        if (state != hipErrorNotReady) {
-            deliverPending(r, state == hipSuccess);
+        const nixl_status_t state = r->state(wait);
+        if (state != NIXL_IN_PROG) {
+            deliverPending(r, state == NIXL_SUCCESS);
             delete r;
         } else
             retired_[keep++] = r;
@@ -639,9 +649,6 @@ nixlHipEngine::prepXfer(const nixl_xfer_op_t &operation,
     }
     req->device = device;
     req->bytes = bytes;
-    const DeviceScope on_device(device);
-    if (!on_device.ok() || !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
-        return NIXL_ERR_BACKEND;
     req->stream = pickStream(device);
     if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
 
@@ -736,9 +743,6 @@ nixlHipEngine::prepXferIndexed(const nixl_xfer_op_t &operation,
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
         return NIXL_ERR_BACKEND;
     }
-    const DeviceScope on_device(device);
-    if (!on_device.ok() || !hipOk(hipEventCreateWithFlags(&req->done, hipEventDisableTiming), "hipEventCreateWithFlags"))
-        return NIXL_ERR_BACKEND;
     req->stream = pickStream(device);
     if (!req->stream && !useExternalStream_) return NIXL_ERR_BACKEND;
     handle = req.release();
@@ -757,18 +761,17 @@ nixlHipEngine::postXfer(const nixl_xfer_op_t &,
     const DeviceScope on_device(req->device);
     if (!on_device.ok()) return NIXL_ERR_BACKEND;
     if (req->posted) {
-        const hipError_t earlier = hipEventQuery(req->done);
-        if (earlier == hipErrorNotReady) return NIXL_ERR_REPOST_ACTIVE;
+        const nixl_status_t earlier = req->state(false);
+        if (earlier == NIXL_IN_PROG) return NIXL_ERR_REPOST_ACTIVE;
         // the notification of an earlier post that nobody polled to completion goes out first
-        deliverPending(req, earlier == hipSuccess);
+        deliverPending(req, earlier == NIXL_SUCCESS);
     }
 
     if (nixl_amd_copy_plan_launch(req->plan, req->stream) != NIXL_AMD_OK) {
         NIXL_ERROR << "HIP backend: " << nixl_amd_last_error();
         return NIXL_ERR_BACKEND;
     }
-    if (!hipOk(hipEventRecord(req->done, req->stream), "hipEventRecord")) return NIXL_ERR_BACKEND;
-    req->posted = true;
+    req->posted = true; // the launch recorded the plan's event behind its kernels
     if (opt_args && opt_args->hasNotif) {
         // only now: whoever sees the flag must find the event of THIS post behind it
         std::lock_guard<std::mutex> lock(pendingMutex_);
@@ -788,34 +791,25 @@ nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_ERR_INVALID_PARAM;
     if (!req->posted) return NIXL_SUCCESS; // nothing outstanding
-    const DeviceScope on_device(req->device);
-    if (!on_device.ok()) return NIXL_ERR_BACKEND;
-    const hipError_t e = hipEventQuery(req->done);
-    if (e == hipSuccess) {
-        // the peer learns of the transfer only after its bytes have landed
-        deliverPending(req, true);
-        return NIXL_SUCCESS;
-    }
-    if (e == hipErrorNotReady) return NIXL_IN_PROG;
-    deliverPending(req, false);
-    NIXL_ERROR << "HIP backend: transfer failed: " << hipGetErrorString(e);
-    return NIXL_ERR_BACKEND;
+    const nixl_status_t state = req->state(false);
+    // the peer learns of the transfer only after its bytes have landed
+    if (state != NIXL_IN_PROG) deliverPending(req, state == NIXL_SUCCESS);
+    return state;
 }
 
 nixl_status_t
 nixlHipEngine::releaseReqH(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_SUCCESS;
-    const DeviceScope on_device(req->device);
-    const hipError_t state = req->posted ? hipEventQuery(req->done) : hipSuccess;
-    if (state == hipErrorNotReady) {
+    const nixl_status_t state = req->state(false);
+    if (state == NIXL_IN_PROG) {
         // A launched kernel cannot be cancelled; keep its plan alive until it has
         // drained and free it from a later call, so that this call never blocks.
         std::lock_guard<std::mutex> lock(retiredMutex_);
         retired_.push_back(req);
         return NIXL_SUCCESS;
     }
-    deliverPending(req, state == hipSuccess);
+    deliverPending(req, state == NIXL_SUCCESS);
     delete req;
     return NIXL_SUCCESS;
 }
@@ -867,14 +861,13 @@ nixlHipEngine::progressLoop() {
             if (stopProgress_) return;
             for (size_t i = 0; i < watched_.size();) {
                 nixlHipReqH *req = watched_[i];
-                const DeviceScope on_device(req->device);
-                const hipError_t state = hipEventQuery(req->done);
-                if (state == hipErrorNotReady) {
+                const nixl_status_t state = req->state(false);
+                if (state == NIXL_IN_PROG) {
                     ++i;
                     continue;
                 }
                 req->notifPending = false;
-                if (state == hipSuccess)
+                if (state == NIXL_SUCCESS)
                     ready.emplace_back(req->notifTarget, req->notifMsg);
                 else
                     NIXL_ERROR << "HIP backend: transfer failed, notification for agent '" << req->notifTarget

@@ -73,7 +73,6 @@ public:
 class nixlHipReqH : public nixlBackendReqH {
 public:
     nixl_amd_copy_plan_t *plan = nullptr;
-    hipEvent_t done = nullptr;
     hipStream_t stream = nullptr;
     int device = 0;
     bool posted = false;
@@ -85,6 +84,8 @@ public:
     std::string notifMsg;
 
     ~nixlHipReqH() override;
+    nixl_status_t
+    state(bool wait) const;
 };
 
 class nixlHipEngine : public nixlBackendEngine {
