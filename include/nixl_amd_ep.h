@@ -46,14 +46,14 @@ nixl_amd_ep_ll_workspace_bytes(int num_ranks, int num_experts, int num_tokens, i
  * (kernels/api.cuh:211-224; kernel kernels/nixl_ep_ll.cu:71-395; host
  * csrc/nixl_ep.cpp:1030-1143).
  *   x                      [R][T][H] bf16
- *   topk_idx               [R][T][K] int32, -1 = no selection; the K entries of one token
- *                          must be distinct (as a top-k selection is).  The reference gives a
- *                          repeated expert a row of its own (kernels/nixl_ep_ll.cu:186-190); here
- *                          the repeats share one row, and the call reports it:
+ *   topk_idx               [R][T][K] int32, -1 = no selection.  A token that names an expert
+ *                          more than once gets a row of that expert per selection, as in the
+ *                          reference (kernels/nixl_ep_ll.cu:186-190: a slot per selection), in
+ *                          (token, selection) order; such a call counts its rows from the
+ *                          selection instead of from the selection bits (slower, and reported:
  *                          nixl_amd_ep_ll_dispatch_status then returns
- *                          NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT.  Dispatch, experts and combine
- *                          together still give the reference's result: its two rows hold the
- *                          same data and its combine reads one of them for both selections
+ *                          NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT).  An expert that would receive
+ *                          more than N rows this way loses the rows beyond N
  *   num_tokens_per_rank    [R] int32 tokens present on each rank (<= T), or NULL = T
  *   mask_buffer            [R][R] int32 or NULL; tokens travel a -> b only if neither
  *                          mask[a][b] nor mask[b][a] is set (kernels/nixl_ep_ll.cu:197,266,319)
@@ -134,9 +134,10 @@ nixl_amd_ep_ll_route_dispatch(void *packed_recv_x,
                               void *stream);
 
 /* Status of the last dispatch that used `workspace`, read back after waiting for `stream`:
- * 0, or NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT if some token's top-k named an expert twice (the
- * reference would have delivered that token to the expert twice; here it arrives once).  No
- * reference counterpart: the reference has no such restriction. */
+ * 0, or NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT if some token's selection named an expert twice
+ * (handled as the reference handles it, a row per selection; a caller whose selection is meant
+ * to be a top-k learns here that it was not).  The word is written by the receive phase.  No
+ * reference counterpart. */
 #define NIXL_AMD_EP_STATUS_DUPLICATE_EXPERT 1
 int
 nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status);
@@ -152,7 +153,10 @@ nixl_amd_ep_ll_dispatch_status(const void *workspace, void *stream, int *status)
  *            selections, at most that long per rank; a rank whose selections have not come is
  *            taken as having sent nothing and mask_buffer[dst][rank] is set for every dst, as
  *            the reference's receivers do (kernels/nixl_ep_ll.cu:316-340; the budget there is
- *            in clock cycles, csrc/nixl_ep.cpp:49-52).  Needs mask_buffer.
+ *            in clock cycles, csrc/nixl_ep.cpp:49-52).  Needs mask_buffer.  At most 100 s (the
+ *            upper end of the reference's defaults).  A receive phase whose workspace holds no
+ *            send phase's stamp (issued on its own, or on another workspace) waits for nothing:
+ *            ranks whose selections are not there are masked at once.
  *   dispatch_wait_recv_cost_stats  [R] int64 or NULL: ticks of the GPU's constant-rate wall
  *            clock spent waiting for each source rank, accumulated (kernels/nixl_ep_ll.cu:349).
  *   withhold_rank  -1, or a rank whose send phase leaves out the word its receivers wait for:

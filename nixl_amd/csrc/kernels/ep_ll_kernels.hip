@@ -51,7 +51,13 @@ constexpr int kRouteTokens = 16;
 constexpr int kGroupTokens = 64; // tokens per word of the selection bits
 constexpr int kMaxTopk = 16; // reference limit, kernels/nixl_ep_ll.cu:412,421
 constexpr int kRouterMaxPerLane = 16; // E <= 1024 when routing
-constexpr size_t kWorkspaceHeader = 256; // [0]: status of the last dispatch on this workspace
+// Words of the workspace header: [0] status of the last dispatch on this workspace, [1] arrival
+// stamp of its last send phase, [2] id of the last call in which a token repeated an expert,
+// [3] id of the last call, [4] kSentMagic ^ [1], which tells a receive phase that a send phase
+// wrote [1] (and not whoever had the memory before).
+constexpr size_t kWorkspaceHeader = 256;
+constexpr int kSentMagic = 0x5e4d1a7c;
+constexpr uint64_t kMaxTimeoutUs = 100ull * 1000 * 1000; // 100 s, the upper end of the reference's defaults
 
 struct LlDims {
     int R, T, H, K, E, El, M, N;
@@ -84,6 +90,7 @@ struct BitsArgs {
     LlDims d;
     int Wr; // words (groups of 64 tokens) per rank
     int stamp; // arrival stamp of this call (0 when nobody checks arrivals)
+    int call_id; // never 0; header[3] receives it, and header[2] too if some group holds a repeated expert
     int withhold_rank; // this rank's groups leave their stamp out (its counts "never arrive"), or -1
 };
 
@@ -168,7 +175,14 @@ ll_bits_kernel(BitsArgs a) {
         // The stamp goes out with the flag, after this group's words: what a receiver that
         // checks arrivals (ll_arrival_kernel) waits for.
         if (tid == 0 && r != a.withhold_rank) a.group_status[blockIdx.x] = dup | (a.stamp << 1);
-        if (tid == 0 && blockIdx.x == 0) a.header[1] = a.stamp;
+        if (tid == 0 && blockIdx.x == 0) {
+            a.header[1] = a.stamp;
+            a.header[3] = a.call_id;
+            a.header[4] = kSentMagic ^ a.stamp;
+        }
+        // One word tells the kernels behind this one whether ANY group holds a repeat: it carries
+        // this call's id then, and an older call's id (or whatever the memory held) otherwise.
+        if (tid == 0 && dup) a.header[2] = a.call_id;
     }
 }
 
@@ -200,6 +214,10 @@ __global__ void __launch_bounds__(kArrivalThreads)
 ll_arrival_kernel(ArrivalArgs a) {
     extern __shared__ int late[]; // [R]
     const int stamp = a.header[1];
+    // A header that no send phase wrote (a receive phase issued on its own, or on another
+    // workspace) holds no stamp anybody will ever publish: nothing is waited for then, and every
+    // rank whose flags do not happen to match is masked at once.
+    const bool sent = a.header[4] == (kSentMagic ^ stamp);
     int any_late = 0;
     for (int r = threadIdx.x; r < a.R; r += kArrivalThreads) {
         const int *flags = a.group_status + r * a.Wr;
@@ -208,7 +226,7 @@ ll_arrival_kernel(ArrivalArgs a) {
         for (int w = 0; w < a.Wr; ++w)
             here &= (__hip_atomic_load(flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 1) == stamp;
         long long waited = 0;
-        if (!here) {
+        if (!here && sent) {
             const long long start = wall_clock64();
             long long polls = 0;
             do {
@@ -248,7 +266,8 @@ struct DispatchArgs {
     const int32_t *topk_idx;
     const int *num_tokens_per_rank;
     const unsigned long long *bits; // [E][R][Wr]
-    const int *group_status; // [n_flags]
+    const int *group_status; // [n_flags]; bit 0: some token of the group names an expert twice
+    const int *mask; // [R][R] or null: pairs of ranks whose selections were left out of the bits
     int n_flags; // R * Wr, or 0 when the selection was made here (a top-k never repeats an expert)
     int *status; // workspace header
     int *rows_out; // [R][T][K] final row e * N + slot, -1 if none; may be null
@@ -258,7 +277,39 @@ struct DispatchArgs {
     int parts; // workgroups per token; each covers blockDim.x of the token's H/16 lanes
 };
 
-// layout_range, recv_count and statistics of expert e from its bits; one wave.
+// A call in which some token names an expert twice: one bit per (expert, token) cannot carry
+// how often, so nothing is counted from the bits then; every count comes from the selection
+// itself.  Selections of expert `e` among the (token, selection) pairs of rank `r` that come
+// before (until_t, until_k) in token-major order, taking tokens first, first + step, ...
+// (until_t >= T counts the whole rank).  Every such pair owns a row of the expert, as in the
+// reference (kernels/nixl_ep_ll.cu:186-190: a slot per selection).  Slow on purpose: a top-k
+// selection never repeats an expert, so this only runs for hand-made index tensors.
+__device__ __forceinline__ int
+selections_before(const DispatchArgs &a, int e, int r, int first, int step, int until_t, int until_k) {
+    const LlDims d = a.d;
+    if (pair_blocked(a.mask, d.R, r, e / d.El)) return 0; // such selections were left out of the bits as well
+    const int nt = a.num_tokens_per_rank ? min(a.num_tokens_per_rank[r], d.T) : d.T;
+    const int32_t *idx = a.topk_idx + static_cast<size_t>(r) * d.T * d.K;
+    int n = 0;
+    for (int t = first; t < nt && t <= until_t; t += step) {
+        const int ks = t == until_t ? until_k : d.K;
+        for (int k = 0; k < ks; ++k)
+            n += idx[static_cast<size_t>(t) * d.K + k] == e;
+    }
+    return n;
+}
+
+// Whether some group of this call holds a repeated expert (see ll_bits_kernel): decided once per
+// workgroup from two header words, so that calls without repeats, which is every call whose
+// selection is a top-k, run the same instructions as if repeats did not exist.
+__device__ __forceinline__ bool
+call_has_repeats(const DispatchArgs &a) {
+    return a.n_flags != 0 && a.status[2] == a.status[3];
+}
+
+// layout_range, recv_count and statistics of expert e from its bits (or, in a call with
+// repeats, from the selection); one wave.
+template<bool REPEATS>
 __device__ __forceinline__ void
 expert_meta(const DispatchArgs &a, int e, int lane) {
     const LlDims d = a.d;
@@ -267,9 +318,13 @@ expert_meta(const DispatchArgs &a, int e, int lane) {
     for (int r0 = 0; r0 < d.R; r0 += kWaveSize) {
         const int r = r0 + lane;
         int n_r = 0;
-        if (r < d.R)
-            for (int w = 0; w < a.Wr; ++w)
-                n_r += __popcll(bw[static_cast<size_t>(r) * a.Wr + w]);
+        if (r < d.R) {
+            if constexpr (REPEATS)
+                n_r = selections_before(a, e, r, 0, 1, d.T, 0);
+            else
+                for (int w = 0; w < a.Wr; ++w)
+                    n_r += __popcll(bw[static_cast<size_t>(r) * a.Wr + w]);
+        }
         int incl = n_r;
 #pragma unroll
         for (int off = 1; off < kWaveSize; off <<= 1) {
@@ -303,7 +358,7 @@ __global__ void __launch_bounds__(256)
 ll_meta_kernel(DispatchArgs a) {
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int e = blockIdx.x * 4 + threadIdx.x / kWaveSize;
-    if (e < a.d.E) expert_meta(a, e, lane);
+    if (e < a.d.E) expert_meta<false>(a, e, lane); // no tokens, no repeats
     if (e == 0) reduce_status(a, lane);
 }
 
@@ -311,7 +366,7 @@ ll_meta_kernel(DispatchArgs a) {
 // (32 bytes of bf16, 16 bytes of fp8), so a 128-channel scale group is 8 neighbouring
 // lanes; a workgroup covers blockDim.x of them (a multiple of 64).
 template<bool FP8>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8)))
 ll_dispatch_kernel(DispatchArgs a) {
     const LlDims d = a.d;
     const int tid = threadIdx.x;
@@ -334,9 +389,14 @@ ll_dispatch_kernel(DispatchArgs a) {
     }
 
     // Receive-side metadata: the workgroup of token i derives it for experts i, i + R*T, ...
+    const bool repeats = call_has_repeats(a);
     if (part == 0 && wave == n_waves - 1)
-        for (int e = token; e < d.E; e += d.R * d.T)
-            expert_meta(a, e, wlane);
+        for (int e = token; e < d.E; e += d.R * d.T) {
+            if (repeats)
+                expert_meta<true>(a, e, wlane);
+            else
+                expert_meta<false>(a, e, wlane);
+        }
     if (blockIdx.x == 0 && wave == 0) reduce_status(a, wlane);
 
     if (t >= nt) {
@@ -355,16 +415,26 @@ ll_dispatch_kernel(DispatchArgs a) {
         if (e >= 0 && e < d.E) {
             const unsigned long long *bw = a.bits + static_cast<size_t>(e) * d.R * a.Wr;
             own = bw[wi];
-            if (q0 == 0) cnt = __popcll(own & ((1ull << (t & 63)) - 1ull));
-            for (int j = q0; j < wi; j += 32)
-                cnt += __popcll(bw[j]);
+            if (!repeats) {
+                if (q0 == 0) cnt = __popcll(own & ((1ull << (t & 63)) - 1ull));
+                for (int j = q0; j < wi; j += 32)
+                    cnt += __popcll(bw[j]);
+            } else {
+                // This selection's place among the (rank, token, selection) triples that name the
+                // expert, in that order: the order of the reference's per-selection slots when
+                // ranks and tokens are taken in turn.  The 32 lanes share the tokens out.
+                cnt = selections_before(a, e, r, q0, 32, t, k);
+                for (int rr = 0; rr < r; ++rr)
+                    cnt += selections_before(a, e, rr, q0, 32, d.T, 0);
+            }
         }
         cnt += __shfl_xor(cnt, 16);
         cnt += __shfl_xor(cnt, 8);
         cnt += __shfl_xor(cnt, 4);
         cnt += __shfl_xor(cnt, 2);
         cnt += __shfl_xor(cnt, 1);
-        if ((own >> (t & 63)) & 1ull) row = e * d.N + cnt;
+        // cnt < N unless repeats push an expert beyond the rows it owns: such a row is dropped
+        if (((own >> (t & 63)) & 1ull) && cnt < d.N) row = e * d.N + cnt;
         if (q0 == 0) row_of_k[k] = row;
     }
     uint4 q = make_uint4(0, 0, 0, 0);
@@ -820,6 +890,8 @@ struct LlDispatchCall {
 
 // Stamps of calls that check arrivals: 1 .. 2^30 - 1, never 0 (the stamp of calls that do not).
 std::atomic<uint32_t> g_arrival_stamp{0};
+// Every send phase gets an id of its own (never 0), see BitsArgs::call_id.
+std::atomic<uint32_t> g_call_id{0};
 
 template<bool ROUTE>
 void
@@ -868,7 +940,7 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
         return bad(NIXL_AMD_ERR_INVALID, "a time-out needs a mask buffer to record late ranks in");
     if (c.withhold_rank >= 0 && (c.timeout_us == 0 || c.timeout_us > 1000000))
         return bad(NIXL_AMD_ERR_INVALID, "a withheld rank is waited for: the time-out must be between 1 us and 1 s");
-    if (c.timeout_us > (1ull << 40)) return bad(NIXL_AMD_ERR_INVALID, "time-out too long");
+    if (c.timeout_us > kMaxTimeoutUs) return bad(NIXL_AMD_ERR_INVALID, "the time-out may be at most 100 s");
 
     hipStream_t s = static_cast<hipStream_t>(c.stream);
     const int Wr = (d.T + kGroupTokens - 1) / kGroupTokens;
@@ -887,6 +959,7 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
         b.group_status = group_status;
         b.header = status;
         b.withhold_rank = c.withhold_rank;
+        b.call_id = static_cast<int>(g_call_id.fetch_add(1, std::memory_order_relaxed) % 0x7fffffffu) + 1;
         if (c.timeout_us > 0) {
             const uint32_t n = g_arrival_stamp.fetch_add(1, std::memory_order_relaxed) % 0x3fffffffu;
             b.stamp = static_cast<int>(n + 1);
@@ -941,6 +1014,7 @@ ll_dispatch_impl(const char *who, const LlDispatchCall &c) {
     a.num_tokens_per_rank = c.num_tokens_per_rank;
     a.bits = bits;
     a.group_status = group_status;
+    a.mask = c.mask_buffer;
     a.n_flags = c.logits ? 0 : static_cast<int>(groups);
     a.status = status;
     a.rows_out = c.row_map;

@@ -175,6 +175,12 @@ nixlHipEngine::nixlHipEngine(const nixlBackendInitParams *init_params)
     mailboxName_ = "/nixl_amd_hip_" + std::to_string(static_cast<long long>(getpid())) + "_" +
         std::to_string(g_mailboxCounter.fetch_add(1));
     mailbox_ = mapMailbox(mailboxName_, true);
+    if (!mailbox_ && errno == EEXIST) {
+        // The name holds this process's id: an object of that name is what a process that died
+        // with the same id left behind.
+        shm_unlink(mailboxName_.c_str());
+        mailbox_ = mapMailbox(mailboxName_, true);
+    }
     if (!mailbox_) {
         NIXL_WARN << "HIP backend: no shared-memory mailbox (" << std::strerror(errno) << "); agents of other processes cannot notify '"
                   << localAgent << "'";
@@ -790,6 +796,7 @@ nixl_status_t
 nixlHipEngine::checkXfer(nixlBackendReqH *handle) const {
     auto *req = static_cast<nixlHipReqH *>(handle);
     if (!req) return NIXL_ERR_INVALID_PARAM;
+    flushBacklog();
     if (!req->posted) return NIXL_SUCCESS; // nothing outstanding
     const nixl_status_t state = req->state(false);
     // the peer learns of the transfer only after its bytes have landed
@@ -857,7 +864,7 @@ nixlHipEngine::progressLoop() {
         std::vector<std::pair<std::string, std::string>> ready;
         {
             std::unique_lock<std::mutex> lock(pendingMutex_);
-            pendingCv_.wait(lock, [&] { return stopProgress_ || !watched_.empty(); });
+            pendingCv_.wait(lock, [&] { return stopProgress_ || !watched_.empty() || backlog_.load(std::memory_order_acquire); });
             if (stopProgress_) return;
             for (size_t i = 0; i < watched_.size();) {
                 nixlHipReqH *req = watched_[i];
@@ -879,6 +886,7 @@ nixlHipEngine::progressLoop() {
         for (const auto &[target, msg] : ready)
             if (genNotif(target, msg) != NIXL_SUCCESS)
                 NIXL_WARN << "HIP backend: notification for agent '" << target << "' could not be delivered";
+        flushBacklog(); // messages that found a peer's ring full
         if (ready.empty()) std::this_thread::sleep_for(nap);
     }
 }
@@ -905,6 +913,7 @@ nixlHipEngine::loadRemoteConnInfo(const std::string &remote_agent, const std::st
         // never be told that a transfer has landed.
         if (peer.mailboxName.empty() || peer.mailboxName[0] != '/') return NIXL_ERR_MISMATCH;
         peer.mailbox = mapMailbox(peer.mailboxName, false);
+        peer.sender = nixl_amd_hip::MailboxSender(peer.mailbox);
         if (!peer.mailbox) {
             NIXL_ERROR << "HIP backend: mailbox '" << peer.mailboxName << "' of agent '" << remote_agent << "' (process " << pid
                        << ") cannot be opened";
@@ -1089,22 +1098,41 @@ nixlHipEngine::genNotif(const std::string &remote_agent, const std::string &msg)
     std::lock_guard<std::mutex> lock(peersMutex_);
     const auto it = peers_.find(remote_agent);
     if (it == peers_.end() || !it->second.mailbox) return NIXL_ERR_NOT_FOUND;
-    if (localAgent.size() + msg.size() > kMailboxSlotBytes) {
+    using Result = nixl_amd_hip::MailboxSender::Result;
+    switch (it->second.sender.send(localAgent, msg)) {
+    case Result::kSent:
+        return NIXL_SUCCESS;
+    case Result::kQueued: // the ring is full: the message waits here, in order, until the peer has drained some
+        backlog_.store(true, std::memory_order_release);
+        if (progressOn_) pendingCv_.notify_one(); // the progress thread keeps trying
+        return NIXL_SUCCESS;
+    case Result::kTooLong:
         NIXL_ERROR << "HIP backend: a notification to another process holds at most " << kMailboxSlotBytes
                    << " bytes (agent name included)";
         return NIXL_ERR_NOT_SUPPORTED;
+    default:
+        NIXL_ERROR << "HIP backend: agent '" << remote_agent << "' has not read its mailbox for "
+                   << nixl_amd_hip::MailboxSender::kMaxBacklog << " notifications; it is taken to be gone";
+        return NIXL_ERR_REMOTE_DISCONNECT;
     }
-    if (!it->second.mailbox->push(localAgent, msg)) {
-        NIXL_ERROR << "HIP backend: the mailbox of agent '" << remote_agent << "' is full";
-        return NIXL_ERR_BACKEND;
-    }
-    return NIXL_SUCCESS;
+}
+
+// Messages that found a peer's ring full go out as soon as the peer has made room.
+void
+nixlHipEngine::flushBacklog() const {
+    if (!backlog_.load(std::memory_order_acquire)) return;
+    std::lock_guard<std::mutex> lock(peersMutex_);
+    bool left = false;
+    for (auto &[name, peer] : peers_)
+        if (peer.mailbox && !peer.sender.flush()) left = true;
+    backlog_.store(left, std::memory_order_release);
 }
 
 nixl_status_t
 nixlHipEngine::getNotifs(notif_list_t &notif_list) {
     // transfers released while in flight may have finished since
     reapRetired(false);
+    flushBacklog();
     std::lock_guard<std::mutex> lock(notifMutex_);
     for (auto &n : notifs_)
         notif_list.push_back(std::move(n));

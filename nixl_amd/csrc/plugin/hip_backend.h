@@ -310,8 +310,14 @@ private:
     struct peerInfo {
         long long pid = 0;
         std::string mailboxName;
-        Mailbox *mailbox = nullptr; // mapped on first use
+        Mailbox *mailbox = nullptr; // null for an agent of this process
+        nixl_amd_hip::MailboxSender sender; // messages that found the peer's ring full wait here
     };
+    // Set while some peer's sender holds waiting messages: the calls that an initiator makes
+    // anyway (checkXfer, getNotifs, genNotif, the progress thread) then try to move them on.
+    mutable std::atomic<bool> backlog_{false};
+    void
+    flushBacklog() const;
     mutable std::mutex peersMutex_;
     mutable std::unordered_map<std::string, peerInfo> peers_;
     // This engine's own mailbox, where agents of other processes leave notifications.

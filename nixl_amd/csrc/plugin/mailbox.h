@@ -14,7 +14,9 @@
 #include <atomic>
 #include <cstdint>
 #include <cstring>
+#include <deque>
 #include <string>
+#include <utility>
 
 namespace nixl_amd_hip {
 
@@ -78,6 +80,51 @@ struct Mailbox {
         c.sequence.store(pos + kMailboxSlots, std::memory_order_release);
         return true;
     }
+};
+
+// The sending side of one peer's mailbox: messages that find the ring full wait here, in
+// order, and go out when the peer has drained some (flush, which every later send also does
+// first).  The reference queues notifications without loss; a full ring must not lose one
+// either.  Not thread-safe: the owner serialises its callers.
+class MailboxSender {
+public:
+    static constexpr size_t kMaxBacklog = 65536; // messages; beyond that the peer is taken to be gone
+
+    enum class Result { kSent, kQueued, kTooLong, kBacklogFull };
+
+    explicit MailboxSender(Mailbox *box = nullptr) : box_(box) {}
+
+    Mailbox *
+    box() const {
+        return box_;
+    }
+
+    Result
+    send(const std::string &sender, const std::string &msg) {
+        if (sender.size() + msg.size() > kMailboxSlotBytes) return Result::kTooLong;
+        flush();
+        if (backlog_.empty() && box_->push(sender, msg)) return Result::kSent;
+        if (backlog_.size() >= kMaxBacklog) return Result::kBacklogFull;
+        backlog_.emplace_back(sender, msg);
+        return Result::kQueued;
+    }
+
+    // Moves waiting messages into the ring while it takes them; true when none is left.
+    bool
+    flush() {
+        while (!backlog_.empty() && box_->push(backlog_.front().first, backlog_.front().second))
+            backlog_.pop_front();
+        return backlog_.empty();
+    }
+
+    size_t
+    waiting() const {
+        return backlog_.size();
+    }
+
+private:
+    Mailbox *box_;
+    std::deque<std::pair<std::string, std::string>> backlog_;
 };
 
 // Creates (O_EXCL) or opens the shared-memory object `name` and maps it; nullptr on failure.

@@ -299,8 +299,9 @@ class Buffer:
         int64, nixl_ep_ll.cu:349-350) then accumulates the wall-clock ticks waited per rank.
         return_recv_hook=True issues the send phase only; the hook issues the receive phase
         (`x` must stay as it is until then: the rows are read by the receive phase).
-        `check_duplicates` waits for the kernels and raises if a token named an expert twice
-        (the reference delivers such a token twice, nixl_ep_ll.cu:186-190; here it arrives once).
+        A token that names an expert twice gets a row per selection, as in the reference
+        (nixl_ep_ll.cu:186-190); `check_duplicates` waits for the kernels and raises if that
+        happened (a top-k selection never does it), with return_recv_hook from inside the hook.
         """
         if topk_idx.dim() != 3 or not topk_idx.is_contiguous() or topk_idx.dtype != topk_idx_t:
             raise EPError("topk_idx must be a contiguous [R, T, K] int32 tensor")
@@ -377,7 +378,13 @@ class Buffer:
             if return_recv_hook:
                 rc = issue(1)
                 keep = (x, topk_idx, ws, stats, wait_stats, num_tokens_per_rank)  # alive until the hook has run
-                hook = lambda keep=keep: _check(issue(2), "low_latency_dispatch (receive phase)")  # noqa: E731
+
+                def hook(keep=keep, look=check_duplicates):
+                    _check(issue(2), "low_latency_dispatch (receive phase)")
+                    if look:  # the status word is written by the receive phase
+                        self._raise_on_repeats(ws)
+
+                check_duplicates = False  # not before the receive phase has run
             else:
                 rc = issue(3)
         elif logits is None:
@@ -388,10 +395,7 @@ class Buffer:
             rc = self._k.nixl_amd_ep_ll_route_dispatch(*head, _ptr(logits), _ptr(topk_idx), _ptr(topk_weights), *tail)
         _check(rc, "low_latency_dispatch")
         if check_duplicates:
-            status = ctypes.c_int(0)
-            _check(self._k.nixl_amd_ep_ll_dispatch_status(_ptr(ws), _stream(), ctypes.byref(status)), "dispatch status")
-            if status.value:
-                raise EPError("a token's top-k names the same expert twice")
+            self._raise_on_repeats(ws)
         event = None
         if async_finish:
             event = torch.cuda.Event()
@@ -402,6 +406,12 @@ class Buffer:
         if return_recv_hook and hook is None:
             hook = lambda: None  # noqa: E731  (routing dispatch: issued whole)
         return topk_idx, topk_weights, recv, packed_recv_count, handle, EventOverlap(event), hook
+
+    def _raise_on_repeats(self, ws):
+        status = ctypes.c_int(0)
+        _check(self._k.nixl_amd_ep_ll_dispatch_status(_ptr(ws), _stream(), ctypes.byref(status)), "dispatch status")
+        if status.value:
+            raise EPError("a token's top-k names the same expert twice")
 
     def dispatch(self, *args, **kwargs):
         return self.low_latency_dispatch(*args, **kwargs)

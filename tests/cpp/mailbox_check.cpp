@@ -60,6 +60,30 @@ main() {
         CHECK(m->pop(sender, msg) && msg == std::to_string(i));
     CHECK(!m->pop(sender, msg));
 
+    // a sender whose messages find the ring full keeps them, in order, and delivers them late
+    {
+        nixl_amd_hip::MailboxSender out(m);
+        using Result = nixl_amd_hip::MailboxSender::Result;
+        const uint32_t total = kMailboxSlots + 300;
+        for (uint32_t i = 0; i < total; ++i) {
+            const Result r = out.send("s", std::to_string(i));
+            CHECK(r == (i < kMailboxSlots ? Result::kSent : Result::kQueued));
+        }
+        CHECK(out.waiting() == 300 && !out.flush()); // still full: nothing moves
+        CHECK(out.send("s", std::string(kMailboxSlotBytes, 'x')) == Result::kTooLong);
+        uint32_t next = 0;
+        for (int round = 0; next < total; ++round) {
+            CHECK(round < 10);
+            while (m->pop(sender, msg)) {
+                CHECK(sender == "s" && msg == std::to_string(next));
+                ++next;
+            }
+            out.flush(); // room again: the waiting messages follow, oldest first
+        }
+        CHECK(out.waiting() == 0 && out.send("s", "after") == Result::kSent);
+        CHECK(m->pop(sender, msg) && msg == "after" && !m->pop(sender, msg));
+    }
+
     // producers: threads 0..3 here, producer 4 in a child process that maps the ring by name
     constexpr int kThreads = 4, kCount = 20000;
     const pid_t child = fork();

@@ -735,22 +735,62 @@ def test_ll_dispatch_reports_a_repeated_expert(cuda):
     buf.dispatch(xd, torch.from_numpy(bad).to(cuda), M, E, check_duplicates=True)
 
 
+def _with_repeats(rng, topk, per_rank, triple=True):
+    """Makes `per_rank` tokens of every rank name one of their experts twice (and one token
+    three times), in place; returns the number of selections that became repeats."""
+    R, T, K = topk.shape
+    made = 0
+    for r in range(R):
+        for n, t in enumerate(rng.choice(T, per_rank, replace=False)):
+            ks = rng.choice(K, 3 if (triple and n == 0 and K >= 3) else 2, replace=False)
+            if topk[r, t, ks[0]] < 0:
+                topk[r, t, ks[0]] = 0
+            for k in ks[1:]:
+                topk[r, t, k] = topk[r, t, ks[0]]
+                made += 1
+    return made
+
+
+@pytest.mark.parametrize("use_fp8", [True, False])
+@pytest.mark.parametrize("shape", [(2, 40, 512, 4, 8, 48), (4, 150, 1024, 8, 32, 160), (3, 64, 512, 3, 6, 80)])
+def test_ll_repeated_expert_gets_a_row_per_selection(cuda, shape, use_fp8):
+    """A token that names an expert twice (or three times): the reference gives every selection
+    a slot of its own (kernels/nixl_ep_ll.cu:186-190, an atomicAdd per selection), so the expert
+    receives the token's row once per selection and recv_count, layout_range and src_info count
+    them all.  Every dispatch output equals the oracle's, whose slots follow (token, selection)
+    order; ranks with fewer tokens, a masked pair of ranks and several groups of 64 tokens per
+    rank included.  The status word still says that a repeat was seen."""
+    R, T, H, K, E, M = shape
+    x, topk, _ = make_world(50 + R, R, T, H, K, E, drop=0.05)
+    rng = np.random.default_rng(R * 7 + T)
+    _with_repeats(rng, topk, min(T // 3, 9))
+    nt = np.full(R, T, np.int32)
+    nt[-1] = T - T // 4
+    mask = np.zeros((R, R), np.int32)
+    mask[0, R - 1] = 1
+    stats = torch.zeros((R, E // R), dtype=torch.int32, device=cuda)
+    rc, got = raw_ll_dispatch(cuda, x, topk, E, M, use_fp8, num_tokens=nt, mask=mask, stats=stats)
+    assert rc == 0, _lib.kernels_error()
+    want = eo.ll_dispatch(bits16(x), topk, E, M, use_fp8, num_tokens=nt, mask=mask, fill=0x55)
+    El = E // R
+    rows = sum(1 for r in range(R) for t in range(nt[r]) for e in topk[r, t]
+               if e >= 0 and not (mask[r, e // El] or mask[e // El, r]))
+    assert int(want["recv_count"].sum()) == rows  # a row per selection, repeats included
+    assert_dispatch_equal(got, want, use_fp8)
+    assert np.array_equal(stats.cpu().numpy(), want["recv_count"])
+
+
 def test_ll_repeated_expert_combines_as_in_the_reference(cuda):
     """A token that names an expert twice: the reference gives the token two rows at that expert
     (kernels/nixl_ep_ll.cu:186-190), both hold the same data, and its combine reads, for each of
     the two selections, the row that was written back last into the token's slot for that
-    expert (kernels/nixl_ep_ll.cu:959-1012): w1 * y + w2 * y.  Here the two selections share one
-    row, so dispatch counts one row less, and combine must give the same bytes as the oracle's
-    pipeline with the reference's slotting."""
+    expert (kernels/nixl_ep_ll.cu:959-1012): w1 * y + w2 * y.  Dispatch gives the two rows here
+    too, combine reads each selection's own row, and the result equals the oracle's pipeline
+    bit for bit, with the row map of the dispatch and with the rows found through src_info."""
     R, T, H, K, E, M = 2, 40, 512, 4, 8, 48
     x, topk, w = make_world(31, R, T, H, K, E, drop=0.0)
     rng = np.random.default_rng(7)
-    dups = 0
-    for r in range(R):
-        for t in rng.choice(T, 6, replace=False):
-            a, b = rng.choice(K, 2, replace=False)
-            topk[r, t, b] = topk[r, t, a]
-            dups += 1
+    _with_repeats(rng, topk, 6, triple=False)
     El = E // R
     buf = Buffer(R, device=cuda)
     td, wd = torch.from_numpy(topk).to(cuda), torch.from_numpy(w).to(cuda)
@@ -764,7 +804,8 @@ def test_ll_repeated_expert_combines_as_in_the_reference(cuda):
     assert torch.equal(got.view(torch.int16), searched.view(torch.int16))
 
     ref = eo.ll_dispatch(bits16(x), topk, E, M, use_fp8=False)  # every (token, selection) a slot of its own
-    assert int(ref["recv_count"].sum()) == R * T * K and int(cnt.sum().item()) == R * T * K - dups
+    assert int(ref["recv_count"].sum()) == R * T * K and int(cnt.sum().item()) == R * T * K
+    assert np.array_equal(cnt.cpu().numpy(), ref["recv_count"])
     ref_x = torch.from_numpy(ref["recv_x"].view(np.int16)).view(torch.bfloat16)
     ref_valid = (np.arange(R * M).reshape(1, 1, -1) < ref["recv_count"][..., None])[..., None]
     ref_y = (ref_x.float() * factor.cpu()).to(torch.bfloat16)
@@ -785,9 +826,11 @@ def test_ll_dispatch_without_tokens(cuda):
 
 # ---- the receive side's bounded wait: time-out -> mask (kernels/nixl_ep_ll.cu:316-340, 846-866) -----
 
-def raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, phases=(3,), timeout_us=0, withhold=-1, wait=None, fill=0x55):
+def raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, phases=(3,), timeout_us=0, withhold=-1, wait=None, fill=0x55,
+                           header=None):
     """nixl_amd_ep_ll_dispatch_phased through the C ABI on buffers pre-filled with `fill`; one
-    call per entry of `phases`, on the same buffers and workspace."""
+    call per entry of `phases`, on the same buffers and workspace.  `header`: the workspace
+    starts zeroed with these int32 words at its front instead of as allocated."""
     k = _lib.ep_kernels()
     R, T, H = x.shape
     K = topk.shape[2]
@@ -799,6 +842,9 @@ def raw_ll_dispatch_phased(cuda, x, topk, E, M, use_fp8, mask, phases=(3,), time
     layout = torch.zeros((R, El, R), dtype=torch.int64, device=cuda)
     count = torch.zeros((R, El), dtype=torch.int32, device=cuda)
     ws = torch.empty(k.nixl_amd_ep_ll_workspace_bytes(R, E, T, K, H), dtype=torch.uint8, device=cuda)
+    if header is not None:
+        ws.zero_()
+        ws[:4 * len(header)].view(torch.int32).copy_(torch.tensor(header, dtype=torch.int32))
     p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
     rcs = []
     for ph in phases:
@@ -873,6 +919,18 @@ def test_ll_dispatch_in_two_phases(cuda):
         assert rcs == [-1], kwargs
     rcs, _, _ = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, None, timeout_us=10)  # a time-out needs a mask buffer
     assert rcs == [-1]
+    rcs, _, _ = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, mask, timeout_us=100_000_001)  # at most 100 s
+    assert rcs == [-1] and "100 s" in _lib.kernels_error()
+    # A receive phase on a workspace that no send phase has written (here: a stamp nobody
+    # published, no flags) must not wait out its budget: every rank is masked at once and nothing
+    # is placed.  The budget is a second; the call is back long before.
+    import time
+    late_mask = torch.zeros((R, R), dtype=torch.int32, device=cuda)
+    t0 = time.perf_counter()
+    rcs, _, got = raw_ll_dispatch_phased(cuda, x, topk, E, M, True, late_mask, phases=(2,), timeout_us=1_000_000,
+                                         header=[0, 12345, 0, 0, 0])
+    assert rcs == [0] and time.perf_counter() - t0 < 0.5
+    assert bool(late_mask.all()) and not got["recv_count"].any()
 
 
 def test_buffer_time_out_hooks_and_ready_flags(cuda):
