@@ -73,6 +73,100 @@ def counter_samples(csv_path, counters, kernel_tag="copy_uniform_kernel", yardst
             len(kernel[counters[0]]))
 
 
+def counter_medians(csv_path, counters, tags, yardstick_tag="CUDAFunctorOnSelf_add<int>"):
+    """The same file read for several kernels at once: ({tag: {counter: median over the
+    dispatches of the kernels whose name contains tag}}, {counter: largest value over the
+    yardstick's dispatches}).  A tag without samples is left out."""
+    import csv
+    import statistics
+    seen = {t: {c: [] for c in counters} for t in tags}
+    yard = {c: [] for c in counters}
+    with open(csv_path, newline="") as f:
+        for row in csv.DictReader(f):
+            c, name = row.get("Counter_Name"), row.get("Kernel_Name", "")
+            if c not in yard:
+                continue
+            if yardstick_tag in name:
+                yard[c].append(float(row["Counter_Value"]))
+            for t in tags:
+                if t in name:
+                    seen[t][c].append(float(row["Counter_Value"]))
+    medians = {t: {c: statistics.median(v) for c, v in per.items()} for t, per in seen.items() if all(per.values())}
+    return medians, {c: (max(v) if v else None) for c, v in yard.items()}
+
+
+def _counter_run(child, counters, timeout=150):
+    """One child run under `rocprofv3 --pmc <counters>`; returns the path of its counter file
+    inside a temporary directory the caller removes, or {"error": why}."""
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    prof = shutil.which("rocprofv3")
+    if not prof:
+        return None, {"error": "rocprofv3 not found"}
+    if any("rocprof" in os.environ.get(k, "") for k in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB")):
+        return None, {"error": "this process already runs under a profiler"}
+    out_dir = tempfile.mkdtemp(prefix="nixl_amd_pmc_", dir="/tmp")
+    cmd = [prof, "--pmc", *counters, "--output-format", "csv", "-d", out_dir, "-o", "t", "--"] + child
+    proc = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, stdout=subprocess.DEVNULL,
+                            stderr=subprocess.DEVNULL, start_new_session=True)
+    try:
+        rc = proc.wait(timeout=timeout)
+    except subprocess.TimeoutExpired:
+        os.killpg(proc.pid, signal.SIGKILL)
+        proc.wait()
+        return out_dir, {"error": f"the counter run did not finish in {timeout} s"}
+    if rc != 0:
+        return out_dir, {"error": f"the counter run ended with status {rc}"}
+    files = glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+        return out_dir, {"error": "the counter run left no counter file"}
+    return out_dir, files[0]
+
+
+def measure_ep_traffic_live():
+    """HBM bytes of each expert-parallel call from hardware counters, measured now: the four
+    calls are run by a child process (nixl_amd/ep_bench.py run_traffic_child) under `rocprofv3
+    --pmc`, once for the read requests by size class and once for WRITE_SIZE, with the same 1 GiB
+    element-wise yardstick as the KV figure; a call's bytes are the sum over its kernels of the
+    median per launch.  Returns {call: {"traffic", "traffic_source", "traffic_by_kernel"}} or
+    {"error": why}."""
+    import shutil
+    from nixl_amd import ep_bench
+    child = [sys.executable, os.path.abspath(__file__), "--ep-traffic-child"]
+    read_classes = {"TCC_EA0_RDREQ_128B_sum": 128, "TCC_EA0_RDREQ_64B_sum": 64, "TCC_EA0_RDREQ_32B_sum": 32}
+    tags = sorted({k for ks in ep_bench.CALL_KERNELS.values() for k in ks})
+    got = {}
+    for run, counters in (("read", list(read_classes)), ("write", ["WRITE_SIZE"])):
+        out_dir, found = _counter_run(child, counters, timeout=200)
+        try:
+            if isinstance(found, dict):
+                return {"error": f"{run}: {found['error']}"}
+            got[run] = counter_medians(found, counters, tags)
+        finally:
+            if out_dir:
+                shutil.rmtree(out_dir, ignore_errors=True)
+    if not got["write"][1]["WRITE_SIZE"]:
+        return {"error": "the write counter shows nothing for the yardstick"}
+    write_scale = (1 << 20) / got["write"][1]["WRITE_SIZE"]
+    out = {}
+    for call, kernels in ep_bench.CALL_KERNELS.items():
+        per_kernel = {}
+        for k in kernels:
+            if k not in got["read"][0] or k not in got["write"][0]:
+                return {"error": f"no counter samples of {k}"}
+            read = sum(got["read"][0][k][c] * size for c, size in read_classes.items())
+            written = got["write"][0][k]["WRITE_SIZE"] * write_scale * 1024.0
+            per_kernel[k] = int(round(read + written))
+        out[call] = {"traffic": sum(per_kernel.values()), "traffic_by_kernel": per_kernel,
+                     "traffic_source": "rocprofv3 --pmc over two child runs of this bench invocation (the four expert-parallel "
+                                       "calls alone), median per launch summed over the call's kernels: reads = the L2's requests "
+                                       "to memory by size class, writes = WRITE_SIZE scaled by a 1 GiB element-wise kernel"}
+    return out
+
+
 def measure_traffic_live(args, blk):
     """HBM bytes per launch of the headline kernel from hardware counters, measured now: the
     headline leg of this file is run twice more as a child process under `rocprofv3 --pmc`.
@@ -447,6 +541,92 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, 
         h.release()
     agent.close()
     del src_pool, dst_pool, staging
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_concurrent_requests(args, blk, counts=(1, 2, 4), steps=10, warmup=3):
+    """Several requests of config 2's shape in flight at once (the reference benchmark drives
+    one request per thread, benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:1847-1879):
+    n gathers posted together, each on a stream of its own (backend parameter num_streams=n),
+    waited for, then the n scatters the same way; aggregate payload GB/s by wall clock beside
+    the same loop with one request at a time.  Every request has its own staging buffer and its
+    own block set; the scatters' destination blocks are disjoint, and the bytes are checked."""
+    import torch
+    from nixl_amd import nixl_agent, nixl_agent_config
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    kv = _kv_layout()
+    pool_blocks, n_sel = args.pool_blocks, args.blocks
+    lk = kv.layers * kv.sub_blocks_per_layer
+    n_max = max(counts)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(77)
+    src_pool = torch.empty((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+    for i in range(lk):
+        src_pool[i] = torch.randn((pool_blocks, blk // 2), generator=gen, device=dev).to(torch.bfloat16)
+    dst_pool = torch.zeros((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+    stagings = [torch.zeros((n_sel * lk, blk // 2), dtype=torch.bfloat16, device=dev) for _ in range(n_max)]
+    n_desc, n_pool = n_sel * lk, lk * pool_blocks
+    pool_offsets = np.arange(n_pool, dtype=np.uint64) * np.uint64(blk)
+    stg_idx = np.arange(n_desc, dtype=np.int32)
+    rng = np.random.default_rng(5)
+    dst_perm = rng.permutation(pool_blocks)
+    out = {}
+    for n in counts:
+        agent = nixl_agent("bench_c", nixl_agent_config(backends=()))
+        agent.create_backend("HIP", {"num_streams": str(n), **dict(kv.split("=", 1) for kv in args.backend_param)})
+        agent.register_memory([src_pool, dst_pool] + stagings[:n])
+        h_src = agent.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+        h_dst = agent.prep_xfer_dlist("bench_c", _triples(np.uint64(dst_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+        handles, gathers, scatters, sets = [h_src, h_dst], [], [], []
+        for i in range(n):
+            stg_addrs = np.uint64(stagings[i].data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
+            h_r = agent.prep_xfer_dlist("bench_c", _triples(stg_addrs, blk), "VRAM")
+            h_l = agent.prep_xfer_dlist("", _triples(stg_addrs, blk), "VRAM")
+            handles += [h_r, h_l]
+            sel = rng.choice(pool_blocks, n_sel, replace=False)
+            dst_ids = dst_perm[i * n_sel:(i + 1) * n_sel]  # disjoint between the requests
+            sets.append((sel, dst_ids))
+            gathers.append(agent.make_prepped_xfer("WRITE", h_src, _kv_indices(lk, pool_blocks, sel, args.order), h_r, stg_idx))
+            scatters.append(agent.make_prepped_xfer("WRITE", h_l, stg_idx, h_dst, _kv_indices(lk, pool_blocks, dst_ids, args.order)))
+
+        def phase(reqs):
+            for req in reqs:
+                if agent.transfer(req) not in ("PROC", "DONE"):
+                    raise RuntimeError("post failed")
+            for req in reqs:
+                state = agent.check_xfer_state(req)
+                while state == "PROC":
+                    state = agent.check_xfer_state(req)
+                if state != "DONE":
+                    raise RuntimeError(f"transfer ended in state {state}")
+
+        torch.cuda.synchronize()
+        for _ in range(warmup):
+            phase(gathers)
+            phase(scatters)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            phase(gathers)
+            phase(scatters)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        for sel, dst_ids in sets:
+            sel_t, dst_t = torch.from_numpy(sel).to(dev), torch.from_numpy(dst_ids).to(dev)
+            if not torch.equal(dst_pool[:, dst_t, :].view(torch.int16), src_pool[:, sel_t, :].view(torch.int16)):
+                raise RuntimeError("scattered blocks differ from the source blocks")
+        out[f"{n}_in_flight"] = {"aggregate_GBps": round(n * 2 * n_desc * blk * steps / wall / 1e9, 1),
+                                 "ms_per_step": round(wall / steps * 1e3, 4), "streams": n}
+        for req in gathers + scatters:
+            req.release()
+        for h in handles:
+            h.release()
+        agent.close()
+    out["note"] = ("n gather requests posted together (a stream each) and waited for, then the n scatter requests: wall clock, "
+                   f"payload of all requests; {steps} steps; descriptors of {blk} B; bytes verified")
+    del src_pool, dst_pool, stagings
     torch.cuda.empty_cache()
     return out
 
@@ -885,6 +1065,7 @@ def main():
                     help="also run one plain element-wise kernel that reads 1 GiB and writes 1 GiB, as the "
                          "known-size yardstick for hardware counter runs")
     ap.add_argument("--prep-breakdown-child", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--ep-traffic-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-live-traffic", action="store_true",
                     help="do not run the headline leg under rocprofv3 --pmc first; roofline.traffic then comes from "
                          "the counter runs summarised under profiles/")
@@ -899,6 +1080,11 @@ def main():
     blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
     if args.prep_breakdown_child:
         run_prep_breakdown_child(args, blk)
+        return
+    if args.ep_traffic_child:
+        from nixl_amd import ep_bench
+        run_calibration_copy()
+        ep_bench.run_traffic_child()
         return
     if args.calibrate_copy:
         run_calibration_copy()
@@ -947,6 +1133,8 @@ def main():
             return others
 
         line["kv"]["other_points"] = _leg(other_points)
+    if not args.quick:
+        line["kv"]["concurrent_requests"] = _leg(run_concurrent_requests, args, blk)
     if not args.no_small:
         line["kv"]["small_descriptor_stress"] = _leg(run_small_descriptors)
     if not args.quick:
@@ -974,6 +1162,13 @@ def main():
     # kernel times unchanged); behind them they disturb nothing.
     if not args.quick:
         line["kv"]["through_prepxfer"]["prep_breakdown_us"] = _leg(measure_prep_breakdown, args, blk)
+    if not args.no_live_traffic and not args.no_ep and "low_latency" in line.get("ep", {}):
+        ep_live = _leg(measure_ep_traffic_live)
+        for mode, call, key in (("low_latency", "dispatch", "ll_dispatch"), ("low_latency", "combine", "ll_combine"),
+                                ("normal", "dispatch", "ht_dispatch"), ("normal", "combine", "ht_combine")):
+            slot = line["ep"].get(mode, {}).get(call)
+            if isinstance(slot, dict):
+                slot.update(ep_live[key] if key in ep_live else {"traffic": None, "traffic_live_error": ep_live.get("error")})
     live = None if args.no_live_traffic else measure_traffic_live(args, blk)
     if live and "bytes" in live:
         line["roofline"]["traffic"] = live["bytes"]

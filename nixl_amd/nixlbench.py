@@ -48,6 +48,9 @@ def parse(argv=None):
     ap.add_argument("--warmup_iter", type=int, default=100)
     ap.add_argument("--large_blk_iter_ftr", type=int, default=16)
     ap.add_argument("--pipeline_depth", type=int, default=1)
+    ap.add_argument("--num_threads", type=int, default=1,
+                    help="threads that each drive their own requests over their own part of the buffers; num_iter must "
+                         "be divisible by it (utils.cpp:94-98)")
     ap.add_argument("--recreate_xfer", action="store_true")
     ap.add_argument("--prepared_xfer", action="store_true")
     ap.add_argument("--randomize_location_mode", default="none", choices=["none", "blockaligned"])
@@ -60,8 +63,10 @@ def parse(argv=None):
         ap.error("batch sizes must satisfy 0 < start_batch_size <= max_batch_size")
     if a.pipeline_depth < 1 or a.num_iter < 1 or a.warmup_iter < 0:
         ap.error("pipeline_depth and num_iter must be positive, warmup_iter non-negative")
-    if a.max_block_size * a.max_batch_size * 2 > a.total_buffer_size:
-        ap.error("max_block_size * max_batch_size needs two buffers inside total_buffer_size")
+    if a.num_threads < 1 or a.num_iter < a.num_threads or a.num_iter % a.num_threads:
+        ap.error("num_iter must be at least num_threads and divisible by it")
+    if a.max_block_size * a.max_batch_size * 2 * a.num_threads > a.total_buffer_size:
+        ap.error("max_block_size * max_batch_size needs two buffers a thread inside total_buffer_size")
     return a
 
 
@@ -88,18 +93,18 @@ class Segment:
             self.addr = self.buf.ctypes.data
         self.dev = device_id if kind == "VRAM" else 0
 
-    def fill(self, host_bytes):
+    def fill(self, host_bytes, at=0):
         if self.kind == "VRAM":
-            self.buf[:host_bytes.size].copy_(self._torch.from_numpy(host_bytes))
+            self.buf[at:at + host_bytes.size].copy_(self._torch.from_numpy(host_bytes))
             self._torch.cuda.synchronize()
         else:
-            self.buf[:host_bytes.size] = host_bytes
+            self.buf[at:at + host_bytes.size] = host_bytes
 
-    def read(self, n):
+    def read(self, n, at=0):
         if self.kind == "VRAM":
             self._torch.cuda.synchronize()
-            return self.buf[:n].cpu().numpy()
-        return self.buf[:n].copy()
+            return self.buf[at:at + n].cpu().numpy()
+        return self.buf[at:at + n].copy()
 
 
 class Stat:
@@ -121,12 +126,75 @@ def _us():
 
 
 def run_point(agent, a, local, remote, block, batch, out):
-    """One (block size, batch size) point: warm-up, timed loop, optional byte check."""
-    rng = np.random.default_rng(a.seed + block + batch)
+    """One (block size, batch size) point: warm-up, timed loop, optional byte check.  With
+    --num_threads N the point runs in N threads at once, each over its own N-th of the two
+    buffers with its own requests and num_iter / N iterations, as the reference's worker does
+    (nixl_worker.cpp:1847-1879, 2004); the bandwidth is all threads' bytes over the wall time."""
+    if a.num_threads > 1:
+        return run_point_threads(agent, a, local, remote, block, batch, out)
+    return run_point_one(agent, a, local, remote, block, batch, out)
+
+
+def run_point_threads(agent, a, local, remote, block, batch, out):
+    import copy
+    import io
+    import threading
+    n = a.num_threads
+    share = a.max_block_size * a.max_batch_size
+    per = copy.copy(a)
+    per.num_threads, per.num_iter, per.warmup_iter = 1, a.num_iter // n, max(a.warmup_iter // n, 0)
+    results, errors = [None] * n, []
+    gate = threading.Barrier(n + 1)
+
+    def work(tid):
+        try:
+            results[tid] = run_point_one(agent, per, local, remote, block, batch, io.StringIO(), base=tid * share,
+                                         seed_salt=tid, gate=gate)
+        except BaseException as e:  # noqa: BLE001 - reported by the caller
+            errors.append(e)
+            try:
+                gate.abort()
+            except threading.BrokenBarrierError:
+                pass
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(n)]
+    for t in threads:
+        t.start()
+    try:
+        gate.wait()  # everybody has warmed up: the timed loops start together
+        t0 = _us()
+        gate.wait()  # ... and have all ended
+        total_us = _us() - t0
+    except threading.BrokenBarrierError:
+        total_us = 0.0
+    for t in threads:
+        t.join()
+    if errors:
+        raise errors[0]
+    moved = sum(r["moved_bytes"] for r in results)
+    bw = moved / 1e9 / (total_us / 1e6)
+    iters = sum(r["iterations"] for r in results)
+    lat = total_us / max(iters * results[0]["per_slot"], 1)
+    ok = None if results[0]["consistent"] is None else all(r["consistent"] for r in results)
+
+    def mean(key):
+        return float(np.mean([r[key] for r in results]))
+
+    out.write(f"{block:<20d}{batch:<15d}{bw:<15.6f}{lat:<15.1f}{mean('avg_prep_us'):<15.1f}{mean('p99_prep_us'):<15.1f}"
+              f"{mean('avg_post_us'):<15.1f}{mean('p99_post_us'):<15.1f}{mean('avg_tx_us'):<15.1f}{mean('p99_tx_us'):<15.1f}"
+              + ("" if ok is None else ("consistency: ok" if ok else "consistency: FAILED")) + "\n")
+    out.flush()
+    return {"block": block, "batch": batch, "gbps": bw, "avg_lat_us": lat, "avg_prep_us": mean("avg_prep_us"),
+            "avg_post_us": mean("avg_post_us"), "avg_tx_us": mean("avg_tx_us"), "consistent": ok, "threads": n}
+
+
+def run_point_one(agent, a, local, remote, block, batch, out, base=0, seed_salt=0, gate=None):
+    """One thread's share of a point: its requests over [base, base + block * batch) of each buffer."""
+    rng = np.random.default_rng(a.seed + block + batch + 7919 * seed_salt)
     slots_per_buf = batch
-    l_off = np.arange(slots_per_buf, dtype=np.uint64) * np.uint64(block)
+    l_off = np.uint64(base) + np.arange(slots_per_buf, dtype=np.uint64) * np.uint64(block)
     r_slots = rng.permutation(slots_per_buf) if a.randomize_location_mode == "blockaligned" else np.arange(slots_per_buf)
-    r_off = r_slots.astype(np.uint64) * np.uint64(block)
+    r_off = np.uint64(base) + r_slots.astype(np.uint64) * np.uint64(block)
     depth = min(a.pipeline_depth, a.num_iter)
     if batch % depth:
         raise SystemExit(f"nixlbench: descriptor count ({batch}) is not divisible by pipeline depth ({depth})")
@@ -227,17 +295,22 @@ def run_point(agent, a, local, remote, block, batch, out):
         s_off, d_off = (l_off, r_off) if a.op_type == "WRITE" else (r_off, l_off)
         image = np.zeros(nbytes, np.uint8)
         for i in range(batch):  # block i of the list sits at its own offset in each buffer
-            image[int(s_off[i]):int(s_off[i]) + block] = pattern[i * block:(i + 1) * block]
-        src.fill(image)
-        dst.fill(np.zeros(nbytes, np.uint8))
+            at = int(s_off[i]) - base
+            image[at:at + block] = pattern[i * block:(i + 1) * block]
+        src.fill(image, base)
+        dst.fill(np.zeros(nbytes, np.uint8), base)
     if n_warm:
         loop(max(n_warm, depth), False)
+    if gate is not None:
+        gate.wait()
     t0 = _us()
     loop(n_iter, True)
     total_us = _us() - t0
+    if gate is not None:
+        gate.wait()
     if a.check_consistency:
-        got = dst.read(block * batch)
-        ok = all(np.array_equal(got[int(d_off[i]):int(d_off[i]) + block], pattern[i * block:(i + 1) * block])
+        got = dst.read(block * batch, base)
+        ok = all(np.array_equal(got[int(d_off[i]) - base:int(d_off[i]) - base + block], pattern[i * block:(i + 1) * block])
                  for i in range(batch))
     for sl in slots:
         recycle(sl)
@@ -250,8 +323,9 @@ def run_point(agent, a, local, remote, block, batch, out):
               f"{post.avg():<15.1f}{post.p99():<15.1f}{tx.avg():<15.1f}{tx.p99():<15.1f}"
               + ("" if ok is None else ("consistency: ok" if ok else "consistency: FAILED")) + "\n")
     out.flush()
-    return {"block": block, "batch": batch, "gbps": bw, "avg_lat_us": lat, "avg_prep_us": prep.avg(),
-            "avg_post_us": post.avg(), "avg_tx_us": tx.avg(), "consistent": ok}
+    return {"block": block, "batch": batch, "gbps": bw, "avg_lat_us": lat, "avg_prep_us": prep.avg(), "p99_prep_us": prep.p99(),
+            "avg_post_us": post.avg(), "p99_post_us": post.p99(), "avg_tx_us": tx.avg(), "p99_tx_us": tx.p99(),
+            "consistent": ok, "moved_bytes": moved, "iterations": n_iter, "per_slot": per_slot}
 
 
 def main(argv=None, out=sys.stdout):
@@ -264,13 +338,14 @@ def main(argv=None, out=sys.stdout):
     agent = nixl_agent("initiator", nixl_agent_config(backends=()), plugin_dirs=[a.plugin_dir] if a.plugin_dir else ())
     params = dict(kv.split("=", 1) for kv in a.backend_params.split(",") if kv)
     agent.create_backend(a.backend, params)
-    half = a.max_block_size * a.max_batch_size
+    half = a.max_block_size * a.max_batch_size * a.num_threads
     pinned = a.backend == "HIP"
     local = Segment(a.initiator_seg_type, half, a.device_id, pinned)
     remote = Segment(a.target_seg_type, half, a.device_id, pinned)
     regs = [agent.register_memory(np.array([[s.addr, s.nbytes, s.dev]], dtype=np.uint64), s.kind) for s in (local, remote)]
     out.write(f"nixlbench (single instance): backend {a.backend}, {a.initiator_seg_type} -> {a.target_seg_type}, "
-              f"{a.op_type}, {'prepared' if a.prepared_xfer else 'create'} transfers, pipeline depth {a.pipeline_depth}\n")
+              f"{a.op_type}, {'prepared' if a.prepared_xfer else 'create'} transfers, pipeline depth {a.pipeline_depth}, "
+              f"{a.num_threads} thread{'s' if a.num_threads > 1 else ''}\n")
     out.write(f"{'Block Size (B)':<20}{'Batch Size':<15}{'B/W (GB/Sec)':<15}{'Avg Lat. (us)':<15}{'Avg Prep (us)':<15}"
               f"{'P99 Prep (us)':<15}{'Avg Post (us)':<15}{'P99 Post (us)':<15}{'Avg Tx (us)':<15}{'P99 Tx (us)':<15}\n")
     out.write("-" * 155 + "\n")

@@ -51,3 +51,23 @@ def test_phase_timers_are_read_from_the_debug_lines():
     assert phases == {"agent_expand_index_pairs": [128.5, 130.0], "plugin_block_pass": [124.525, 0.0],
                       "plugin_plan_from_records": [8.03, 0.0], "plugin_rest": [0.611, 2500.5]}
     assert paths == ["blocks", "general"]
+
+
+def test_counter_file_is_read_for_several_kernels_at_once(tmp_path):
+    """The expert-parallel traffic figures: medians per kernel tag from one counter file, a tag
+    without samples left out, the yardstick apart."""
+    sys.path.insert(0, ROOT)
+    import bench
+    rows = [("void (anonymous namespace)::ll_bits_kernel<false, 1>(a)", "A", 3.0),
+            ("void (anonymous namespace)::ll_bits_kernel<true, 4>(a)", "A", 100.0),
+            ("void (anonymous namespace)::ll_dispatch_kernel<true>(a)", "A", 10.0),
+            ("void (anonymous namespace)::ll_dispatch_kernel<true>(a)", "A", 30.0),
+            ("void (anonymous namespace)::ll_dispatch_kernel<true>(a)", "A", 20.0),
+            ("void at::native::vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<int>, a>(b)", "A", 8.0)]
+    path = tmp_path / "t_counter_collection.csv"
+    with open(path, "w") as f:
+        f.write('"Dispatch_Id","Kernel_Name","Counter_Name","Counter_Value"\n')
+        for i, (k, c, v) in enumerate(rows):
+            f.write(f'{i},"{k}","{c}",{v}\n')
+    medians, yard = bench.counter_medians(str(path), ["A"], ["ll_bits_kernel<false", "ll_dispatch_kernel<true>", "ll_scales_kernel"])
+    assert medians == {"ll_bits_kernel<false": {"A": 3.0}, "ll_dispatch_kernel<true>": {"A": 20.0}} and yard == {"A": 8.0}

@@ -31,6 +31,19 @@ def test_sweep_on_cpu_backend(oracle_plugin_dir, extra):
     assert len([l for l in lines if l.endswith("consistency: ok")]) == 9
 
 
+def test_threads_share_a_point_on_cpu_backend(oracle_plugin_dir):
+    """--num_threads: each thread drives its own requests over its own part of the buffers
+    (benchmark/nixlbench/src/worker/nixl/nixl_worker.cpp:1847-1879); every thread's bytes are
+    checked, the report has one line a point."""
+    rc, results, text = _run(["--backend", "MEMCPY", "--plugin_dir", oracle_plugin_dir, "--initiator_seg_type", "DRAM",
+                              "--target_seg_type", "DRAM", "--num_threads", "3", "--pipeline_depth", "2"] + COMMON)
+    assert rc == 0, text
+    assert len(results) == 9 and all(r["consistent"] is True and r["threads"] == 3 and r["gbps"] > 0 for r in results)
+    assert "3 threads" in text.splitlines()[0]
+    with pytest.raises(SystemExit):
+        nixlbench.parse(["--num_threads", "5", "--num_iter", "12"])
+
+
 def test_bad_flags_are_rejected():
     with pytest.raises(SystemExit):
         nixlbench.parse(["--start_block_size", "8192", "--max_block_size", "4096"])
@@ -44,6 +57,14 @@ def test_sweep_on_hip_backend(cuda, extra):
     rc, results, text = _run(["--backend", "HIP"] + COMMON + extra)
     assert rc == 0, text
     assert len(results) == 9 and all(r["consistent"] is True for r in results)
+
+
+@pytest.mark.gpu
+def test_threads_on_hip_backend(cuda):
+    rc, results, text = _run(["--backend", "HIP", "--backend_params", "num_streams=2", "--num_threads", "2", "--prepared_xfer"]
+                             + COMMON)
+    assert rc == 0, text
+    assert len(results) == 9 and all(r["consistent"] is True and r["threads"] == 2 for r in results)
 
 
 @pytest.mark.gpu
