@@ -262,7 +262,7 @@ def _triples(addrs, blk):
     return np.stack([addrs, np.full(n, blk, np.uint64), np.zeros(n, np.uint64)], 1)
 
 
-def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, descriptor_path=False):
+def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, descriptor_path=False, pad_blocks=0):
     """Gather + scatter of config 2's shape with `blk`-byte descriptors.  The pools and the
     staging buffer are prepared ONCE as descriptor lists (prep_xfer_dlist); every request is
     made from index vectors into those lists (make_prepped_xfer), the call pattern of the
@@ -277,10 +277,13 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, 
     lk = layers * kv.sub_blocks_per_layer
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    src_pool = torch.empty((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+    # pad_blocks > 0: every (layer, K|V) slab of the two pools is that many blocks longer than the
+    # blocks it is used for, so that the slabs do not lie a power of two apart
+    slab_blocks = pool_blocks + pad_blocks
+    src_pool = torch.empty((lk, slab_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
     for i in range(lk):
-        src_pool[i] = torch.randn((pool_blocks, blk // 2), generator=gen, device=dev).to(torch.bfloat16)
-    dst_pool = torch.zeros((lk, pool_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
+        src_pool[i] = torch.randn((slab_blocks, blk // 2), generator=gen, device=dev).to(torch.bfloat16)
+    dst_pool = torch.zeros((lk, slab_blocks, blk // 2), dtype=torch.bfloat16, device=dev)
     staging = torch.zeros((n_sel * lk, blk // 2), dtype=torch.bfloat16, device=dev)
 
     # Launches go to a stream of ours so that HIP events recorded on that same stream
@@ -291,7 +294,8 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, 
     agent.register_memory([src_pool, dst_pool, staging])
 
     n_desc, n_pool = n_sel * lk, lk * pool_blocks
-    pool_offsets = np.arange(n_pool, dtype=np.uint64) * np.uint64(blk)
+    pool_offsets = ((np.arange(lk, dtype=np.uint64)[:, None] * np.uint64(slab_blocks)
+                     + np.arange(pool_blocks, dtype=np.uint64)[None, :]) * np.uint64(blk)).reshape(-1)
     stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
     t0 = time.perf_counter()
     h_src = agent.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM")
@@ -629,6 +633,73 @@ def run_concurrent_requests(args, blk, counts=(1, 2, 4), steps=10, warmup=3):
     del src_pool, dst_pool, stagings
     torch.cuda.empty_cache()
     return out
+
+
+def run_counter_sequence(args, blk, repeats=6):
+    """A fixed sequence of launches for hardware-counter runs (rocprofv3 --pmc ... -- python3
+    bench.py --counter-sequence), so that counters can be told apart per access pattern although
+    the kernel is the same: copy_uniform_kernel `repeats` times each as (1) gather and (2)
+    scatter of config 2 listed layer by layer, (3) gather and (4) scatter listed block by block,
+    (5) one contiguous descriptor of the same payload; then the small-descriptor stress
+    (copy_piece_kernel) and the low-latency dispatch and combine, whose kernels have names of
+    their own.  Prints the order as one JSON line; times nothing."""
+    import torch
+    from nixl_amd import nixl_agent, nixl_agent_config
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    kv = _kv_layout()
+    pool_blocks, n_sel = args.pool_blocks, args.blocks
+    lk = kv.layers * kv.sub_blocks_per_layer
+    n_desc, n_pool = n_sel * lk, lk * pool_blocks
+    src_pool = torch.randint(0, 255, (lk, pool_blocks, blk), dtype=torch.uint8, device=dev)
+    dst_pool = torch.zeros((lk, pool_blocks, blk), dtype=torch.uint8, device=dev)
+    staging = torch.zeros((n_desc, blk), dtype=torch.uint8, device=dev)
+    agent = nixl_agent("seq", nixl_agent_config(backends=()))
+    agent.create_backend("HIP", dict(kv.split("=", 1) for kv in args.backend_param))
+    agent.register_memory([src_pool, dst_pool, staging])
+    pool_offsets = np.arange(n_pool, dtype=np.uint64) * np.uint64(blk)
+    stg_addrs = np.uint64(staging.data_ptr()) + np.arange(n_desc, dtype=np.uint64) * np.uint64(blk)
+    h_src = agent.prep_xfer_dlist("", _triples(np.uint64(src_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+    h_dst = agent.prep_xfer_dlist("seq", _triples(np.uint64(dst_pool.data_ptr()) + pool_offsets, blk), "VRAM")
+    h_stg_r = agent.prep_xfer_dlist("seq", _triples(stg_addrs, blk), "VRAM")
+    h_stg_l = agent.prep_xfer_dlist("", _triples(stg_addrs, blk), "VRAM")
+    stg_idx = np.arange(n_desc, dtype=np.int32)
+    rng = np.random.default_rng(99)
+    sel = rng.choice(pool_blocks, n_sel, replace=False)
+    dst_ids = rng.permutation(pool_blocks)[:n_sel]
+
+    def run(req):
+        state = agent.transfer(req)
+        while state == "PROC":
+            state = agent.check_xfer_state(req)
+        if state != "DONE":
+            raise RuntimeError(f"transfer ended in state {state}")
+
+    order = []
+    for listing in ("layer", "block"):
+        gather = agent.make_prepped_xfer("WRITE", h_src, _kv_indices(lk, pool_blocks, sel, listing), h_stg_r, stg_idx)
+        scatter = agent.make_prepped_xfer("WRITE", h_stg_l, stg_idx, h_dst, _kv_indices(lk, pool_blocks, dst_ids, listing))
+        for name, req in ((f"gather, listed {listing} by {listing}", gather), (f"scatter, listed {listing} by {listing}", scatter)):
+            for _ in range(repeats):
+                run(req)
+                order.append(name)
+        gather.release()
+        scatter.release()
+    one = np.array([[src_pool.data_ptr(), n_desc * blk, 0]], dtype=np.uint64), np.array([[dst_pool.data_ptr(), n_desc * blk, 0]], dtype=np.uint64)
+    req = agent.initialize_xfer("WRITE", agent.get_xfer_descs(one[0], "VRAM"), agent.get_xfer_descs(one[1], "VRAM"), "seq")
+    for _ in range(repeats):
+        run(req)
+        order.append("one contiguous descriptor of the same payload")
+    req.release()
+    for h in (h_src, h_dst, h_stg_r, h_stg_l):
+        h.release()
+    agent.close()
+    del src_pool, dst_pool, staging
+    torch.cuda.empty_cache()
+    run_small_descriptors(steps=repeats, warmup=1)
+    from nixl_amd import ep_bench
+    ep_bench.run_traffic_child(repeats=repeats, normal_mode=False)
+    print(json.dumps({"copy_uniform_kernel_launches": order, "descriptor_bytes": blk, "repeats": repeats}))
 
 
 def run_prep_breakdown_child(args, blk):
@@ -1066,6 +1137,8 @@ def main():
                          "known-size yardstick for hardware counter runs")
     ap.add_argument("--prep-breakdown-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--ep-traffic-child", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--counter-sequence", action="store_true",
+                    help="run a fixed sequence of launches for hardware-counter runs and print its order; nothing is timed")
     ap.add_argument("--no-live-traffic", action="store_true",
                     help="do not run the headline leg under rocprofv3 --pmc first; roofline.traffic then comes from "
                          "the counter runs summarised under profiles/")
@@ -1080,6 +1153,9 @@ def main():
     blk = args.block_bytes or 16384  # the metric is quoted "@16KB blocks"
     if args.prep_breakdown_child:
         run_prep_breakdown_child(args, blk)
+        return
+    if args.counter_sequence:
+        run_counter_sequence(args, blk)
         return
     if args.ep_traffic_child:
         from nixl_amd import ep_bench
@@ -1125,6 +1201,12 @@ def main():
                     "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
                     "make_request_pair_ms": r["kv"]["make_request_pair_ms"],
                     "value_including_prepare": r["kv"]["value_including_prepare"]}
+            r = run_kv(args, 16384, "block", max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2, pad_blocks=1)
+            others["16KiB_block_order_slabs_one_block_longer"] = {
+                "value_GBps": round(r["value"], 1), "roofline": r["roofline"],
+                "note": "the same requests over pools whose (layer, K|V) slabs are 8193 blocks long instead of 8192, so that "
+                        "the 64 sub-blocks of a block id no longer lie a power of two (128 MiB) apart: what the layout, not "
+                        "the engine, decides"}
             r = run_kv(args, blk, args.order, max(args.steps // 2, 1), max(args.warmup // 2, 1), fresh_requests=2, sorted_ids=True)
             others[f"{blk // 1024}KiB_{args.order}_order_source_blocks_ascending"] = {
                 "value_GBps": round(r["value"], 1), "roofline": r["roofline"],

@@ -141,8 +141,13 @@ copy_uniform_kernel(const UniformRec *recs, uint32_t first_chunk, uint32_t n_chu
     const uint32_t c = uniform(first_chunk + wg * WAVES + wave); // n_chunks, n_wgs: of this launch
     const uint32_t r = c / chunks_per_rec;
     const uint64_t off = static_cast<uint64_t>(c % chunks_per_rec) * (kWaveSize * UPL * 16u) + lane * 16u;
-    const uint64_t s = uniform64(recs[r].src) + off;
-    const uint64_t d = uniform64(recs[r].dst) + off;
+    // The record is the same for every lane and does not change while the kernel runs: read
+    // through the constant address space it comes with ONE scalar load (left as an ordinary
+    // global access the compiler makes it a 16-byte vector load by all 64 lanes, followed by
+    // four lane-0 read-outs).
+    const auto *words = reinterpret_cast<const __attribute__((address_space(4))) uint64_t *>(reinterpret_cast<uintptr_t>(recs + r));
+    const uint64_t s = words[0] + off; // UniformRec::src
+    const uint64_t d = words[1] + off; // UniformRec::dst
     v4u v[UPL];
 #pragma unroll
     for (int k = 0; k < UPL; ++k)
