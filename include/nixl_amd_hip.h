@@ -200,7 +200,9 @@ nixl_amd_copy_plan_launch(nixl_amd_copy_plan_t *plan, void *stream);
  * is made to be polled), another negative status if a launch failed.  With `wait` non-zero the
  * call blocks until the answer is not BUSY.  This is what nixlBackendEngine::checkXfer
  * (src/api/cpp/backend/backend_engine.h:153) asks of a posted request.  Launches recorded
- * into a HIP graph are not tracked. */
+ * into a HIP graph are not tracked.  The answer follows the stream of the LAST launch: a
+ * caller that launches one plan on several streams orders those streams itself.  Launch,
+ * status and destroy of one plan are not to be called from several threads at once. */
 int
 nixl_amd_copy_plan_status(nixl_amd_copy_plan_t *plan, int wait);
 
