@@ -641,8 +641,8 @@ def run_counter_sequence(args, blk, repeats=6):
     the kernel is the same: copy_uniform_kernel `repeats` times each as (1) gather and (2)
     scatter of config 2 listed layer by layer, (3) gather and (4) scatter listed block by block,
     (5) one contiguous descriptor of the same payload; then the small-descriptor stress
-    (copy_piece_kernel) and the low-latency dispatch and combine, whose kernels have names of
-    their own.  Prints the order as one JSON line; times nothing."""
+    (copy_piece_kernel) and the expert-parallel dispatch and combine of both modes, whose
+    kernels have names of their own.  Prints the order as one JSON line; times nothing."""
     import torch
     from nixl_amd import nixl_agent, nixl_agent_config
     dev = torch.device("cuda:0")
@@ -698,7 +698,7 @@ def run_counter_sequence(args, blk, repeats=6):
     torch.cuda.empty_cache()
     run_small_descriptors(steps=repeats, warmup=1)
     from nixl_amd import ep_bench
-    ep_bench.run_traffic_child(repeats=repeats, normal_mode=False)
+    ep_bench.run_traffic_child(repeats=repeats, normal_mode=True)
     print(json.dumps({"copy_uniform_kernel_launches": order, "descriptor_bytes": blk, "repeats": repeats}))
 
 
