@@ -740,23 +740,61 @@ firstIndexOutside(const std::vector<int> &indices, size_t flat) {
     return indices.size();
 }
 
-// Walks a prepared list by flat index; consecutive look-ups usually stay inside one run.
+// Walks a prepared list by flat index.  Consecutive look-ups usually stay inside one run or
+// step into the next one; any other index is looked for from a proportional first guess (run
+// number = index x runs / blocks) by doubling steps and a bisection of the stretch they
+// bracket.  A list that hardly compresses (runs of one block with a run of two here and there)
+// made the list's own find() bisect 260 000 runs for every index: its first guess divides by
+// the rounded-up mean run length.
 class runCursor {
 public:
     explicit runCursor(const nixl_stride_dlist_t &runs)
-        : runs_(runs),
-          // ceiling division keeps find()'s first probe inside the run array
-          guess_((runs.flatSize() + static_cast<size_t>(runs.descCount()) - 1) / static_cast<size_t>(runs.descCount())) {}
+        : first_(&runs[0]),
+          n_runs_(static_cast<size_t>(runs.descCount())),
+          blocks_(runs.flatSize()) {}
 
     const nixlStrideDesc &
     at(size_t index) {
-        if (!run_ || index - run_->start_idx >= run_->count) run_ = &runs_.find(index, guess_);
-        return *run_;
+        if (run_) {
+            if (index - run_->start_idx < run_->count) return *run_;
+            const nixlStrideDesc *next = run_ + 1;
+            if (next < first_ + n_runs_ && index - next->start_idx < next->count) return *(run_ = next);
+        }
+        return *(run_ = locate(index));
     }
 
 private:
-    const nixl_stride_dlist_t &runs_;
-    const size_t guess_;
+    // `index` is below blocks_ (the caller has checked the index vectors)
+    const nixlStrideDesc *
+    locate(size_t index) const {
+        size_t at = static_cast<size_t>(static_cast<unsigned __int128>(index) * n_runs_ / blocks_);
+        if (index - first_[at].start_idx < first_[at].count) return first_ + at;
+        size_t lo, hi; // the run lies in [lo, hi]
+        if (first_[at].start_idx > index) {
+            size_t step = 1;
+            hi = at - 1;
+            while (step <= hi && first_[hi + 1 - step].start_idx > index)
+                step <<= 1;
+            lo = step <= hi ? hi + 1 - step : 0;
+        } else {
+            size_t step = 1;
+            lo = at + 1;
+            while (lo + step < n_runs_ && first_[lo + step].start_idx <= index)
+                step <<= 1;
+            hi = std::min(lo + step, n_runs_) - 1;
+        }
+        while (lo < hi) { // last run whose start_idx is at most index
+            const size_t mid = (lo + hi + 1) >> 1;
+            if (first_[mid].start_idx <= index)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        return first_ + lo;
+    }
+
+    const nixlStrideDesc *const first_;
+    const size_t n_runs_, blocks_;
     const nixlStrideDesc *run_ = nullptr;
 };
 

@@ -148,6 +148,50 @@ def test_agent_runs_and_merge_match_oracle(cpu_agent):
         hr.release()
 
 
+def test_agent_index_lookup_in_long_irregular_lists(cpu_agent):
+    """Prepared lists of a few thousand descriptors that hardly compress (runs of one block with
+    longer runs strewn in, on one side none at all): index vectors that ascend, descend, jump at
+    random and repeat must expand to what the oracle's expansion gives, merged and unmerged.
+    (The run look-up steps to the next run, guesses proportionally and brackets by doubling.)"""
+    rng = np.random.default_rng(11)
+    a = cpu_agent
+    ln = 64
+    bufs = [np.zeros(1 << 20, np.uint8) for _ in range(2)]
+    for b in bufs:
+        a.register_memory(_np_descs(b, [0], [b.nbytes]), "DRAM")
+    regions = [(b.ctypes.data, b.nbytes, 0) for b in bufs]
+
+    def side(buf, n, run_lengths):
+        out, slot = [], 0
+        while len(out) < n:
+            k = int(rng.choice(run_lengths))
+            out += [(buf.ctypes.data + (slot + j) * ln, ln, 0) for j in range(k)]
+            slot += k + int(rng.integers(1, 4))  # a gap ends the run
+        return out[:n]
+
+    n = 3000
+    for run_lengths in ([1, 1, 1, 1, 1, 1, 2], [1, 1, 1, 7, 30], [1]):
+        ld, rd = side(bufs[0], n, run_lengths), side(bufs[1], n, [1, 2, 3])
+        hl = a.prep_xfer_dlist("", np.array(ld, dtype=np.uint64), "DRAM")
+        hr = a.prep_xfer_dlist("agent", np.array(rd, dtype=np.uint64), "DRAM")
+        lruns, rruns = ko.stride_runs(ld, regions), ko.stride_runs(rd, regions)
+        assert hl.run_count() == len(lruns) and hr.run_count() == len(rruns)
+        walks = [(np.arange(n), np.arange(n)), (np.arange(n)[::-1].copy(), np.arange(n)),
+                 (rng.integers(0, n, 2000), rng.integers(0, n, 2000)),
+                 (np.repeat(rng.integers(0, n, 40), 5), np.sort(rng.integers(0, n, 200))),
+                 (np.array([0, n - 1, 0, n - 1, n // 2]), np.array([n - 1, 0, n - 1, 0, 1]))]
+        for li, ri in walks:
+            for skip in (False, True):
+                req = a.make_prepped_xfer("WRITE", hl, li, hr, ri, skip_desc_merge=skip)
+                want = ko.expand_and_merge(lruns, rruns, li, ri, skip_merge=skip)
+                count, nbytes = req.desc_count()
+                assert count == len(want) and nbytes == sum(w[2] for w in want)
+                assert [req.get_desc(i) for i in range(count)] == want
+                req.release()
+        hl.release()
+        hr.release()
+
+
 def test_agent_reference_example_merge_counts(cpu_agent):
     # Same known answers as test_oracle_merge_counts_match_reference_example, now for the
     # C++ agent at the reference's full size (32 x 65536 descriptors of 8 bytes).
