@@ -902,6 +902,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
     vsrc.reserve(n);
     vdst.reserve(n);
     vprefix.reserve(n + 1);
+    pieces.reserve(n);
     uint64_t units = 0, payload = 0, n_generic_descs = 0, n_piece_descs = 0;
     for (size_t i = 0; i < n; ++i) {
         const nixl_amd_copy_desc_t &d = descs[i];
