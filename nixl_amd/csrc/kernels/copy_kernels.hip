@@ -413,6 +413,28 @@ index_records_runs_kernel(UniformRec *recs, const int32_t *src_index, const int3
                              run_address(first[1], base[1], stride[1], n_dst, static_cast<uint64_t>(dst_index[i]))};
 }
 
+// Records of a plan whose runs of uniform chunks differ in length: run r covers chunks
+// first_chunk[r] .. first_chunk[r + 1] - 1 and chunk c of it lies c - first_chunk[r] chunks
+// behind the run's start on both sides.  A thread per chunk finds its run by bisection (the
+// table stays in the L2), so that one long run among short ones costs no more than any other;
+// 16 bytes per run cross the bus instead of 16 per chunk.
+__global__ void __launch_bounds__(256)
+expand_runs_kernel(UniformRec *recs, const UniformRec *runs, const uint32_t *first_chunk, uint32_t n_runs, uint32_t n_chunks,
+                   uint32_t chunk_bytes) {
+    for (uint64_t c64 = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; c64 < n_chunks;
+         c64 += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
+        const uint32_t c = static_cast<uint32_t>(c64);
+        uint32_t lo = 0, hi = n_runs; // first_chunk[lo] <= c < first_chunk[hi]
+        while (hi - lo > 1) {
+            const uint32_t mid = lo + (hi - lo) / 2;
+            if (first_chunk[mid] <= c) lo = mid;
+            else hi = mid;
+        }
+        const uint64_t off = static_cast<uint64_t>(c - first_chunk[lo]) * chunk_bytes;
+        recs[c] = UniformRec{runs[lo].src + off, runs[lo].dst + off};
+    }
+}
+
 // Largest grid of one launch: HIP refuses grids of 2^32 or more threads, i.e. 2^22 workgroups of
 // 16 waves; a plan with more work than that goes out as several launches.
 constexpr uint32_t kMaxGrid = 1u << 21;
@@ -1003,6 +1025,7 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         }
     }
     std::vector<UniformRec> uni;
+    std::vector<uint32_t> first_chunk; // runs of different lengths: run r starts at uniform chunk first_chunk[r]
     uint32_t chunks_per_rec = 1;
     if (all_whole) {
         chunks_per_rec = common_run;
@@ -1014,26 +1037,39 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         uni.reserve(runs.size());
         for (const Run &r : runs)
             uni.push_back(UniformRec{r.src, r.dst});
-    } else {
-        uni.reserve(n_uniform_chunks);
-        const uint64_t chunk_bytes = chunk_units * 16u;
-        for (const Run &r : runs)
-            for (uint32_t k = 0; k < r.chunks; ++k)
-                uni.push_back(UniformRec{r.src + k * chunk_bytes, r.dst + k * chunk_bytes});
+    } else if (!runs.empty()) {
+        // a record per chunk, written on the device from a record per run
+        uni.reserve(runs.size());
+        first_chunk.reserve(runs.size() + 1);
+        uint32_t at = 0;
+        for (const Run &r : runs) {
+            uni.push_back(UniformRec{r.src, r.dst});
+            first_chunk.push_back(at);
+            at += r.chunks;
+        }
+        first_chunk.push_back(at);
     }
+    const bool expand = !first_chunk.empty();
+    const size_t n_uniform_recs = expand ? n_uniform_chunks : uni.size();
 
     // ---- one device arena for all plan arrays --------------------------------------
     auto align256 = [](size_t x) { return (x + 255) & ~size_t(255); };
     const bool need_desc_arrays = !mixed.empty();
+    // The arena starts with the records the copy kernel reads.  When they are expanded on the
+    // device, that stretch is not uploaded: the upload starts behind it, and the records per run
+    // and their first chunks travel at the arena's end.
     const size_t off_uni = 0;
-    const size_t off_src = off_uni + align256(uni.size() * sizeof(UniformRec));
+    const size_t off_src = off_uni + align256(n_uniform_recs * sizeof(UniformRec));
     const size_t off_dst = off_src + (need_desc_arrays ? align256(nv * 8) : 0);
     const size_t off_prefix = off_dst + (need_desc_arrays ? align256(nv * 8) : 0);
     const size_t off_span = off_prefix + (need_desc_arrays ? align256((nv + 1) * 8) : 0);
     const size_t off_mixed = off_span + (need_desc_arrays ? align256(span.size() * sizeof(uint2)) : 0);
     const size_t off_pieces = off_mixed + align256(mixed.size() * sizeof(uint32_t));
     const size_t off_items = off_pieces + align256(pieces.size() * sizeof(PieceRec));
-    const size_t total = off_items + align256(items.size() * sizeof(GenericItem));
+    const size_t off_runs = off_items + align256(items.size() * sizeof(GenericItem));
+    const size_t off_first = off_runs + (expand ? align256(uni.size() * sizeof(UniformRec)) : 0);
+    const size_t total = off_first + (expand ? align256(first_chunk.size() * sizeof(uint32_t)) : 0);
+    const size_t upload_from = expand ? off_src : 0;
 
     auto *plan = new nixl_amd_copy_plan();
     plan->device = device;
@@ -1066,22 +1102,27 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         void *staging = nullptr;
         size_t staging_cap = 0;
         reap_uploads(device);
-        hipError_t e = upload_cache().get(device, total, &staging, &staging_cap);
+        hipError_t e = upload_cache().get(device, std::max<size_t>(total - upload_from, 256), &staging, &staging_cap);
         if (e != hipSuccess) {
             delete plan;
             return nixl_amd_fail(NIXL_AMD_ERR_HIP, std::string("hipHostMalloc(plan upload buffer): ") + hipGetErrorString(e));
         }
-        auto *host = static_cast<uint8_t *>(staging);
-        if (!uni.empty()) std::memcpy(host + off_uni, uni.data(), uni.size() * sizeof(UniformRec));
+        // the pinned buffer mirrors the arena from upload_from on
+        const auto host = [&](size_t arena_offset) { return static_cast<uint8_t *>(staging) + (arena_offset - upload_from); };
+        if (expand) {
+            std::memcpy(host(off_runs), uni.data(), uni.size() * sizeof(UniformRec));
+            std::memcpy(host(off_first), first_chunk.data(), first_chunk.size() * sizeof(uint32_t));
+        } else if (!uni.empty())
+            std::memcpy(host(off_uni), uni.data(), uni.size() * sizeof(UniformRec));
         if (need_desc_arrays) {
-            std::memcpy(host + off_src, vsrc.data(), nv * 8);
-            std::memcpy(host + off_dst, vdst.data(), nv * 8);
-            std::memcpy(host + off_prefix, vprefix.data(), (nv + 1) * 8);
-            std::memcpy(host + off_span, span.data(), span.size() * sizeof(uint2));
-            std::memcpy(host + off_mixed, mixed.data(), mixed.size() * sizeof(uint32_t));
+            std::memcpy(host(off_src), vsrc.data(), nv * 8);
+            std::memcpy(host(off_dst), vdst.data(), nv * 8);
+            std::memcpy(host(off_prefix), vprefix.data(), (nv + 1) * 8);
+            std::memcpy(host(off_span), span.data(), span.size() * sizeof(uint2));
+            std::memcpy(host(off_mixed), mixed.data(), mixed.size() * sizeof(uint32_t));
         }
-        if (!pieces.empty()) std::memcpy(host + off_pieces, pieces.data(), pieces.size() * sizeof(PieceRec));
-        if (!items.empty()) std::memcpy(host + off_items, items.data(), items.size() * sizeof(GenericItem));
+        if (!pieces.empty()) std::memcpy(host(off_pieces), pieces.data(), pieces.size() * sizeof(PieceRec));
+        if (!items.empty()) std::memcpy(host(off_items), items.data(), items.size() * sizeof(GenericItem));
         e = arena_cache().get(device, total, &plan->arena, &plan->arena_cap);
         if (e != hipSuccess) {
             upload_cache().put(device, staging, staging_cap);
@@ -1092,7 +1133,17 @@ nixl_amd_copy_plan_create(const nixl_amd_copy_desc_t *descs,
         // stream, and the pinned buffer is recycled once the copy has completed.
         hipStream_t up = nullptr;
         e = upload_stream(device, &up);
-        if (e == hipSuccess) e = hipMemcpyAsync(plan->arena, host, total, hipMemcpyHostToDevice, up);
+        auto *arena = static_cast<uint8_t *>(plan->arena);
+        if (e == hipSuccess && total > upload_from)
+            e = hipMemcpyAsync(arena + upload_from, staging, total - upload_from, hipMemcpyHostToDevice, up);
+        if (e == hipSuccess && expand) {
+            const uint32_t wgs = static_cast<uint32_t>(std::min<uint64_t>((static_cast<uint64_t>(n_uniform_chunks) + 255) / 256, 1u << 20));
+            hipLaunchKernelGGL(expand_runs_kernel, dim3(wgs), dim3(256), 0, up, reinterpret_cast<UniformRec *>(arena + off_uni),
+                               reinterpret_cast<const UniformRec *>(arena + off_runs),
+                               reinterpret_cast<const uint32_t *>(arena + off_first), static_cast<uint32_t>(uni.size()),
+                               n_uniform_chunks, static_cast<uint32_t>(chunk_units * 16u));
+            e = hipGetLastError();
+        }
         if (e == hipSuccess) e = hipEventCreateWithFlags(&plan->uploaded, hipEventDisableTiming);
         if (e == hipSuccess) e = hipEventRecord(plan->uploaded, up);
         if (e != hipSuccess) {
