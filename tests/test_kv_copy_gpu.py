@@ -184,6 +184,26 @@ def test_random_mixture_of_every_descriptor_class(cuda, seed):
     assert info.generic_descs > 0 and info.piece_items > 0 and info.vec_descs > 0
 
 
+def test_runs_of_different_lengths_are_expanded_on_the_device(cuda):
+    """Line-aligned descriptors of at least 8 KiB whose lengths differ: the chunks inside each
+    descriptor share nothing, so every chunk has a record, and those records are written on the
+    device from one record per run.  One descriptor of 24 MiB among two thousand of 8 to 64 KiB
+    (whole chunks, and lengths that leave a tail for the next chunk), every byte against the
+    oracle; the plan holds a record per chunk."""
+    import torch
+    rng = np.random.default_rng(77)
+    lens = [int(x) * 1024 for x in rng.integers(8, 65, 1200)] + [int(x) * 16 for x in rng.integers(512, 4097, 800)]
+    lens.insert(700, 24 << 20)
+    half = int(sum(lens) + len(lens) * 256 + (1 << 20))
+    half = (half + 4095) // 4096 * 4096
+    so = _disjoint_layout(rng, lens, 128, half)
+    do = _disjoint_layout(rng, lens, 128, half) + half
+    info = _check_against_oracle(torch, cuda, 2 * half, so, do, lens, seed=5)
+    assert info.vec_descs == len(lens) and info.piece_items == 0 and info.generic_descs == 0
+    assert info.uniform_chunks > 24 * 1024 and info.mixed_chunks > 0
+    assert info.plan_device_bytes >= info.uniform_chunks * 16
+
+
 def test_zero_length_and_empty(cuda):
     import torch
     dev = torch.zeros(4096, dtype=torch.uint8, device=cuda)
