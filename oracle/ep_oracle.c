@@ -152,6 +152,10 @@ masked(const int32_t *mask, int R, int a, int b) {
  * The reference hands out slots and segment begins with atomicAdd, so any order inside a
  * segment and any order of segments is a valid result.  This restatement fixes the
  * canonical one: tokens ascending inside a segment, segments by source rank ascending.
+ * A token that names an expert more than once takes a slot per selection (:186-190), so the
+ * expert receives its row once per selection, next to each other in the canonical order.  More
+ * than M selections from one rank to one expert would run past the reference's receive area:
+ * refused here with -3.
  * A message travels from a to b only if neither mask[a][b] nor mask[b][a] is set
  * (send side :197,266; receive side :319-338 treats a masked or silent rank as zero tokens).
  */
@@ -176,6 +180,7 @@ oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t *nu
         return -2;
     }
     (void)threads;
+    int overflow = 0; /* a rank names one expert more often than its M slots there hold (only repeats can) */
 
     /* send phase */
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
@@ -196,6 +201,11 @@ oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t *nu
                 if (e < 0) continue;
                 const int d = e / El, le = e % El;
                 const int slot = next_slot[e]++;
+                if (slot >= M) { /* the reference would write past its receive area: refused here */
+                    __atomic_store_n(&overflow, 1, __ATOMIC_RELAXED);
+                    next_slot[e] = M;
+                    continue;
+                }
                 if (masked(mask, R, r, d)) continue;
                 memcpy(area + ((((size_t)d * El + le) * R + r) * M + slot) * msg_bytes, msg, msg_bytes);
             }
@@ -245,7 +255,7 @@ oracle_ll_dispatch(const uint16_t *x, const int32_t *topk_idx, const int32_t *nu
     }
     free(area);
     free(count_words);
-    return 0;
+    return overflow ? -3 : 0;
 }
 
 /*

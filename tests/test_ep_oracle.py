@@ -200,6 +200,51 @@ def test_ll_dispatch_brute_force_and_reference_invariants(use_fp8, round_scale, 
             assert np.all(o["src_info"][d, le, n:].view(np.uint8) == fill)
 
 
+def test_ll_dispatch_repeated_expert_takes_a_slot_per_selection():
+    """A token whose top-k names one expert more than once: the reference's send phase takes a
+    slot per (token, selection) with an atomicAdd (kernels/nixl_ep_ll.cu:186-190) and its
+    receive phase packs whatever the count word says (:319-338), so the expert receives the
+    token's row once per selection.  Enumerated here selection by selection, without the
+    oracle's slot arithmetic: counts, ranges, sources and rows must agree, in the oracle's
+    canonical order (tokens ascending, a token's selections together).  More selections from
+    one rank to one expert than its slots hold is refused."""
+    rng = np.random.default_rng(23)
+    R, T, H, K, E, M = 3, 10, 256, 4, 6, 20
+    x, topk, _ = _world(rng, R, T, H, K, E, drop=0.05)
+    for r, t, k_from, k_to in [(0, 1, 0, 2), (0, 1, 0, 3), (1, 4, 1, 0), (2, 9, 3, 2), (2, 0, 0, 1)]:
+        topk[r, t, k_to] = topk[r, t, k_from] if topk[r, t, k_from] >= 0 else 0
+    topk[1, 7, :] = 5  # every selection of one token goes to the same expert
+    xb = bf16_bits(x).reshape(R, T, H)
+    fill = 0x55
+    o = eo.ll_dispatch(xb, topk, E, M, False, fill=fill)
+    El = E // R
+    assert int(o["recv_count"].sum()) == int((topk >= 0).sum())
+    for d in range(R):
+        for le in range(El):
+            e = d * El + le
+            begin = 0
+            for r in range(R):
+                picks = [t for t in range(T) for k in range(K) if topk[r, t, k] == e]
+                lr = int(o["layout_range"][d, le, r])
+                assert (lr & 0xFFFFFFFF) == len(picks)
+                if picks:
+                    assert (lr >> 32) == begin
+                assert o["src_info"][d, le, begin:begin + len(picks)].tolist() == picks
+                for i, t in enumerate(picks):
+                    assert np.array_equal(o["recv_x"][d, le, begin + i], xb[r, t])
+                begin += len(picks)
+            assert o["recv_count"][d, le] == begin
+            assert np.all(o["recv_x"][d, le, begin:].view(np.uint8) == fill)
+    # the expert of rank 1, token 7 holds that token four times in a row
+    seg = int(o["layout_range"][5 // El, 5 % El, 1])
+    rows = o["src_info"][5 // El, 5 % El, (seg >> 32):(seg >> 32) + (seg & 0xFFFFFFFF)].tolist()
+    assert rows.count(7) == K
+    crowded = topk.copy()
+    crowded[0, :, :] = 2  # rank 0 sends T * K = 40 rows to expert 2, which holds M = 20 of its rows
+    with pytest.raises(ValueError):
+        eo.ll_dispatch(xb, crowded, E, M, False)
+
+
 def test_ll_dispatch_reference_test_pattern():
     # Data pattern of tests/elastic/elastic.py:131-134: every channel = rank - 128 except the
     # last 128 channels, which hold the token index; bf16 dispatch must deliver it verbatim
