@@ -30,8 +30,9 @@ extern "C" {
 
 /* Launch-shape knob of the low-latency kernels (no reference counterpart): the largest
  * workgroup, in lanes, of the dispatch and combine kernels; a multiple of 64 in [64, 1024],
- * or 0 to leave a value unchanged.  Until it is set, dispatch takes a workgroup per token and
- * combine one per row, or two halves for a row of more than 512 lanes.  Process-wide; may be called from any thread: a dispatch or
+ * 0 to leave a value unchanged, or -1 to return to the built-in choice: dispatch takes a
+ * workgroup per token, combine one per row, or two halves for a row of more than 512 lanes.
+ * Process-wide; may be called from any thread: a dispatch or
  * combine call that runs at the same time uses the old or the new value. */
 int
 nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes);

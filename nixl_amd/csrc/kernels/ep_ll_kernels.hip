@@ -841,11 +841,12 @@ extern "C" {
 
 int
 nixl_amd_ep_ll_set_tuning(int dispatch_lanes, int combine_lanes) {
-    auto ok = [](int v) { return v == 0 || (v >= 64 && v <= 1024 && v % 64 == 0); };
+    auto ok = [](int v) { return v == 0 || v == -1 || (v >= 64 && v <= 1024 && v % 64 == 0); };
     if (!ok(dispatch_lanes) || !ok(combine_lanes))
-        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_set_tuning: lanes must be 0 or a multiple of 64 in [64, 1024]");
-    if (dispatch_lanes) g_dispatch_lanes.store(dispatch_lanes, std::memory_order_relaxed);
-    if (combine_lanes) g_combine_lanes.store(combine_lanes, std::memory_order_relaxed);
+        return nixl_amd_fail(NIXL_AMD_ERR_INVALID, "ll_set_tuning: lanes must be 0, -1 or a multiple of 64 in [64, 1024]");
+    // -1: back to what the library starts with
+    if (dispatch_lanes) g_dispatch_lanes.store(dispatch_lanes == -1 ? 1024 : dispatch_lanes, std::memory_order_relaxed);
+    if (combine_lanes) g_combine_lanes.store(combine_lanes == -1 ? 0 : combine_lanes, std::memory_order_relaxed);
     return NIXL_AMD_OK;
 }
 

@@ -137,6 +137,13 @@ def test_ll_every_hidden_size_of_the_reference(cuda, hidden):
     torch.cuda.synchronize()
     want = eo.ll_combine(bits16(y).reshape(R, El, R * M, hidden), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(), E, M)
     assert np.array_equal(bits16(out).reshape(R, T, hidden), want)
+    # rows of more than 512 lanes are combined by two workgroups: the LogFMT codec's groups of
+    # 16 lanes must stay whole (agreement with the libm restatement as in test_ll_combine_logfmt)
+    out, _, _ = buf.combine(y, td, wd, handle, use_logfmt=True)
+    torch.cuda.synchronize()
+    want = eo.ll_combine(bits16(y).reshape(R, El, R * M, hidden), topk, w, handle[0].cpu().numpy(), handle[1].cpu().numpy(), E, M,
+                         use_fma=True, use_logfmt=True)
+    assert np.mean(bits16(out).reshape(R, T, hidden) == want) > 0.98
 
 
 def test_ll_dispatch_extreme_values(cuda):
@@ -1260,4 +1267,4 @@ def test_ll_narrow_workgroups_give_the_same_bytes(cuda):
                     else:
                         assert np.array_equal(bits16(out).reshape(R, T, H), ref)
     finally:
-        k.nixl_amd_ep_ll_set_tuning(1024, 1024)
+        assert k.nixl_amd_ep_ll_set_tuning(-1, -1) == 0  # back to the built-in choice
