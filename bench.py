@@ -42,8 +42,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 _KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc runs of this file, not this run)"
 MEASURED_TRAFFIC = {
     (1024, 8192, 16384): {"bytes": 2155883520, "source": _KV_PROFILE},
-    (1024, 8192, 32768): {"bytes": 4303367520, "source": _KV_PROFILE},
-    ("small", 262144): {"bytes": 938868352,
+    (1024, 8192, 32768): {"bytes": 4303367456, "source": _KV_PROFILE},
+    ("small", 262144): {"bytes": 938500160,
                         "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
                                   "this file, not this run)"},
 }
