@@ -520,8 +520,8 @@ namespace {
 
 // Plan arenas and the pinned buffers they are uploaded from are recycled: a request whose
 // descriptor list changes every time (paged KV) would otherwise pay a hipMalloc and a
-// pageable-memory copy per request.  Blocks are kept by power-of-two size class, a few per
-// class; what does not fit the cache is freed.
+// pageable-memory copy per request.  Blocks come in power-of-two sizes; the cache keeps the
+// most recently returned ones up to a count and a byte limit and frees the oldest beyond that.
 class BlockCache {
 public:
     explicit BlockCache(bool pinned) : pinned_(pinned) {}
@@ -547,20 +547,31 @@ public:
         return pinned_ ? hipHostMalloc(out, size, hipHostMallocDefault) : hipMalloc(out, size);
     }
 
+    // The block just given back is the likeliest to be asked for again (the next request of the
+    // same shape), so when the cache is full the oldest blocks make room for it.
     void
     put(int device, void *ptr, size_t size) {
+        std::vector<Block> evicted;
         {
             std::lock_guard<std::mutex> lock(mutex_);
-            if (held_ + size <= kMaxHeld && free_.size() < kMaxBlocks) {
+            if (size <= kMaxHeld) {
+                while (!free_.empty() && (held_ + size > kMaxHeld || free_.size() >= kMaxBlocks)) {
+                    evicted.push_back(free_.front());
+                    held_ -= free_.front().size;
+                    free_.erase(free_.begin());
+                }
                 free_.push_back(Block{ptr, size, device});
                 held_ += size;
-                return;
+            } else {
+                evicted.push_back(Block{ptr, size, device});
             }
         }
-        if (pinned_)
-            (void)hipHostFree(ptr);
-        else
-            (void)hipFree(ptr);
+        for (const Block &b : evicted) {
+            if (pinned_)
+                (void)hipHostFree(b.ptr);
+            else
+                (void)hipFree(b.ptr);
+        }
     }
 
 private:
