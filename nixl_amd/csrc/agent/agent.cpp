@@ -698,8 +698,7 @@ nixlDescStoragePool::adopt(nixl_meta_dlist_t &list, size_t count) {
         if (best != kept_.size()) {
             taken.swap(kept_[best]);
             keptBytes_ -= taken.capacity() * sizeof(nixlMetaDesc);
-            kept_[best].swap(kept_.back());
-            kept_.pop_back();
+            kept_.erase(kept_.begin() + static_cast<std::ptrdiff_t>(best)); // keeps the rest in order of age
         }
     }
     taken.resize(count); // shrinking costs nothing; growing a kept vector touches only its new tail
@@ -711,12 +710,17 @@ nixlDescStoragePool::surrender(nixl_meta_dlist_t &list) {
     storage_t taken;
     storageOf(list).swap(taken);
     const size_t bytes = taken.capacity() * sizeof(nixlMetaDesc);
-    if (taken.capacity() < kMinPooled) return;
+    if (taken.capacity() < kMinPooled || bytes > kMaxKeptBytes) return;
+    std::vector<storage_t> dropped; // freed after the lock is gone
     std::lock_guard<std::mutex> guard(mutex_);
-    if (kept_.size() < kMaxKept && keptBytes_ + bytes <= kMaxKeptBytes) {
-        keptBytes_ += bytes;
-        kept_.push_back(std::move(taken));
+    // the storage just returned is the likeliest to be wanted again: the oldest make room for it
+    while (!kept_.empty() && (kept_.size() >= kMaxKept || keptBytes_ + bytes > kMaxKeptBytes)) {
+        keptBytes_ -= kept_.front().capacity() * sizeof(nixlMetaDesc);
+        dropped.push_back(std::move(kept_.front()));
+        kept_.erase(kept_.begin());
     }
+    keptBytes_ += bytes;
+    kept_.push_back(std::move(taken));
 }
 
 namespace {
