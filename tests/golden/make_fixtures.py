@@ -86,7 +86,10 @@ def cast_row(row):
     return q.numpy(), inv.numpy()
 
 
-def ll_world(seed=21):
+def ll_world(seed=21, repeats=(), name="ll_world.npz"):
+    """repeats: (rank, token, from k, to k) entries that make a token name one expert more than
+    once; the reference gives such a token a row per selection (kernels/nixl_ep_ll.cu:186-190),
+    next to each other here (tokens ascending, a token's selections together)."""
     R, T, H, K, E, M = 4, 5, 512, 3, 8, 6
     El, N = E // R, R * M
     rng = np.random.default_rng(seed)
@@ -97,6 +100,8 @@ def ll_world(seed=21):
     topk = np.stack([np.stack([rng.permutation(E)[:K] for _ in range(T)]) for _ in range(R)]).astype(np.int32)
     topk[0, 1, 2] = -1
     topk[2, 4, 0] = -1
+    for r_, t_, k_from, k_to in repeats:
+        topk[r_, t_, k_to] = topk[r_, t_, k_from]
     num_tokens = np.array([5, 3, 5, 4], np.int32)
     w = rng.random((R, T, K)).astype(np.float32)
 
@@ -118,17 +123,24 @@ def ll_world(seed=21):
                     if not ks:
                         continue
                     q, inv = cast_row(x[s, t])
-                    recv_fp8[d, le, n] = q
-                    recv_bf16[d, le, n] = bf16_bits(xf[s, t])
-                    scales[d, le, :, n] = inv
-                    src_info[d, le, n] = t
-                    row_of[s, t, ks[0]] = (d * El + le) * N + n
-                    n += 1
+                    for k in ks:  # a row per selection
+                        recv_fp8[d, le, n] = q
+                        recv_bf16[d, le, n] = bf16_bits(xf[s, t])
+                        scales[d, le, :, n] = inv
+                        src_info[d, le, n] = t
+                        row_of[s, t, k] = (d * El + le) * N + n
+                        n += 1
                 layout_range[d, le, s] = (n - begin) | (begin << 32)
             recv_count[d, le] = n
 
     # expert outputs: random bf16 rows where valid; combine = fma chain in top-k order
     y = torch.randn(R, El, N, H, generator=g).to(torch.bfloat16)
+    # an expert gives the rows of one token the same output (same input, same function)
+    flat = y.view(R * El * N, H)
+    for r_, t_, k_from, k_to in repeats:
+        ks = [k for k in range(K) if topk[r_, t_, k] == topk[r_, t_, k_from]]
+        for k in ks[1:]:
+            flat[row_of[r_, t_, k]] = flat[row_of[r_, t_, ks[0]]]
     yb = bf16_bits(y).reshape(R * El * N, H)
     yf = y.float().numpy().reshape(R * El * N, H)
     combined = np.zeros((R, T, H), np.uint16)
@@ -145,7 +157,7 @@ def ll_world(seed=21):
             combined[r, t] = bf16_bits(torch.from_numpy(acc))
     valid = np.arange(N)[None, None, :] < recv_count[:, :, None]
     yb = np.where(valid.reshape(-1)[:, None], yb, 0).reshape(R, El, N, H).astype(np.uint16)
-    np.savez_compressed(os.path.join(HERE, "ll_world.npz"), x=bf16_bits(xf), topk_idx=topk, topk_weights=w,
+    np.savez_compressed(os.path.join(HERE, name), x=bf16_bits(xf), topk_idx=topk, topk_weights=w,
              num_tokens=num_tokens, num_experts=E, max_tok=M, recv_fp8=recv_fp8, recv_bf16=recv_bf16, scales=scales,
              src_info=src_info, layout_range=layout_range, recv_count=recv_count, expert_out=yb, combined=combined)
     return True
@@ -248,6 +260,9 @@ if __name__ == "__main__":
     router_vectors()
     seed = 21
     while ll_world(seed) is None:  # move to another seed if an fp64 sum sits on an fp32 tie
+        seed += 1
+    seed = 31
+    while ll_world(seed, repeats=[(0, 2, 0, 1), (2, 1, 2, 0), (3, 0, 0, 1), (3, 0, 0, 2)], name="ll_world_repeats.npz") is None:
         seed += 1
     ht_world()
     kv_vectors()

@@ -1026,8 +1026,9 @@ def test_golden_encoder_and_router(cuda):
     assert np.allclose(w.cpu().numpy(), r["topk_weights"], rtol=2e-6, atol=0)
 
 
-def test_golden_low_latency_world(cuda):
-    g = _golden("ll_world.npz")
+@pytest.mark.parametrize("world", ["ll_world.npz", "ll_world_repeats.npz"])
+def test_golden_low_latency_world(cuda, world):
+    g = _golden(world)
     E, M = int(g["num_experts"]), int(g["max_tok"])
     R, T, H = g["x"].shape
     El, N = E // R, R * M

@@ -4,6 +4,7 @@ touch the oracle).  The GPU tests compare the HIP path with the same files."""
 import os
 
 import numpy as np
+import pytest
 
 from oracle import ep_oracle as eo
 from oracle import kv_oracle as ko
@@ -43,16 +44,20 @@ def check_ll_dispatch(got, g, use_fp8):
                 assert np.array_equal(got["scales"][d, le, :, :n].view(np.uint32), g["scales"][d, le, :, :n].view(np.uint32))
 
 
-def test_ll_dispatch_golden():
-    g = load("ll_world.npz")
+# ll_world_repeats.npz: some tokens name one expert two or three times and get a row per
+# selection (kernels/nixl_ep_ll.cu:186-190)
+@pytest.mark.parametrize("world", ["ll_world.npz", "ll_world_repeats.npz"])
+def test_ll_dispatch_golden(world):
+    g = load(world)
     E, M = int(g["num_experts"]), int(g["max_tok"])
     for use_fp8 in (True, False):
         got = eo.ll_dispatch(g["x"], g["topk_idx"], E, M, use_fp8=use_fp8, num_tokens=g["num_tokens"])
         check_ll_dispatch(got, g, use_fp8)
 
 
-def test_ll_combine_golden():
-    g = load("ll_world.npz")
+@pytest.mark.parametrize("world", ["ll_world.npz", "ll_world_repeats.npz"])
+def test_ll_combine_golden(world):
+    g = load(world)
     E, M = int(g["num_experts"]), int(g["max_tok"])
     out = eo.ll_combine(g["expert_out"], g["topk_idx"], g["topk_weights"], g["src_info"], g["layout_range"], E, M,
                         num_tokens=g["num_tokens"], use_fma=True)
