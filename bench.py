@@ -42,8 +42,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak, decimal GB/s
 _KV_PROFILE = "profiles/copy_uniform_kernel_kv_llama3_16KiB_32KiB.txt (rocprofv3 --pmc runs of this file, not this run)"
 MEASURED_TRAFFIC = {
     (1024, 8192, 16384): {"bytes": 2155883520, "source": _KV_PROFILE},
-    (1024, 8192, 32768): {"bytes": 4303367456, "source": _KV_PROFILE},
-    ("small", 262144): {"bytes": 938500160,
+    (1024, 8192, 32768): {"bytes": 4303367616, "source": _KV_PROFILE},
+    ("small", 262144): {"bytes": 938782368,
                         "source": "profiles/copy_piece_kernel_small_descriptor_stress_262144x512B-4KiB.txt (rocprofv3 --pmc runs of "
                                   "this file, not this run)"},
 }
@@ -414,7 +414,7 @@ def run_kv(args, blk, order, steps, warmup, fresh_requests=4, sorted_ids=False, 
                                                           f"copies: wall clock over {len(lists)} pairs back to back"}
 
     rng = np.random.default_rng(99)
-    fresh = fresh_pairs(agent, handles, rng)
+    fresh = {} if getattr(args, "headline_only", False) else fresh_pairs(agent, handles, rng)
     # The same loops with every request written out as descriptors and passed through prepXfer:
     # what an agent that knows nothing of this plugin's index entry does (the reference's
     # makeXferReq, src/core/nixl_agent.cpp:799-880).  A second agent over the same memory whose
@@ -1136,6 +1136,9 @@ def main():
     ap.add_argument("--fresh-requests", type=int, default=4,
                     help="request pairs with a new block list each, timed with their preparation")
     ap.add_argument("--quick", action="store_true", help="headline point only, no other sizes or orders")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="nothing but the headline's steady-state loop (for a kernel trace whose rows are that loop's "
+                         "launches alone); implies --quick --no-ep --no-small --no-cpu-baseline --no-live-traffic")
     ap.add_argument("--order", choices=("layer", "block"), default="layer",
                     help="descriptor list order: layer by layer, or block by block")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -1154,6 +1157,8 @@ def main():
                     help="do not run the headline leg under rocprofv3 --pmc first; roofline.traffic then comes from "
                          "the counter runs summarised under profiles/")
     args = ap.parse_args()
+    if args.headline_only:
+        args.quick = args.no_ep = args.no_small = args.no_cpu_baseline = args.no_live_traffic = True
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (virtual ranks are regions of one "
                  "GPU's HBM); --gpus must be 1")
