@@ -753,7 +753,7 @@ firstIndexOutside(const std::vector<int> &indices, size_t flat) {
 class runCursor {
 public:
     explicit runCursor(const nixl_stride_dlist_t &runs)
-        : first_(&runs[0]),
+        : first_(runs.descCount() > 0 ? &runs[0] : nullptr),
           n_runs_(static_cast<size_t>(runs.descCount())),
           blocks_(runs.flatSize()) {}
 
